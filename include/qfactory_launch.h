@@ -1,0 +1,77 @@
+/*
+ * C ABI of one compiled specialisation of the quantized-linear kernel.
+ *
+ * The JIT produces one shared object per (bits, group size, symmetric?, N, K, M, tiling).  Every
+ * such object exports the entry points below; all problem and tiling parameters are constants
+ * inside the object.  All pointers are device addresses owned by the caller, `stream` is a
+ * hipStream_t, the call only enqueues work (no synchronisation), every element of `output` is
+ * written exactly once (no pre-zeroing needed) and nothing is retained after return.
+ *
+ * Return code (written through the last argument): 0 launched, 1 the object's static
+ * configuration is invalid (reason on stderr), 2 the HIP launch itself failed.
+ *
+ * A translation unit selects which of the two `launch` signatures it implements by defining
+ * QF_LAUNCH_GROUPED or QF_LAUNCH_PLAIN before including this header; with neither defined only
+ * the function-pointer types are declared (that is what a dlopen/dlsym or ctypes caller needs).
+ */
+#ifndef QFACTORY_LAUNCH_H
+#define QFACTORY_LAUNCH_H
+
+#ifdef __cplusplus
+#define QF_RC_ARG int&
+extern "C" {
+#else
+#define QF_RC_ARG int*
+#endif
+
+/*
+ * Grouped-scale kernel: output (M,N) fp16 = activation (M,K) fp16 x dequant(weight, scale, zero)^T.
+ *   weight (N, K*b/8) int8, scale (N, K/GS) fp16, zero (N, K/GS*b/8) int8 -- the packed layout of
+ *   qfactory/convert.py:55-81; `zero` is ignored (may be any valid pointer) by symmetric objects.
+ * Replaces the reference's generated
+ *   extern "C" void launch(void* _activation, void* _weight, void* _output, void* _scale,
+ *                          void* _zero, void* _stream, int& __return_code)
+ * (emitted at qfactory/core/qfunc.py:133-152, bound through ctypes at qfactory/jit/runtime.py:37-49,
+ *  implemented by gptq_gemv_impl, qfactory/include/gptq_gemv.h:156-205).  M is the object's constant.
+ */
+typedef void (*qf_launch_grouped_fn)(void* activation, void* weight, void* output, void* scale,
+                                     void* zero, void* stream, int* return_code);
+
+/*
+ * Same computation for `m` activation rows (any m >= 1) instead of the object's constant M.
+ * No counterpart in the reference, whose grouped kernel silently computes exactly its compile-time
+ * M rows (qfactory/core/matmul.py:128 checks only activation.shape[0] == output.shape[0]).
+ */
+typedef void (*qf_launch_grouped_m_fn)(int m, void* activation, void* weight, void* output,
+                                       void* scale, void* zero, void* stream, int* return_code);
+
+/*
+ * group_size == -1 kernel: output (m,N) fp16 = activation (m,K) fp16 x q^T with raw unsigned fields.
+ * Replaces the reference's generated
+ *   extern "C" void launch(int m, void* _activation, void* _weight, void* _output, void* _stream,
+ *                          int& __return_code)
+ * (emitted at qfactory/core/qfunc.py:263-316, implemented by gemv_impl, qfactory/include/gemv.h:96-135).
+ */
+typedef void (*qf_launch_plain_fn)(int m, void* activation, void* weight, void* output, void* stream,
+                                   int* return_code);
+
+/* Static string naming the specialisation ("regime=gemv M=1 N=4096 K=4096 NBITS=4 ..."). */
+typedef const char* (*qf_describe_fn)(void);
+
+#if defined(QF_LAUNCH_GROUPED)
+void launch(void* _activation, void* _weight, void* _output, void* _scale, void* _zero, void* _stream,
+            QF_RC_ARG __return_code);
+void launch_m(int m, void* _activation, void* _weight, void* _output, void* _scale, void* _zero,
+              void* _stream, QF_RC_ARG __return_code);
+const char* qf_describe(void);
+#elif defined(QF_LAUNCH_PLAIN)
+void launch(int m, void* _activation, void* _weight, void* _output, void* _stream, QF_RC_ARG __return_code);
+const char* qf_describe(void);
+#endif
+
+#ifdef __cplusplus
+}
+#endif
+#undef QF_RC_ARG
+
+#endif /* QFACTORY_LAUNCH_H */

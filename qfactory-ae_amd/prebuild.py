@@ -1,0 +1,112 @@
+"""Ahead-of-time population of the JIT cache.
+
+The kernels are specialised per problem and compiled on first use; a GPU job should not spend its
+time in hipcc.  This module lists the problems the repository's own tests, smoke check and
+benchmark construct and compiles their specialisations (in parallel, no GPU needed) into
+``$QFACTORY_CACHE_DIR`` (default: ``jit_cache/`` beside this file).
+
+Run as ``python prebuild.py [--force]`` or through ``__graft_entry__.build()``.
+"""
+import argparse
+import os
+import sys
+from concurrent.futures import ThreadPoolExecutor, as_completed
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+if HERE not in sys.path:
+    sys.path.insert(0, HERE)
+os.environ.setdefault("QFACTORY_CACHE_DIR", os.path.join(HERE, "jit_cache"))
+
+LLAMA2_7B = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]        # (N, K): qkv, o, gate_up, down
+LLAMA3_70B = [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]
+
+
+def _case(M, N, K, NBITS=4, GS=128, sym=False):
+    return {"M": M, "N": N, "K": K, "NBITS": NBITS, "GS": GS, "sym": sym}
+
+
+def parity_cases():
+    """Problems the GPU parity tests run (tests/test_qlinear_gpu.py imports this list)."""
+    cases = []
+    for N, K in LLAMA2_7B:                                   # W4A16 g128 asymmetric GEMV sweep
+        for M in (1, 4, 16):
+            cases.append(_case(M, N, K))
+    for M in (1, 16):                                        # bit-width scaling at N = K = 8192
+        for nbits in (2, 4, 8):
+            for sym in (False, True):
+                cases.append(_case(M, 8192, 8192, nbits, 128, sym))
+    # ragged / small shapes: N not a multiple of the rows per block, odd M, other group sizes
+    cases += [_case(1, 100, 256, 4, 128), _case(2, 100, 256, 4, 64), _case(3, 130, 512, 4, 32),
+              _case(5, 77, 1024, 4, 128), _case(7, 1000, 2048, 8, 128), _case(2, 64, 512, 2, 64),
+              _case(1, 48, 4096, 2, 128, True), _case(3, 48, 1024, 8, 256, True),
+              _case(1, 256, 11008, 4, 128)]
+    for nbits in (2, 4, 8):                                  # group_size == -1: raw integer weights
+        cases += [_case(1, 4096, 4096, nbits, -1), _case(3, 100, 256, nbits, -1)]
+    return cases
+
+
+def bench_cases():
+    cases = [_case(1, N, K) for N, K in LLAMA2_7B]
+    return cases
+
+
+def smoke_cases():
+    return [_case(1, 512, 1024, 4, 128), _case(1, 512, 1024, 4, -1)]
+
+
+def misc_test_cases():
+    """Other modules the GPU tests construct (row-count dispatch, argument checks)."""
+    return [_case(M, 96, 512, 4, 128) for M in (1, 2, 3, 6)] + [_case(1, 64, 256, 4, 128)]
+
+
+def all_cases():
+    seen, out = set(), []
+    for c in parity_cases() + bench_cases() + smoke_cases() + misc_test_cases():
+        key = tuple(sorted(c.items()))
+        if key not in seen:
+            seen.add(key)
+            out.append(c)
+    return out
+
+
+def qfuncs_of(case):
+    """The default specialisation(s) ``QLinear`` compiles for a case (no search flags)."""
+    import torch
+    from qfactory.core import QMatmul, Matmul
+    from qfactory.qlinear import _m_bucket
+    if case["GS"] == -1:
+        op = Matmul(case["N"], case["K"], case["NBITS"], torch.float16, torch.int8)
+    else:
+        op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
+                     torch.float16, torch.int8, case["GS"])
+    op.init_qfuncs()
+    return op.qfuncs
+
+
+def prebuild(cases=None, force=False, workers=None, verbose=True):
+    from qfactory.jit import jit
+    qfuncs, seen = [], set()
+    for case in (cases if cases is not None else all_cases()):
+        for q in qfuncs_of(case):
+            path, _ = jit.runtime_path_of(q)
+            if path not in seen:
+                seen.add(path)
+                qfuncs.append(q)
+    workers = workers or min(16, os.cpu_count() or 4)
+    done = 0
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        futures = [pool.submit(jit.compile, q, force) for q in qfuncs]
+        for f in as_completed(futures):
+            f.result()
+            done += 1
+            if verbose and (done % 10 == 0 or done == len(futures)):
+                print(f"[prebuild] {done}/{len(futures)} specialisations", flush=True)
+    return len(qfuncs)
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--force", action="store_true", help="recompile even if cached")
+    args = ap.parse_args()
+    n = prebuild(force=args.force)
+    print(f"[prebuild] {n} specialisations in {os.environ['QFACTORY_CACHE_DIR']}")

@@ -1,0 +1,254 @@
+"""Quantized matmul operators: build the QFunc(s), compile, optionally time the candidates, and
+return the closure that ``QLinear.forward`` calls.
+
+Interface of the reference's ``qfactory/core/matmul.py`` (QMatmul :14-153, Matmul :155-270): same
+constructor arguments, same ``compile_profile(enable_transform, enable_schedule, enable_lower)``,
+same ``$QFACTORY_CONFIG`` lookup keyed ``"{nbits}-{m}-{n}-{k}-{group_size}"``, and closures with the
+same argument lists and checks.  Differences that matter to callers:
+
+* the closure launches for the *actual* number of activation rows (the reference silently computes
+  only the rows it was compiled for, matmul.py:128);
+* supported widths are 2/3/4/8 bits; M may be anything >= 1 (large M runs on the matrix cores).
+"""
+import json
+import logging
+import os
+from concurrent.futures import ThreadPoolExecutor, as_completed
+from itertools import chain
+
+import torch
+
+from .qtile import QTile, SymQTile, AsymQTile
+from .qfunc import QMatmulQFunc, MatmulQFunc
+from ..convert import weight_row_bytes, zero_row_bytes
+from ..jit import jit
+
+logger = logging.getLogger(__name__)
+
+
+def require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("qfactory kernels need a HIP device (torch.cuda.is_available() is False); "
+                           "there is no CPU fallback")
+
+
+def _load_predefined(shape_key):
+    path = os.getenv("QFACTORY_CONFIG")
+    if path is None or not os.path.exists(path):
+        return None
+    with open(path) as f:
+        config = json.load(f)
+    return config.get(shape_key)
+
+
+def _compile_all(qfuncs):
+    runtimes = [None] * len(qfuncs)
+    workers = min(len(qfuncs), int(os.environ.get("QFACTORY_JIT_WORKERS", os.cpu_count() or 4)))
+    with ThreadPoolExecutor(max_workers=max(1, workers)) as executor:
+        futures = {executor.submit(jit.compile, q): i for i, q in enumerate(qfuncs)}
+        for future in as_completed(futures):
+            runtimes[futures[future]] = future.result()
+    return runtimes
+
+
+def _pick_best(runtimes, qfuncs, dummy_inputs, what):
+    """Time every candidate that accepts its configuration; keep the fastest."""
+    if len(runtimes) == 1:
+        return runtimes[0], qfuncs[0]
+    from ..profile import benchmark
+    best = (None, None, None)
+    for runtime, qfunc in zip(runtimes, qfuncs):
+        if runtime.run(*dummy_inputs) != 0:
+            continue
+        t = benchmark(lambda: runtime.run(*dummy_inputs))
+        logger.debug(f"[Profile] Kernel: {t * 1e6:.2f} us  {runtime.description}")
+        if best[0] is None or t < best[2]:
+            best = (runtime, qfunc, t)
+    assert best[0] is not None, "No valid runtime found"
+    logger.info(f"[Profile] Best latency for {what}: {best[2] * 1e6:.2f} us  ({best[0].description})")
+    return best[0], best[1]
+
+
+class QMatmul:
+    def __init__(self, m: int, n: int, k: int, nbits: int, sym: bool, dtype_a, dtype_b,
+                 group_size: int = -1, layout: str = "nt", base_impl: bool = False):
+        self.m, self.n, self.k = m, n, k
+        self.nbits, self.sym = nbits, sym
+        self.dtype_a, self.dtype_b = dtype_a, dtype_b
+        self.group_size = k if group_size == -1 else group_size
+        self.layout = layout
+        self.base_impl = base_impl
+        assert self.k % self.group_size == 0, f"Group size {self.group_size} must divide k {self.k}"
+        assert self.layout == "nt", f"Layout {layout} is not supported"
+        assert dtype_a == torch.float16, f"Data type {dtype_a} is not supported"
+        assert dtype_b == torch.int8, f"Data type {dtype_b} is not supported"
+        assert nbits in (2, 3, 4, 8), f"{nbits}-bit weights are not supported"
+
+    # packed operand shapes
+    @property
+    def weight_shape(self):
+        return (self.n, weight_row_bytes(self.k, self.nbits))
+
+    @property
+    def scale_shape(self):
+        return (self.n, self.k // self.group_size)
+
+    @property
+    def zero_shape(self):
+        return (self.n, zero_row_bytes(self.k // self.group_size, self.nbits))
+
+    def init_qfuncs(self):
+        tile_b = SymQTile if self.sym else AsymQTile
+        self.qfuncs = [QMatmulQFunc(
+            QTile((self.m, self.k), self.dtype_a, 16),
+            tile_b((self.n, self.k), self.dtype_b, self.nbits, (1, self.group_size)),
+            "nt", self.base_impl)]
+
+    def get_dummy_inputs(self):
+        require_gpu()
+        activation = torch.zeros((self.m, self.k), dtype=self.dtype_a, device="cuda")
+        weight = torch.zeros(self.weight_shape, dtype=self.dtype_b, device="cuda")
+        output = torch.empty((self.m, self.n), dtype=self.dtype_a, device="cuda")
+        scale = torch.zeros(self.scale_shape, dtype=self.dtype_a, device="cuda")
+        zero = torch.zeros(self.zero_shape, dtype=self.dtype_b, device="cuda")
+        return activation, weight, output, scale, zero, torch.cuda.current_stream()
+
+    def compile_profile(self, enable_transform: bool = False, enable_schedule: bool = False,
+                        enable_lower: bool = False):
+        self.init_qfuncs()
+        shape = f"{self.nbits}-{self.m}-{self.n}-{self.k}-{self.group_size}"
+        predefined = _load_predefined(shape)
+        if predefined is not None:
+            logger.info(f"[Profile] Using predefined config for {shape}")
+            qfunc = self.qfuncs[0]
+            for key, value in predefined.items():
+                setattr(qfunc, key, value)
+            self.qfuncs = [qfunc]
+        else:
+            if enable_transform:
+                self.qfuncs = list(chain.from_iterable(q.transform() for q in self.qfuncs))
+            if enable_schedule:
+                self.qfuncs = list(chain.from_iterable(q.schedule() for q in self.qfuncs))
+            if enable_lower:
+                self.qfuncs = list(chain.from_iterable(q.lower() for q in self.qfuncs))
+
+        self.runtimes = _compile_all(self.qfuncs)
+        dummy = self.get_dummy_inputs() if len(self.runtimes) > 1 else None
+        self.best_runtime, self.best_qfunc = _pick_best(self.runtimes, self.qfuncs, dummy, shape)
+        return self._wrap(self.best_runtime)
+
+    def _wrap(self, runtime):
+        n, k = self.n, self.k
+        w_shape, s_shape, z_shape = self.weight_shape, self.scale_shape, self.zero_shape
+        zero_empty = None
+        if self.sym:
+            require_gpu()
+            zero_empty = torch.empty(z_shape, dtype=torch.int8, device="cuda")
+
+        def inner(activation, weight, output, scale, zero):
+            # tensor shape check
+            assert activation.shape[1] == k
+            assert weight.shape == w_shape
+            assert output.shape[1] == n
+            assert activation.shape[0] == output.shape[0]
+            assert scale.shape == s_shape
+            assert zero.shape == z_shape
+            # tensor dtype check
+            assert activation.dtype == torch.float16
+            assert weight.dtype == torch.int8
+            assert output.dtype == torch.float16
+            assert scale.dtype == torch.float16
+            assert zero.dtype == torch.int8
+            # contiguous check
+            assert activation.is_contiguous()
+            assert weight.is_contiguous()
+            assert output.is_contiguous()
+            assert scale.is_contiguous()
+            assert zero.is_contiguous()
+            assert activation.is_cuda and weight.is_cuda and output.is_cuda
+            return runtime.run_raw(
+                activation.shape[0],
+                (activation.data_ptr(), weight.data_ptr(), output.data_ptr(), scale.data_ptr(), zero.data_ptr()),
+                torch.cuda.current_stream().cuda_stream)
+
+        def inner_sym(activation, weight, output, scale):
+            return inner(activation, weight, output, scale, zero_empty)
+
+        func = inner_sym if self.sym else inner
+        func.runtime = runtime
+        return func
+
+
+class Matmul:
+    """group_size == -1: no scales, no zero-points, raw unsigned fields (reference matmul.py:155-270)."""
+
+    def __init__(self, n: int, k: int, nbits: int, dtype_a, dtype_b, layout: str = "nt"):
+        self.n, self.k = n, k
+        self.nbits = nbits
+        self.dtype_a, self.dtype_b = dtype_a, dtype_b
+        self.layout = layout
+        assert self.layout == "nt", f"Layout {layout} is not supported"
+        assert dtype_a == torch.float16, f"Data type {dtype_a} is not supported"
+        assert dtype_b == torch.int8, f"Data type {dtype_b} is not supported"
+        assert nbits in (2, 3, 4, 8), f"{nbits}-bit weights are not supported"
+
+    @property
+    def weight_shape(self):
+        return (self.n, weight_row_bytes(self.k, self.nbits))
+
+    def init_qfuncs(self):
+        self.qfuncs = [MatmulQFunc(
+            QTile((0, self.k), self.dtype_a, 16),
+            QTile((self.n, self.k), self.dtype_b, self.nbits),
+            "nt")]
+
+    def get_dummy_inputs(self):
+        require_gpu()
+        m = 1
+        activation = torch.zeros((m, self.k), dtype=self.dtype_a, device="cuda")
+        weight = torch.zeros(self.weight_shape, dtype=self.dtype_b, device="cuda")
+        output = torch.empty((m, self.n), dtype=self.dtype_a, device="cuda")
+        return m, activation, weight, output, torch.cuda.current_stream()
+
+    def compile_profile(self, enable_transform: bool = False, enable_schedule: bool = False,
+                        enable_lower: bool = False):
+        self.init_qfuncs()
+        shape = f"{self.nbits}-{1}-{self.n}-{self.k}-{-1}"
+        predefined = _load_predefined(shape)
+        if predefined is not None:
+            logger.info(f"[Profile] Using predefined config for {shape}")
+            qfunc = self.qfuncs[0]
+            for key, value in predefined.items():
+                setattr(qfunc, key, value)
+            self.qfuncs = [qfunc]
+        else:
+            if enable_schedule:
+                self.qfuncs = list(chain.from_iterable(q.schedule() for q in self.qfuncs))
+            if enable_lower:
+                self.qfuncs = list(chain.from_iterable(q.lower() for q in self.qfuncs))
+
+        self.runtimes = _compile_all(self.qfuncs)
+        dummy = self.get_dummy_inputs() if len(self.runtimes) > 1 else None
+        self.best_runtime, self.best_qfunc = _pick_best(self.runtimes, self.qfuncs, dummy, shape)
+        return self._wrap(self.best_runtime)
+
+    def _wrap(self, runtime):
+        n, k, w_shape = self.n, self.k, self.weight_shape
+
+        def inner(activation, weight, output):
+            m = activation.shape[0]
+            assert activation.shape == (m, k)
+            assert weight.shape == w_shape
+            assert output.shape == (m, n)
+            assert activation.dtype == torch.float16
+            assert weight.dtype == torch.int8
+            assert output.dtype == torch.float16
+            assert activation.is_contiguous()
+            assert weight.is_contiguous()
+            assert output.is_contiguous()
+            assert activation.is_cuda and weight.is_cuda and output.is_cuda
+            return runtime.run_raw(m, (activation.data_ptr(), weight.data_ptr(), output.data_ptr()),
+                                   torch.cuda.current_stream().cuda_stream)
+
+        inner.runtime = runtime
+        return inner

@@ -1,0 +1,212 @@
+"""QFuncs: a quantized matmul described over QTiles, its search space, and the HIP translation unit
+it emits.
+
+Mirrors the reference's ``qfactory/core/qfunc.py`` at the interface level -- ``QMatmulQFunc`` /
+``MatmulQFunc`` with ``arg_name_type() / transform() / schedule() / lower() / emit()`` and the
+attributes a tuned-config JSON may set verbatim (``parallel_strategy``, ``tiling_configs``,
+``decode_strategy``, ``l2cache_a``, ``l2cache_b``, ``smem_quant``; qfunc.py:27-41, matmul.py:76-77)
+-- but what is emitted is a specialisation of the gfx950 templates in ``qfactory/include`` for one
+(bits, group size, N, K, M-tile), compiled by hipcc.
+
+The emitted object exports the reference's entry point (qfunc.py:139-152 / 233-238)
+
+    extern "C" void launch(<pointers...>, void* stream, int& return_code)
+
+plus ``launch_m`` (same, with the number of activation rows as a leading ``int``) and
+``qf_describe`` (a string naming the specialisation).
+"""
+import copy
+from typing import List
+
+import torch
+
+from . import tiling
+
+Python2CppTypes = {  # python-side type -> (type in the C signature, type used inside)
+    int: ("int", "int"),
+    torch.float16: ("void*", "uint16_t*"),
+    torch.int8: ("void*", "uint8_t*"),
+    torch.cuda.streams.Stream: ("void*", "hipStream_t"),
+}
+
+
+class QFunc:
+    regime = "gemv"
+
+    def arg_name_type(self):
+        raise NotImplementedError
+
+    def emit(self) -> str:
+        raise NotImplementedError
+
+    def clone(self, **attrs):
+        other = copy.deepcopy(self)
+        for key, value in attrs.items():
+            setattr(other, key, value)
+        return other
+
+    # -- shared emit helpers --------------------------------------------------------------
+    def _signature(self, name, leading_m):
+        lines = [f'extern "C" void {name} (']
+        if leading_m:
+            lines.append("\tint m,")
+        for arg, t in self.arg_name_type():
+            if t is int:
+                continue
+            lines.append(f"\t{Python2CppTypes[t][0]} _{arg},")
+        lines.append("\tint& __return_code")
+        lines.append(") {")
+        return "\n".join(lines) + "\n"
+
+
+def _problem_of(qtile_a, qtile_b):
+    m, k = qtile_a.shape
+    n, kb = qtile_b.shape
+    assert k == kb, f"Shape mismatch: {k} != {kb}"
+    return m, n, k
+
+
+class QMatmulQFunc(QFunc):
+    """activation (M,K) fp16  x  quantized weight (N,K), per-group scale (and zero)  ->  (M,N) fp16."""
+
+    def __init__(self, qtile_a, qtile_b, layout, base_impl=False):
+        self.qtile_a, self.qtile_b, self.layout = qtile_a, qtile_b, layout
+        assert qtile_a.quant_method == "none", "Quantization method not supported for A"
+        assert qtile_b.quant_method in ("sym", "asym"), "Quantization method of B must be 'sym' or 'asym'"
+        assert layout == "nt", f"Layout {layout} is not supported"
+        m, n, k = _problem_of(qtile_a, qtile_b)
+        gs = qtile_b.quant_granularity[1]
+
+        # Template-based code generation: which kernel family and how it is tiled
+        self.regime = tiling.regime_for(m)
+        self.parallel_strategy = "row"          # teams sweep rows, K split over lanes and waves
+        self.tiling_configs = self.default_tiling(self.regime)
+        # Computation transformation: "deferred" applies scale and zero once per chunk / group in
+        # fp32 after the integer dot product; "eager" dequantises every element to fp16 first.
+        self.decode_strategy = "deferred" if self.regime == "gemv" else "eager"
+        # Load-path scheduling
+        self.l2cache_a = True                   # activations: normal (cached) loads
+        self.l2cache_b = False                  # weights: streaming (non-temporal) loads
+        self.smem_quant = False                 # stage scales/zeros through LDS
+        self.base_impl = base_impl
+        self._gs = gs
+
+    # -- description ------------------------------------------------------------------------
+    @property
+    def problem(self):
+        m, n, k = _problem_of(self.qtile_a, self.qtile_b)
+        return {"M": m, "N": n, "K": k, "NBITS": self.qtile_b.nbits, "GS": self._gs,
+                "SYM": self.qtile_b.quant_method == "sym"}
+
+    def default_tiling(self, regime):
+        p = {"M": self.qtile_a.shape[0], "N": self.qtile_b.shape[0], "K": self.qtile_b.shape[1]}
+        nbits, gs = self.qtile_b.nbits, self.qtile_b.quant_granularity[1]
+        if regime == "gemv":
+            return tiling.gemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
+        return tiling.mfma_tiling(p["M"], p["N"], p["K"], nbits, gs)
+
+    def arg_name_type(self):
+        return [
+            ("activation", torch.float16), ("weight", torch.int8), ("output", torch.float16),
+            ("scale", torch.float16), ("zero", torch.int8),
+            ("stream", torch.cuda.streams.Stream),
+        ]
+
+    # -- search space -------------------------------------------------------------------------
+    def transform(self) -> List[QFunc]:
+        if self.regime == "gemv":
+            return [self.clone(decode_strategy="deferred")]
+        return [self.clone(decode_strategy=d) for d in ("eager", "deferred")]
+
+    def schedule(self) -> List[QFunc]:
+        return [self.clone(l2cache_a=True, l2cache_b=b) for b in (False, True)]
+
+    def lower(self) -> List[QFunc]:
+        p = self.problem
+        if self.regime == "gemv":
+            cands = tiling.gemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
+        else:
+            cands = tiling.mfma_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
+        return [self.clone(tiling_configs=c) for c in cands]
+
+    # -- code generation ----------------------------------------------------------------------
+    def emit(self) -> str:
+        p = self.problem
+        t = self.tiling_configs
+        b = lambda x: "true" if x else "false"
+        code = "// QFactory-HIP generated translation unit\n\n"
+        if self.regime == "gemv":
+            code += '#include "qf_gemv.hip.h"\n'
+            cfg = (f"qf::GemvCfg<{p['NBITS']}, {p['GS']}, {b(p['SYM'])}, true, {p['N']}, {p['K']}, "
+                   f"{t['MT']}, {t['WK']}, {t['WN']}, {t['U']}, {t['STEPS']}, {t['VB']}, {b(not self.l2cache_b)}>")
+            call = "qf::gemv_launch<Cfg>"
+        elif self.regime == "mfma":
+            code += '#include "qf_mfma.hip.h"\n'
+            cfg = tiling.mfma_cfg_string(p, t, self.decode_strategy, not self.l2cache_b)
+            call = "qf::mfma_launch<Cfg>"
+        else:
+            raise ValueError(f"unknown regime {self.regime}")
+        code += '#if __has_include("qfactory_launch.h")\n#define QF_LAUNCH_GROUPED 1\n#include "qfactory_launch.h"\n#endif\n\n'
+        code += f"using Cfg = {cfg};\nconstexpr int M = {p['M']};\n\n"
+        args = "_activation, _weight, _output, _scale, _zero"
+        code += self._signature("launch", leading_m=False)
+        code += f"\t__return_code = {call}({args}, M, (hipStream_t)_stream);\n}}\n\n"
+        code += self._signature("launch_m", leading_m=True)
+        code += f"\t__return_code = {call}({args}, m, (hipStream_t)_stream);\n}}\n\n"
+        desc = (f"regime={self.regime} M={p['M']} N={p['N']} K={p['K']} NBITS={p['NBITS']} GS={p['GS']} "
+                f"SYM={int(p['SYM'])} decode={self.decode_strategy} nt_b={int(not self.l2cache_b)} "
+                + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
+        code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
+        return code
+
+
+class MatmulQFunc(QFunc):
+    """group_size == -1: activation (M,K) fp16 x raw unsigned low-bit weight (N,K) -> (M,N) fp16."""
+
+    def __init__(self, qtile_a, qtile_b, layout):
+        self.qtile_a, self.qtile_b, self.layout = qtile_a, qtile_b, layout
+        assert qtile_a.quant_method == "none", "Quantization method not supported for A"
+        assert qtile_b.quant_method == "none", "Quantization method not supported for B"
+        assert layout == "nt", f"Layout {layout} is not supported"
+        _problem_of(qtile_a, qtile_b)
+        self.regime = "gemv"
+        self.parallel_strategy = "row"
+        self.tiling_configs = tiling.gemv_tiling(1, qtile_b.shape[0], qtile_b.shape[1], qtile_b.nbits, None)
+        self.l2cache_a = True
+        self.l2cache_b = False
+
+    @property
+    def problem(self):
+        return {"M": 1, "N": self.qtile_b.shape[0], "K": self.qtile_b.shape[1], "NBITS": self.qtile_b.nbits}
+
+    def arg_name_type(self):
+        return [
+            ("m", int),
+            ("activation", torch.float16), ("weight", torch.int8), ("output", torch.float16),
+            ("stream", torch.cuda.streams.Stream),
+        ]
+
+    def schedule(self) -> List[QFunc]:
+        return [self.clone(l2cache_a=a, l2cache_b=b) for a in (True, False) for b in (True, False)]
+
+    def lower(self) -> List[QFunc]:
+        p = self.problem
+        return [self.clone(tiling_configs=c)
+                for c in tiling.gemv_candidates(1, p["N"], p["K"], p["NBITS"], None)]
+
+    def emit(self) -> str:
+        p = self.problem
+        t = self.tiling_configs
+        b = lambda x: "true" if x else "false"
+        code = "// QFactory-HIP generated translation unit\n\n"
+        code += '#include "qf_gemv.hip.h"\n'
+        code += '#if __has_include("qfactory_launch.h")\n#define QF_LAUNCH_PLAIN 1\n#include "qfactory_launch.h"\n#endif\n\n'
+        code += (f"using Cfg = qf::GemvCfg<{p['NBITS']}, 0, false, false, {p['N']}, {p['K']}, "
+                 f"{t['MT']}, {t['WK']}, {t['WN']}, {t['U']}, {t['STEPS']}, {t['VB']}, {b(not self.l2cache_b)}>;\n\n")
+        code += self._signature("launch", leading_m=True)
+        code += ("\t__return_code = qf::gemv_launch<Cfg>(_activation, _weight, _output, nullptr, nullptr, m, "
+                 "(hipStream_t)_stream);\n}\n\n")
+        desc = (f"regime=gemv-plain N={p['N']} K={p['K']} NBITS={p['NBITS']} nt_b={int(not self.l2cache_b)} "
+                + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
+        code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
+        return code

@@ -1,0 +1,190 @@
+// Shared device helpers for the gfx950 quantized-linear kernels: vector loads, the
+// magic-number int->fp16 decode for 2/4/8-bit fields, and wave64 cross-lane exchange.
+//
+// Weight layout consumed here is the reference's packed layout (qfactory/convert.py:49-68):
+// row n holds its K fields K-contiguously; inside every 32-bit word the even-indexed
+// elements sit in bits 0..15 and the odd-indexed ones in bits 16..31, so that
+// (word >> b*i) & (MASK | MASK << 16) is the pair (element 2i, element 2i+1)
+// (qfactory/include/utils.h:11-25 decodes in the same order).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qf {
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kMagic = 0x64006400u;  // the fp16 pair (1024, 1024): 1024 + q is exact for q < 1024
+
+__device__ __forceinline__ f16x2 as_f16x2(uint32_t v) { return __builtin_bit_cast(f16x2, v); }
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+
+// ---- global loads of NW 32-bit words (NW in {1,2,4}); NT = streaming (non-temporal) ----
+template <int NW, bool NT>
+__device__ __forceinline__ void load_words(const void* p, uint32_t (&dst)[NW]) {
+    static_assert(NW == 1 || NW == 2 || NW == 4, "vector width must be 4, 8 or 16 bytes");
+    if constexpr (NW == 4) {
+        u32x4 v = NT ? __builtin_nontemporal_load((const u32x4*)p) : *(const u32x4*)p;
+        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+    } else if constexpr (NW == 2) {
+        u32x2 v = NT ? __builtin_nontemporal_load((const u32x2*)p) : *(const u32x2*)p;
+        dst[0] = v.x; dst[1] = v.y;
+    } else {
+        dst[0] = NT ? __builtin_nontemporal_load((const uint32_t*)p) : *(const uint32_t*)p;
+    }
+}
+
+// ---- field decode: one packed word -> PAIRS fp16 pairs holding 1024 + SCALE(class) * q ----
+//
+// Instead of shifting every field down to bit 0, fields are masked in place: a field at bit
+// offset o inside its half-word decodes to 1024 + 2^o * q, still exact in fp16.  Pairs with the
+// same o form a "class"; a dot product keeps one fp32 accumulator per class and folds the 2^-o
+// factors and the 1024 offsets in once per chunk (see gemv kernel).  Only the upper byte of each
+// half-word needs one shift per word.
+template <int NBITS> struct Decode;
+
+template <> struct Decode<4> {
+    static constexpr int PAIRS = 4;   // pairs per 32-bit word
+    static constexpr int NCLS = 2;    // field offsets 0 and 4
+    __host__ __device__ static constexpr int cls(int pair) { return pair & 1; }
+    __host__ __device__ static constexpr float inv_scale(int c) { return c == 0 ? 1.0f : 0.0625f; }
+    __device__ __forceinline__ static void word(uint32_t w, uint32_t (&x)[PAIRS]) {
+        const uint32_t w8 = w >> 8;
+        x[0] = (w & 0x000F000Fu) | kMagic;
+        x[1] = (w & 0x00F000F0u) | kMagic;
+        x[2] = (w8 & 0x000F000Fu) | kMagic;
+        x[3] = (w8 & 0x00F000F0u) | kMagic;
+    }
+};
+
+template <> struct Decode<2> {
+    static constexpr int PAIRS = 8;
+    static constexpr int NCLS = 4;    // field offsets 0, 2, 4, 6
+    __host__ __device__ static constexpr int cls(int pair) { return pair & 3; }
+    __host__ __device__ static constexpr float inv_scale(int c) {
+        return c == 0 ? 1.0f : c == 1 ? 0.25f : c == 2 ? 0.0625f : 0.015625f;
+    }
+    __device__ __forceinline__ static void word(uint32_t w, uint32_t (&x)[PAIRS]) {
+        const uint32_t w8 = w >> 8;
+        x[0] = (w & 0x00030003u) | kMagic;
+        x[1] = (w & 0x000C000Cu) | kMagic;
+        x[2] = (w & 0x00300030u) | kMagic;
+        x[3] = (w & 0x00C000C0u) | kMagic;
+        x[4] = (w8 & 0x00030003u) | kMagic;
+        x[5] = (w8 & 0x000C000Cu) | kMagic;
+        x[6] = (w8 & 0x00300030u) | kMagic;
+        x[7] = (w8 & 0x00C000C0u) | kMagic;
+    }
+};
+
+template <> struct Decode<8> {
+    static constexpr int PAIRS = 2;
+    static constexpr int NCLS = 1;
+    __host__ __device__ static constexpr int cls(int) { return 0; }
+    __host__ __device__ static constexpr float inv_scale(int) { return 1.0f; }
+    __device__ __forceinline__ static void word(uint32_t w, uint32_t (&x)[PAIRS]) {
+        // 8-bit fields are stored in natural byte order (PERMUTE_ORDER[8] is the identity):
+        // byte-permute (b0, 0x64, b1, 0x64) and (b2, 0x64, b3, 0x64) in one instruction each.
+        x[0] = __builtin_amdgcn_perm(0x64646464u, w, 0x04010400u);
+        x[1] = __builtin_amdgcn_perm(0x64646464u, w, 0x04030402u);
+    }
+};
+
+// ---- wave64 lane exchange: value held by lane (l ^ D) ----
+template <int D>
+__device__ __forceinline__ float lane_xor(float v) {
+    const int iv = __builtin_bit_cast(int, v);
+    int r;
+    if constexpr (D == 1) {
+        r = __builtin_amdgcn_update_dpp(0, iv, 0xB1, 0xF, 0xF, true);      // quad_perm [1,0,3,2]
+    } else if constexpr (D == 2) {
+        r = __builtin_amdgcn_update_dpp(0, iv, 0x4E, 0xF, 0xF, true);      // quad_perm [2,3,0,1]
+    } else if constexpr (D == 4) {
+        r = __builtin_amdgcn_ds_swizzle(iv, 0x101F);                       // bit mode, xor 4
+    } else if constexpr (D == 8) {
+        r = __builtin_amdgcn_update_dpp(0, iv, 0x128, 0xF, 0xF, true);     // row_ror:8 == xor 8 in a row of 16
+    } else if constexpr (D == 16) {
+        r = __builtin_amdgcn_ds_swizzle(iv, 0x401F);                       // bit mode, xor 16
+    } else {
+        static_assert(D == 32, "lane distance must be a power of two below 64");
+        r = __builtin_amdgcn_ds_bpermute(((int)__lane_id() ^ 32) << 2, iv);
+    }
+    return __builtin_bit_cast(float, r);
+}
+
+// One "halving" butterfly step at lane distance D over the first VC entries of v: lanes with bit D
+// clear keep the first half, lanes with bit D set keep the second half, each adding what its
+// partner sent.  Afterwards the first VC/2 entries are live.
+template <int D, int VC, int V>
+__device__ __forceinline__ void halve_step(float (&v)[V], int lane) {
+    constexpr int H = VC / 2;
+    const bool up = (lane & D) != 0;
+#pragma unroll
+    for (int i = 0; i < H; i++) {
+        const float keep = up ? v[i + H] : v[i];
+        const float send = up ? v[i] : v[i + H];
+        v[i] = keep + lane_xor<D>(send);
+    }
+}
+
+// Order in which lane-distance bits are consumed by wave_reduce_many: DPP-only distances first
+// (they carry the most values), the LDS-crossbar ones last.
+__host__ __device__ constexpr int kLaneOrder(int t) {
+    return t == 0 ? 1 : t == 1 ? 2 : t == 2 ? 8 : t == 3 ? 4 : t == 4 ? 16 : 32;
+}
+
+template <int VC, int T, int V>
+__device__ __forceinline__ void reduce_from(float (&v)[V], int lane) {
+    if constexpr (T < 6) {
+        constexpr int D = kLaneOrder(T);
+        if constexpr (VC > 1) {
+            halve_step<D, VC, V>(v, lane);
+            reduce_from<VC / 2, T + 1, V>(v, lane);
+        } else {
+            v[0] += lane_xor<D>(v[0]);
+            reduce_from<1, T + 1, V>(v, lane);
+        }
+    }
+}
+
+// Sum V (power of two, <= 64) per-lane values across the 64 lanes of a wave.  On return v[0] of
+// lane l holds the wave-wide total of the input value with index reduce_index<V>(l); lanes for
+// which reduce_owner<V>(l) is true hold the V distinct totals.
+template <int V>
+__device__ __forceinline__ void wave_reduce_many(float (&v)[V], int lane) {
+    static_assert(V >= 1 && V <= 64 && (V & (V - 1)) == 0, "V must be a power of two <= 64");
+    reduce_from<V, 0, V>(v, lane);
+}
+
+template <int V>
+__device__ __forceinline__ int reduce_index(int lane) {
+    int idx = 0, span = V;
+#pragma unroll
+    for (int t = 0; t < 6; t++) {
+        if (span > 1) {
+            span >>= 1;
+            if (lane & kLaneOrder(t)) idx += span;
+        }
+    }
+    return idx;
+}
+
+template <int V>
+__device__ __forceinline__ bool reduce_owner(int lane) {
+    int used = 0, span = V;
+#pragma unroll
+    for (int t = 0; t < 6; t++) {
+        if (span > 1) { span >>= 1; used |= kLaneOrder(t); }
+    }
+    return (lane & ~used & 63) == 0;
+}
+
+}  // namespace qf

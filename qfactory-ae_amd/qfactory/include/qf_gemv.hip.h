@@ -1,0 +1,258 @@
+// Dequant-fused low-bit GEMV for gfx950, small-M regime (HBM-bound).
+//
+//   C[m][n] = fp16( sum_k A[m][k] * (q[n][k] - Z[n][k/GS]) * s[n][k/GS] )        (grouped)
+//   C[m][n] = fp16( sum_k A[m][k] * q[n][k] )                                    (QPARAM == false)
+//
+// Replaces kernel_gptq / gptq_gemv_impl (qfactory/include/gptq_gemv.h:14-205) and kernel_gemv /
+// gemv_impl (qfactory/include/gemv.h:12-135) of the reference; consumes the same packed tensors.
+//
+// Mapping (one "team" = WK waves sweeps rows of the packed weight matrix):
+//   * a lane owns IT fixed 'chunks' of the K axis (VB bytes of packed weight each, chunk index
+//     tt + 64*WK*it) so that every wave-wide weight load is 64*VB contiguous bytes of one row;
+//   * the activations of those chunks are loaded once and stay in registers for all the rows the
+//     team visits (A-stationary), the weights stream through with U rows in flight per stage and
+//     the next stage prefetched while the current one is consumed;
+//   * fields are decoded to fp16 pairs holding 1024 + 2^o*q and fed to v_dot2_f32_f16 with fp32
+//     accumulators; the 1024 offsets, the 2^-o factors, the zero-point and the scale are applied
+//     once per chunk in fp32:  s * (sum a*q - Z * sum a);
+//   * the U*MT partial sums of a stage are summed across the wave with a halving butterfly, across
+//     the WK waves through LDS, and every output element is written exactly once.
+#pragma once
+
+#include <cstdio>
+#include "qf_common.hip.h"
+
+namespace qf {
+
+template <int NBITS_, int GS_, bool SYM_, bool QPARAM_, int N_, int K_, int MT_, int WK_, int WN_,
+          int U_, int STEPS_, int VB_, bool NT_B_>
+struct GemvCfg {
+    static constexpr int NBITS = NBITS_;      // weight field width: 2, 4 or 8
+    static constexpr int GS = GS_;            // group size along K (ignored when !QPARAM)
+    static constexpr bool SYM = SYM_;         // implicit zero-point 2^(b-1), no zero tensor read
+    static constexpr bool QPARAM = QPARAM_;   // false: no scale / zero at all (group_size == -1 path)
+    static constexpr int N = N_, K = K_;
+    static constexpr int MT = MT_;            // activation rows handled per block (grid.y tiles M)
+    static constexpr int WK = WK_;            // waves along K per team
+    static constexpr int WN = WN_;            // teams per block
+    static constexpr int U = U_;              // weight rows in flight per team and stage
+    static constexpr int STEPS = STEPS_;      // stages per block
+    static constexpr int VB = VB_;            // bytes of packed weight per lane and load: 16, 8 or 4
+    static constexpr bool NT_B = NT_B_;       // stream the weights with non-temporal loads
+
+    static constexpr int NW = VB / 4;                   // 32-bit words per chunk
+    static constexpr int EPC = VB * 8 / NBITS;          // elements per chunk
+    static constexpr int NCH = K / EPC;                 // chunks per row
+    static constexpr int T = 64 * WK;                   // threads per team
+    static constexpr int IT = (NCH + T - 1) / T;        // chunks per lane and row
+    static constexpr int THREADS = 64 * WK * WN;
+    static constexpr int RPT = U * STEPS;               // rows per team
+    static constexpr int RPB = RPT * WN;                // rows per block
+    static constexpr int V = U * MT;                    // partial sums per stage
+    static constexpr int RB = K * NBITS / 8;            // packed weight row bytes
+    static constexpr int G = QPARAM ? K / (GS > 0 ? GS : 1) : 0;   // groups per row
+    static constexpr int ZRB = G * NBITS / 8;           // packed zero row bytes
+    static constexpr int GRID_X = (N + RPB - 1) / RPB;
+};
+
+template <class C>
+__global__ __launch_bounds__(C::THREADS) void gemv_kernel(
+    const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
+    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
+    using D = Decode<C::NBITS>;
+    constexpr int NW = C::NW, EPC = C::EPC, NCH = C::NCH, T = C::T, IT = C::IT;
+    constexpr int MT = C::MT, U = C::U, STEPS = C::STEPS, V = C::V, WK = C::WK;
+    constexpr int PAIRS = D::PAIRS, NCLS = D::NCLS;
+    constexpr int AR = NW * PAIRS;                     // 32-bit activation registers per chunk
+    constexpr int P8 = 8 / C::NBITS;                   // zero-point fields per byte
+    constexpr uint32_t ZMASK = (1u << C::NBITS) - 1u;
+
+    __shared__ float red[C::WN][WK][STEPS * V];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wk = wave % WK;
+    const int team = wave / WK;
+    const int tt = wk * 64 + lane;
+    const int m0 = blockIdx.y * MT;
+    const int row_base = blockIdx.x * C::RPB + team * C::RPT;
+
+    // ---- per-lane chunk bookkeeping and the stationary activations ----
+    int coff[IT];            // byte offset of the chunk inside a packed weight row
+    int goff[IT];            // group index of the chunk
+    uint32_t a[MT][IT][AR];
+    float c1[MT][IT];        // sum over classes of 1024 * 2^-o * (sum of a in that class)
+    float sa[MT][IT];        // sum of a over the chunk
+
+#pragma unroll
+    for (int it = 0; it < IT; it++) {
+        const int c = tt + T * it;
+        const bool valid = c < NCH;
+        const int cc = valid ? c : 0;
+        coff[it] = cc * C::VB;
+        goff[it] = C::QPARAM ? (cc * EPC) / (C::GS > 0 ? C::GS : 1) : 0;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const int mm = min(m0 + m, m_total - 1);
+            const uint16_t* ap = A + (size_t)mm * C::K + (size_t)cc * EPC;
+            float cls_sum[NCLS];
+#pragma unroll
+            for (int c2 = 0; c2 < NCLS; c2++) cls_sum[c2] = 0.0f;
+#pragma unroll
+            for (int r = 0; r < AR; r += (AR >= 4 ? 4 : AR)) {
+                constexpr int LW = AR >= 4 ? 4 : AR;
+                uint32_t tmp[LW];
+                load_words<LW, false>(ap + 2 * r, tmp);
+#pragma unroll
+                for (int j = 0; j < LW; j++) {
+                    const uint32_t val = valid ? tmp[j] : 0u;
+                    a[m][it][r + j] = val;
+                    const f16x2 h = as_f16x2(val);
+                    cls_sum[D::cls((r + j) % PAIRS)] += (float)h.x + (float)h.y;
+                }
+            }
+            float c1v = 0.0f, sav = 0.0f;
+#pragma unroll
+            for (int c2 = 0; c2 < NCLS; c2++) {
+                c1v += 1024.0f * D::inv_scale(c2) * cls_sum[c2];
+                sav += cls_sum[c2];
+            }
+            c1[m][it] = c1v;
+            sa[m][it] = sav;
+        }
+    }
+
+    // ---- streaming stages ----
+    struct Stage {
+        uint32_t w[U][IT][NW];
+        uint16_t s[U][IT];
+        uint8_t z[U][IT];
+    };
+
+    auto load_stage = [&](Stage& st, int step) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int row = min(row_base + step * U + u, C::N - 1);
+            const uint8_t* wrow = W + (size_t)row * C::RB;
+#pragma unroll
+            for (int it = 0; it < IT; it++) {
+                load_words<NW, C::NT_B>(wrow + coff[it], st.w[u][it]);
+                if constexpr (C::QPARAM) {
+                    st.s[u][it] = S[(size_t)row * C::G + goff[it]];
+                    if constexpr (!C::SYM) st.z[u][it] = Zp[(size_t)row * C::ZRB + goff[it] / P8];
+                }
+            }
+        }
+    };
+
+    auto compute_stage = [&](const Stage& st, int step) {
+        float part[V];
+#pragma unroll
+        for (int v = 0; v < V; v++) part[v] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int it = 0; it < IT; it++) {
+                float acc[MT][NCLS];
+#pragma unroll
+                for (int m = 0; m < MT; m++)
+#pragma unroll
+                    for (int c2 = 0; c2 < NCLS; c2++) acc[m][c2] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < NW; j++) {
+                    uint32_t x[PAIRS];
+                    D::word(st.w[u][it][j], x);
+#pragma unroll
+                    for (int p = 0; p < PAIRS; p++)
+#pragma unroll
+                        for (int m = 0; m < MT; m++)
+                            acc[m][D::cls(p)] = __builtin_amdgcn_fdot2(
+                                as_f16x2(a[m][it][j * PAIRS + p]), as_f16x2(x[p]), acc[m][D::cls(p)], false);
+                }
+                float sc = 1.0f, zf = 0.0f;
+                if constexpr (C::QPARAM) {
+                    sc = f16_bits_to_f32(st.s[u][it]);
+                    if constexpr (C::SYM) {
+                        zf = (float)(1 << (C::NBITS - 1));
+                    } else {
+                        zf = (float)((st.z[u][it] >> ((goff[it] % P8) * C::NBITS)) & ZMASK);
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    float t = acc[m][0];
+#pragma unroll
+                    for (int c2 = 1; c2 < NCLS; c2++) t = __builtin_fmaf(acc[m][c2], D::inv_scale(c2), t);
+                    t -= c1[m][it];                              // = sum a*q over the chunk
+                    if constexpr (C::QPARAM) {
+                        t = __builtin_fmaf(-zf, sa[m][it], t);   // sum a*(q - Z)
+                        part[u * MT + m] = __builtin_fmaf(sc, t, part[u * MT + m]);
+                    } else {
+                        part[u * MT + m] += t;
+                    }
+                }
+            }
+        }
+        wave_reduce_many<V>(part, lane);
+        if (reduce_owner<V>(lane)) red[team][wk][step * V + reduce_index<V>(lane)] = part[0];
+    };
+
+    Stage st0, st1;
+    load_stage(st0, 0);
+#pragma unroll
+    for (int step = 0; step < STEPS; step += 2) {
+        if (step + 1 < STEPS) load_stage(st1, step + 1);
+        compute_stage(st0, step);
+        if (step + 1 < STEPS) {
+            if (step + 2 < STEPS) load_stage(st0, step + 2);
+            compute_stage(st1, step + 1);
+        }
+    }
+
+    __syncthreads();
+
+    // ---- cross-wave sum and the single store of every output element ----
+    for (int j = tt; j < STEPS * V; j += T) {
+        float total = 0.0f;
+#pragma unroll
+        for (int w2 = 0; w2 < WK; w2++) total += red[team][w2][j];
+        const int step = j / V, v = j % V;
+        const int u = v / MT, m = v % MT;
+        const int row = row_base + step * U + u;
+        if (row < C::N && m0 + m < m_total) Cout[(size_t)(m0 + m) * C::N + row] = f32_to_f16_bits(total);
+    }
+}
+
+// Host launcher: static validity checks (return 1 and say why on stderr), then the launch.
+template <class C>
+int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m,
+                hipStream_t stream) {
+    const char* why = nullptr;
+    if (C::NBITS != 2 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 4 or 8 for this kernel";
+    else if (C::VB != 4 && C::VB != 8 && C::VB != 16) why = "VB must be 4, 8 or 16";
+    else if ((C::K * C::NBITS) % (8 * C::VB) != 0) why = "K*NBITS/8 must be a multiple of VB";
+    else if (C::QPARAM && (C::GS <= 0 || C::K % C::GS != 0)) why = "GS must divide K";
+    else if (C::QPARAM && C::GS % C::EPC != 0) why = "a VB-byte chunk must lie inside one group";
+    else if (C::QPARAM && !C::SYM && (C::G % (8 / C::NBITS)) != 0) why = "K/GS must fill whole zero-point bytes";
+    else if ((C::V & (C::V - 1)) != 0 || C::V > 64) why = "U*MT must be a power of two <= 64";
+    else if (C::THREADS > 1024) why = "block too large";
+    else if (C::WN * C::WK * C::STEPS * C::V * 4 > 64 * 1024) why = "reduction scratch exceeds LDS";
+    if (why) {
+        fprintf(stderr, "qfactory gemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT=%d WK=%d WN=%d U=%d STEPS=%d VB=%d)\n",
+                why, C::NBITS, C::GS, C::N, C::K, C::MT, C::WK, C::WN, C::U, C::STEPS, C::VB);
+        return 1;
+    }
+    if (m <= 0) return 0;
+    dim3 grid(C::GRID_X, (m + C::MT - 1) / C::MT);
+    hipLaunchKernelGGL(gemv_kernel<C>, grid, dim3(C::THREADS), 0, stream, (const uint16_t*)A, (const uint8_t*)W,
+                       (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        fprintf(stderr, "qfactory gemv: launch failed: %s\n", hipGetErrorString(err));
+        return 2;
+    }
+    return 0;
+}
+
+}  // namespace qf

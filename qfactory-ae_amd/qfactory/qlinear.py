@@ -1,0 +1,149 @@
+"""``nn.Module`` front end of the quantized linear layer.
+
+Drop-in for the reference's ``qfactory/qlinear.py``: ``QLinear.init(...)`` / ``QLinear.empty(...)``
+return a ``GPTQLinear`` (grouped scales, optional zero-points) or a ``GEMVLinear``
+(``group_size == -1``: raw integer weights) whose ``forward(x)`` maps ``(M, K) fp16`` to ``(M, N) fp16``
+on ``x``'s device.  Attributes ``.w .s .z .func`` keep the reference's meaning (packed tensors and
+the compiled closure for the constructor's ``batch_size``).
+
+Beyond the reference: ``forward`` accepts any number of rows.  The specialisation compiled at
+construction is tuned for ``batch_size``; other row counts get their own specialisation (per M
+bucket) on first use, because the best kernel family changes with M (register-resident GEMV for a
+few rows, matrix-core GEMM for many).
+"""
+import torch
+
+from .convert import convert_params, weight_row_bytes, zero_row_bytes
+from .core import QMatmul, Matmul
+from .core import tiling
+
+
+def _m_bucket(m):
+    """Row count a specialisation is compiled for when ``m`` rows arrive."""
+    if m <= tiling.GEMV_MAX_M:
+        return m
+    if m <= 16:
+        return 16
+    bucket = 32
+    while bucket < m and bucket < 256:
+        bucket *= 2
+    return bucket
+
+
+class GPTQLinear(torch.nn.Module):
+    def __init__(self, in_features, out_features, n_bits, weight, group_size, scale, zero, bias,
+                 compile_flags, skip_convert, batch_size, base_impl=False):
+        super().__init__()
+
+        if bias:
+            raise NotImplementedError("Bias is not supported")
+
+        if skip_convert:
+            w, s, z = weight, scale, zero
+        else:
+            w, s, z = convert_params({
+                "K": in_features,
+                "N": out_features,
+                "NBITS": n_bits,
+                "GS": group_size,
+            }, (weight, scale, zero))
+
+        n_groups = in_features // group_size
+        assert in_features % (group_size * 2) == 0
+        assert w.dtype == torch.int8
+        assert s.dtype == torch.float16
+        assert len(w.shape) == 2
+        assert w.shape[0] * w.shape[1] == out_features * weight_row_bytes(in_features, n_bits)
+        assert s.shape == (out_features, n_groups)
+        if z is not None:
+            assert z.dtype == torch.int8
+            assert z.shape == (out_features, zero_row_bytes(n_groups, n_bits))
+
+        self.in_features, self.out_features = in_features, out_features
+        self.n_bits, self.group_size = n_bits, group_size
+        self.w, self.s, self.z = w, s, z
+        self.compile_flags = dict(compile_flags)
+        self.base_impl = base_impl
+        self.batch_size = batch_size
+
+        self._funcs = {}
+        self.func = self._compile(batch_size, self.compile_flags)
+        self._funcs[_m_bucket(batch_size)] = self.func
+
+    def _compile(self, m, compile_flags):
+        matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
+                         torch.float16, torch.int8, self.group_size, base_impl=self.base_impl)
+        return matmul.compile_profile(**compile_flags)
+
+    def func_for(self, m):
+        bucket = _m_bucket(m)
+        func = self._funcs.get(bucket)
+        if func is None:
+            func = self._funcs[bucket] = self._compile(bucket, self.compile_flags)
+        return func
+
+    def forward(self, x: torch.Tensor):
+        output = torch.empty(x.shape[0], self.w.shape[0], dtype=torch.float16, device=x.device)
+        func = self.func_for(x.shape[0])
+        if self.z is not None:
+            rc = func(x, self.w, output, self.s, self.z)
+        else:
+            rc = func(x, self.w, output, self.s)
+        if rc != 0:
+            raise RuntimeError(f"quantized linear launch failed with return code {rc}")
+        return output
+
+
+class GEMVLinear(torch.nn.Module):
+    def __init__(self, in_features, out_features, n_bits, weight, bias, compile_flags, skip_convert):
+        super().__init__()
+
+        if bias:
+            raise NotImplementedError("Bias is not supported")
+
+        if skip_convert:
+            w = weight
+        else:
+            w = convert_params({
+                "K": in_features,
+                "N": out_features,
+                "NBITS": n_bits,
+            }, (weight,))
+
+        assert w.dtype == torch.int8
+        assert len(w.shape) == 2
+        assert w.shape[0] * w.shape[1] == out_features * weight_row_bytes(in_features, n_bits)
+
+        self.in_features, self.out_features, self.n_bits = in_features, out_features, n_bits
+        self.w = w
+
+        matmul = Matmul(out_features, in_features, n_bits, torch.float16, torch.int8)
+        self.func = matmul.compile_profile(**compile_flags)
+
+    def forward(self, x: torch.Tensor):
+        output = torch.empty(x.shape[0], self.w.shape[0], dtype=torch.float16, device=x.device)
+        rc = self.func(x, self.w, output)
+        if rc != 0:
+            raise RuntimeError(f"quantized linear launch failed with return code {rc}")
+        return output
+
+
+class QLinear():
+    @staticmethod
+    def init(batch_size, in_features, out_features, n_bits, weight, group_size=-1, scale=None,
+             zero=None, bias=False, compile_flags={}):
+        if group_size == -1:
+            return GEMVLinear(in_features, out_features, n_bits, weight, bias, compile_flags,
+                              skip_convert=False)
+        return GPTQLinear(in_features, out_features, n_bits, weight, group_size, scale, zero, bias,
+                          compile_flags, skip_convert=False, batch_size=batch_size)
+
+    @staticmethod
+    def empty(M, K, N, NBITS, GS, sym, compile_flags, base_impl=False):
+        w = torch.empty(N, weight_row_bytes(K, NBITS), dtype=torch.int8, device='cuda')
+        if GS == -1:
+            return GEMVLinear(K, N, NBITS, w, False, compile_flags, skip_convert=True)
+        s = torch.empty(N, K // GS, dtype=torch.float16, device='cuda')
+        z = torch.empty(N, zero_row_bytes(K // GS, NBITS), dtype=torch.int8, device='cuda')
+        return GPTQLinear(K, N, NBITS, w, GS, s, None if sym else z, False, compile_flags,
+                          skip_convert=True, batch_size=M, base_impl=base_impl)

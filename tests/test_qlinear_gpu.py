@@ -1,0 +1,98 @@
+"""GPU parity: QLinear (HIP kernels through the C ABI) against the CPU oracle on seeded inputs.
+
+Tolerances are the acceptance bar: max relative error <= 1e-2 and normalised RMS error <= 1e-3 in
+fp16 (definitions in tests/helpers.py); packed tensors must equal the oracle's bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+import prebuild
+from helpers import assert_close, make_problem, reference_output
+
+pytestmark = pytest.mark.gpu
+
+NO_SEARCH = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
+
+
+def _id(c):
+    return f"M{c['M']}-N{c['N']}-K{c['K']}-b{c['NBITS']}-g{c['GS']}-{'sym' if c['sym'] else 'asym'}"
+
+
+@pytest.fixture(scope="module")
+def qf():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from qfactory import QLinear
+    return QLinear
+
+
+@pytest.mark.parametrize("case", prebuild.parity_cases(), ids=_id)
+def test_qlinear_matches_oracle(qf, oracle, case):
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
+    print(f"[case] {_id(case)}", flush=True)
+    A, weight, scale, zero = make_problem(1234 + N + K + M + nbits, M, N, K, nbits, GS, sym)
+    dev = "cuda"
+    if GS == -1:
+        layer = qf.init(M, K, N, nbits, weight.to(dev), compile_flags={"enable_schedule": False, "enable_lower": False})
+        s = z = None
+    else:
+        layer = qf.init(M, K, N, nbits, weight.to(dev), GS, scale.to(dev),
+                        None if zero is None else zero.to(dev), compile_flags=NO_SEARCH)
+        s, z = layer.s, layer.z
+    # repacked tensors: bit-exact against the oracle's packer
+    assert np.array_equal(layer.w.cpu().numpy(), oracle.pack_weight(weight.numpy(), nbits))
+    if GS != -1:
+        assert np.array_equal(s.cpu().numpy(), oracle.transpose_scale(scale.numpy()))
+        if not sym:
+            assert np.array_equal(z.cpu().numpy(), oracle.pack_zero(zero.numpy(), nbits))
+    out = layer(A.to(dev))
+    torch.cuda.synchronize()
+    assert out.shape == (M, N) and out.dtype == torch.float16 and out.is_cuda
+    # big problems: check a seeded subset of output columns (each is an independent dot product)
+    rows = None
+    if N * K * M > 2 ** 31:
+        rows = np.sort(np.random.default_rng(0).choice(N, size=2048, replace=False))
+    ref = reference_output(oracle, A, layer.w, s, z, nbits, GS, rows)
+    got = out.cpu().numpy()
+    assert_close(oracle, got if rows is None else got[:, rows], ref, _id(case))
+
+
+def test_output_is_fully_overwritten_and_deterministic(qf, oracle):
+    M, N, K, nbits, GS = 1, 100, 256, 4, 128
+    A, weight, scale, zero = make_problem(99, M, N, K, nbits, GS)
+    layer = qf.init(M, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
+    x = A.cuda()
+    first = layer(x).clone()
+    # call the closure on a poisoned output buffer: every element must be rewritten
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    rc = layer.func(x, layer.w, out, layer.s, layer.z)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.equal(out, first)
+
+
+def test_forward_with_other_row_counts_than_constructed(qf, oracle):
+    # the module is built for batch 1 and then fed 1, 2, 3 and 6 rows
+    N, K, nbits, GS = 96, 512, 4, 128
+    _, weight, scale, zero = make_problem(5, 1, N, K, nbits, GS)
+    layer = qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
+    for M in (1, 2, 3, 6):
+        A = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).to(torch.float16)
+        out = layer(A.cuda())
+        ref = reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS)
+        assert_close(oracle, out.cpu().numpy(), ref, f"M={M}")
+
+
+def test_closure_rejects_bad_tensors(qf):
+    N, K, nbits, GS = 64, 256, 4, 128
+    A, weight, scale, zero = make_problem(6, 1, N, K, nbits, GS)
+    layer = qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
+    out = torch.empty(1, N, dtype=torch.float16, device="cuda")
+    x = A.cuda()
+    with pytest.raises(AssertionError):
+        layer.func(x.float(), layer.w, out, layer.s, layer.z)            # dtype
+    with pytest.raises(AssertionError):
+        layer.func(x[:, :128], layer.w, out, layer.s, layer.z)           # K mismatch
+    with pytest.raises(AssertionError):
+        layer.func(x, layer.w.T, out, layer.s, layer.z)                  # shape / contiguity
+    with pytest.raises(NotImplementedError):
+        qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), bias=True)
