@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Workload (BASELINE.json configs[1] at M = 1): the four W4A16 g128 asymmetric quantized linears of a
+Llama-2-7B decoder layer -- fused QKV (12288x4096), O-proj (4096x4096), gate+up (22016x4096) and
+down (4096x11008) -- applied to one fp16 activation row.  One *step* is one pass over those four
+linears for one layer.  Consecutive steps use different layers' weights (NL resident copies, more
+than the 256 MB Infinity Cache in total), so every step streams its weights from HBM as a decode
+pass over a real model does.  All K timed steps are captured in one HIP graph (the launch-bound
+inner loop of a decode step) and replayed once between synchronisations.
+
+Printed JSON: `value` = algorithmic bytes moved per second over the timed region (the reference's
+own footprint formula, reproduce/fig9/plot_bandwidth_size.py:37-44); `roofline` = the dominant
+kernel (gate+up) against the 8 TB/s HBM peak, its duration measured here with HIP events on the
+launch stream; `cpu_baseline` = the torch CPU dequant+matmul port of the reference's test path on
+the same four shapes, on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG_PARENT = os.path.join(ROOT, "qfactory-ae_amd")
+for _p in (ROOT, PKG_PARENT):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+os.environ.setdefault("QFACTORY_CACHE_DIR", os.path.join(PKG_PARENT, "jit_cache"))
+os.environ.setdefault("QFACTORY_LOG_LEVEL", "WARNING")
+
+HBM_PEAK_GBPS = 8000.0
+SHAPES = [("qkv", 12288, 4096), ("o", 4096, 4096), ("gate_up", 22016, 4096), ("down", 4096, 11008)]  # (name, N, K)
+NBITS, GS = 4, 128
+DOMINANT = "gate_up"
+
+
+def algorithmic_bytes(M, N, K, nbits=NBITS, gs=GS, sym=False):
+    b = (M * K + M * N) * 2 + N * K * nbits / 8 + N * (K // gs) * 2
+    if not sym:
+        b += N * (K // gs) * nbits / 8
+    return b
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_layers(n_layers, M):
+    import torch
+    from qfactory import QLinear
+    flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
+    g = torch.Generator(device="cuda").manual_seed(0)
+    layers = []
+    for _ in range(n_layers):
+        layer = {}
+        for name, N, K in SHAPES:
+            lin = QLinear.empty(M, K, N, NBITS, GS, sym=False, compile_flags=flags)
+            lin.w.copy_(torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=g))
+            lin.s.copy_((torch.rand(lin.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
+            lin.z.copy_(torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=g))
+            layer[name] = lin
+        layers.append(layer)
+    acts = {K: torch.randn(M, K, device="cuda", generator=g).to(torch.float16) for K in {k for _, _, k in SHAPES}}
+    return layers, acts
+
+
+def run_step(layer, acts):
+    outs = []
+    for name, N, K in SHAPES:
+        outs.append(layer[name](acts[K]))
+    return outs
+
+
+def check_against_oracle(layer, acts):
+    """One linear of the benchmark data against the CPU oracle (the checker, not the thing timed)."""
+    import numpy as np
+    from oracle import qf_oracle
+    lin = layer["o"]
+    out = lin(acts[4096]).cpu().numpy()
+    rows = np.arange(0, 4096, 8)
+    ref = qf_oracle.qlinear_np(acts[4096].cpu().numpy(), lin.w.cpu().numpy()[rows], lin.s.cpu().numpy()[rows],
+                               lin.z.cpu().numpy()[rows], NBITS, GS)
+    m = qf_oracle.error_metrics(out[:, rows], ref)
+    assert m["max_rel"] <= 1e-2 and m["nrms"] <= 1e-3, f"benchmark data fails parity: {m}"
+    return m
+
+
+def kernel_event_time_us(lins, x, reps=64):
+    """Average duration of one launch of a layer type with cold weights.
+
+    `reps` back-to-back launches (rotating over the layers' distinct weight copies) are captured in
+    a HIP graph on a side stream; the replay is bracketed by HIP events recorded on the stream it is
+    launched on, and the elapsed time is divided by `reps`.  Back-to-back launches on one stream
+    serialise on this GPU, so this is the per-launch duration a kernel trace reports.
+    """
+    import torch
+    outs = [torch.empty(x.shape[0], lin.w.shape[0], dtype=torch.float16, device="cuda") for lin in lins]
+
+    def launches():
+        for i in range(reps):
+            lin, out = lins[i % len(lins)], outs[i % len(lins)]
+            rc = lin.func(x, lin.w, out, lin.s, lin.z)
+            assert rc == 0
+
+    launches()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launches()
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()
+    torch.cuda.synchronize()
+    best = []
+    for _ in range(5):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        best.append(start.elapsed_time(end) * 1e3 / reps)
+    best.sort()
+    return best[len(best) // 2]
+
+
+def cpu_baseline(budget_s=15.0):
+    """torch-CPU dequant + fp32 matmul over the same four shapes, bounded to about `budget_s`."""
+    import torch
+    from oracle import qf_oracle
+    g = torch.Generator().manual_seed(0)
+    probs = []
+    for name, N, K in SHAPES:
+        w = torch.randint(-128, 128, (N, K * NBITS // 8), dtype=torch.int8, generator=g)
+        s = (torch.rand(N, K // GS, generator=g) * 0.019 + 0.001).to(torch.float16)
+        z = torch.randint(-128, 128, (N, K // GS * NBITS // 8), dtype=torch.int8, generator=g)
+        A = torch.randn(1, K, generator=g).to(torch.float16)
+        probs.append((A, w, s, z))
+    total_bytes = sum(algorithmic_bytes(1, N, K) for _, N, K in SHAPES)
+
+    def one_pass():
+        for A, w, s, z in probs:
+            qf_oracle.torch_cpu_forward(A, w, s, z, NBITS, GS)
+
+    one_pass()                                          # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": total_bytes / med / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(times)} passes over the 4 Llama-2-7B W4A16 g128 shapes at M=1 "
+                      f"(torch CPU unpack + fp16 dequant + fp32 matmul), median {med * 1e3:.1f} ms per pass",
+            "ms_per_step": med * 1e3, "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=8, help="distinct resident weight copies cycled through")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the path; this build runs on exactly one GPU (--gpus 1)")
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    torch.cuda.set_device(0)
+    M = 1
+    layers, acts = build_layers(args.layers, M)
+    parity = check_against_oracle(layers[0], acts)
+    log(f"[bench] parity of benchmark data vs oracle: {parity}")
+
+    step_bytes = sum(algorithmic_bytes(M, N, K) for _, N, K in SHAPES)
+
+    for i in range(args.warmup):
+        run_step(layers[i % len(layers)], acts)
+    torch.cuda.synchronize()
+
+    if args.no_graph:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            run_step(layers[i % len(layers)], acts)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    else:
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(args.steps):
+                    run_step(layers[i % len(layers)], acts)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph.replay()                                   # untimed: uploads the graph
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = step_bytes / (elapsed / args.steps) / 1e9
+
+    # per-kernel durations (HIP events on the launch stream), cold weights
+    shapes_report = []
+    dominant = None
+    for name, N, K in SHAPES:
+        us = kernel_event_time_us([layer[name] for layer in layers], acts[K])
+        b = algorithmic_bytes(M, N, K)
+        rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
+               "TFLOP/s": round(2 * M * N * K / us / 1e6, 3), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
+               "bytes": int(b), "kernel": layers[0][name].func.runtime.description}
+        shapes_report.append(rec)
+        log(f"[bench] {name:8s} N={N:6d} K={K:6d}  {us:7.2f} us  {rec['GB/s']:7.1f} GB/s  {100 * rec['hbm_frac']:5.1f}% of HBM peak")
+        if name == DOMINANT:
+            dominant = rec
+
+    result = {
+        "metric": "W4A16 g128 GEMV (M=1) algorithmic HBM throughput over the Llama-2-7B linear shapes",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1] at M=1: W4A16 g128 asymmetric GEMV over Llama-2-7B shapes "
+                               "(12288x4096, 4096x4096, 22016x4096, 4096x11008), one step = the four linears of one layer",
+                   "bits": NBITS, "group_size": GS, "M": M, "weight_copies": args.layers,
+                   "bytes_per_step": int(step_bytes), "timed_with": "eager" if args.no_graph else "one HIP graph of all steps"},
+        "hbm_frac_whole_step": round(value / HBM_PEAK_GBPS, 4),
+        "roofline": {"bound": "hbm", "achieved": dominant["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(dominant["GB/s"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": f"qf::gemv_kernel {DOMINANT} N=22016 K=4096 M=1", "avg_launch_us": dominant["us"],
+                     "algorithmic_bytes_per_launch": dominant["bytes"]},
+        "shapes": shapes_report,
+        "parity": parity,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+        log(f"[bench] cpu baseline: {result['cpu_baseline']}")
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,59 @@
+/*
+ * C ABI of libqfactory_hip.so, the ahead-of-time part of the MI355X quantized-linear path:
+ * device-side repacking (the load-time half of the path) and the memory-system calibration
+ * kernels the benchmark uses to put its roofline numbers on a measured footing.
+ *
+ * All pointers are device addresses owned by the caller; `stream` is a hipStream_t; calls only
+ * enqueue work.  Every function returns 0 on success, 1 on invalid arguments (reason on stderr),
+ * 2 if the HIP launch failed.
+ */
+#ifndef QFACTORY_HIP_H
+#define QFACTORY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Library / interface version: major * 100 + minor. */
+int qf_version(void);
+
+/*
+ * Repack GPTQ-orientation integer weights on the device.
+ *   weight (K, N) int32 row-major, values in [0, 2^nbits)  ->  out (N, K*nbits/8) int8.
+ * nbits in {2, 3, 4, 8}; K must be a multiple of 32.  Bit-identical to the reference's
+ * _transform_weight_basic (qfactory/convert.py:55-68), which this replaces for device tensors;
+ * nbits == 3 produces this project's two-plane layout (no reference counterpart).
+ */
+int qf_pack_weight(const int32_t* weight, int8_t* out, int64_t K, int64_t N, int nbits, void* stream);
+
+/*
+ * Repack zero-points on the device.
+ *   zero (G, N) int32 in [0, 2^nbits)  ->  out (N, G*fb/8) int8 holding min(zero + 1, 2^nbits - 1),
+ * fb = nbits (4 for nbits == 3), group g in field g % (8/fb) of byte g / (8/fb).
+ * Replaces _transform_zero (qfactory/convert.py:74-81).
+ */
+int qf_pack_zero(const int32_t* zero, int8_t* out, int64_t G, int64_t N, int nbits, void* stream);
+
+/*
+ * scale (G, N) fp16 -> out (N, G) fp16.  Replaces _transform_scale (qfactory/convert.py:70-72).
+ */
+int qf_transpose_scale(const uint16_t* scale, uint16_t* out, int64_t G, int64_t N, void* stream);
+
+/*
+ * Calibration kernels (no reference counterpart; the reference times with triton's do_bench only,
+ * qfactory/profile.py:5-10).  qf_stream_read reads `bytes` (multiple of 16) with 128-bit loads and
+ * writes one checksum word per block to `sink` (>= 4096 uint32); qf_stream_copy copies `bytes`
+ * (multiple of 16) from src to dst.  They give the achievable HBM rate for a given footprint and a
+ * known-traffic dispatch against which hardware counters can be scaled.
+ */
+int qf_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
+int qf_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* QFACTORY_HIP_H */

@@ -42,7 +42,18 @@ def parity_cases():
               _case(1, 256, 11008, 4, 128)]
     for nbits in (2, 4, 8):                                  # group_size == -1: raw integer weights
         cases += [_case(1, 4096, 4096, nbits, -1), _case(3, 100, 256, nbits, -1)]
+    # matrix-core regime: ragged M and N, M above one block tile, other widths and group sizes
+    cases += [_case(33, 100, 512, 4, 128), _case(100, 1000, 1024, 4, 64), _case(300, 256, 2048, 4, 128),
+              _case(48, 130, 1024, 2, 64), _case(17, 96, 512, 8, 32), _case(64, 512, 1024, 4, 128, True),
+              _case(128, 256, 11008, 4, 128)]
     return cases
+
+
+def large_parity_cases():
+    """W4A16 g128 GEMM at M in {32..256} on Llama-3-70B-style shapes.  The weights are too large to
+    build from int32 tensors in a test; the tests fill packed tensors directly (every byte pattern
+    is a valid packed weight) and check a seeded subset of output columns."""
+    return [_case(M, N, K) for N, K in LLAMA3_70B for M in (32, 64, 128, 256)]
 
 
 def bench_cases():
@@ -61,7 +72,7 @@ def misc_test_cases():
 
 def all_cases():
     seen, out = set(), []
-    for c in parity_cases() + bench_cases() + smoke_cases() + misc_test_cases():
+    for c in parity_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases():
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)

@@ -15,11 +15,15 @@ Two regimes:
 
 NUM_CUS = 256
 GEMV_MAX_M = 4          # largest M served by the dot2 GEMV before the MFMA kernel takes over
-MFMA_AVAILABLE = False  # flipped once include/qf_mfma.hip.h provides qf::MfmaCfg / mfma_launch
+MFMA_AVAILABLE = True
 
 
-def regime_for(M):
-    return "gemv" if (M <= GEMV_MAX_M or not MFMA_AVAILABLE) else "mfma"
+def regime_for(M, K=None, nbits=None, group_size=None):
+    if M <= GEMV_MAX_M or not MFMA_AVAILABLE:
+        return "gemv"
+    if K is not None and not mfma_supported(K, nbits, group_size):
+        return "gemv"
+    return "mfma"
 
 
 def elements_per_chunk(nbits, vb):
@@ -47,7 +51,7 @@ def _pow2_floor(x):
 
 
 def gemv_wave_split(K, nbits, vb, mt, max_waves=8, a_reg_budget=128):
-    """(WK, IT) choices ranked by idle-lane waste, then by fewer waves."""
+    """(WK, IT) choices ranked by idle-lane waste, then by fewer chunks per lane (more waves)."""
     epc = elements_per_chunk(nbits, vb)
     nch = K // epc
     a_regs_per_chunk = epc // 2
@@ -57,7 +61,7 @@ def gemv_wave_split(K, nbits, vb, mt, max_waves=8, a_reg_budget=128):
         if it * a_regs_per_chunk * mt > a_reg_budget:
             continue
         waste = (64 * wk * it - nch) / nch
-        out.append((waste, wk * it, wk, it))
+        out.append((round(waste, 3), it, wk, it))
     if not out:
         wk = max_waves
         out.append((0.0, 0, wk, -(-nch // (64 * wk))))
@@ -78,14 +82,13 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
         it = -(-(K // elements_per_chunk(nbits, vb)) // (64 * wk))
     if u is None:
         # keep about 8 x 16 bytes of weight in flight per lane and stage, U*MT a power of two <= 64
-        u = max(1, min(8 // it if it <= 8 else 1, 64 // mt))
+        u = max(1, min(8 // it if it <= 8 else 1, 64 // mt, 8))
         u = _pow2_floor(u)
     if wn is None:
-        wn = max(1, 4 // wk)                          # blocks of about four waves
+        wn = 2 if wk * 2 <= 16 else 1                 # two teams per block measured best on MI355X
     if steps is None:
-        # aim at >= 2 blocks per CU but let a team amortise its activation load over >= 8 rows
-        rows_per_team = max(u, min(32, N // (2 * NUM_CUS * wn)))
-        steps = max(1, rows_per_team // u)
+        # a team amortises its activation load over about 8 rows
+        steps = max(1, 8 // u)
     return {"MT": mt, "WK": wk, "WN": wn, "U": u, "STEPS": steps, "VB": vb}
 
 
@@ -112,3 +115,74 @@ def gemv_candidates(M, N, K, nbits, group_size):
                 for steps in (1, 2, 4):
                     add({"MT": mt, "WK": wk, "WN": wn, "U": u, "STEPS": steps, "VB": vb})
     return out
+
+
+# --------------------------------------------------------------------------------------------
+# MFMA regime
+# --------------------------------------------------------------------------------------------
+
+def mfma_supported(K, nbits, group_size):
+    """The matrix-core kernel needs whole K-iterations and a lane's 16 bytes inside one group."""
+    if nbits not in (2, 4, 8):
+        return False
+    epl = 128 // nbits
+    return K % (4 * epl) == 0 and group_size % epl == 0
+
+
+def mfma_tiling(M, N, K, nbits, group_size, **pins):
+    """Default tile shape: AT x BT 16-row tiles per wave, WM x WN x WK waves per block."""
+    m16 = -(-M // 16)
+    if m16 <= 4:
+        at, wm = m16, 1
+    elif m16 <= 8:
+        at, wm = (m16 + 1) // 2, 2
+    else:
+        at, wm = 4, 4
+    bt = 2
+    wn = max(1, 4 // wm)
+    iters = K // (4 * (128 // nbits))
+    wk = 1
+    # small tiles leave the machine empty: split K over waves of the block until there are
+    # 8 waves per block or the K-iterations run out
+    while wm * wn * wk < 8 and wk * 2 <= iters and m16 <= 2:
+        wk *= 2
+    # too few blocks for 256 CUs: narrow the block along N
+    while (N // (wn * bt * 16)) < 2 * NUM_CUS and wn > 1:
+        wn //= 2
+    if (N // (wn * bt * 16)) < NUM_CUS and bt > 1:
+        bt = 1
+    cfg = {"AT": at, "BT": bt, "WM": wm, "WN": wn, "WK": wk}
+    cfg.update(pins)
+    return cfg
+
+
+def mfma_candidates(M, N, K, nbits, group_size):
+    base = mfma_tiling(M, N, K, nbits, group_size)
+    seen, out = set(), []
+    iters = K // (4 * (128 // nbits))
+
+    def add(cfg):
+        key = tuple(sorted(cfg.items()))
+        threads = 64 * cfg["WM"] * cfg["WN"] * cfg["WK"]
+        if key in seen or threads > 1024 or cfg["WK"] > iters or cfg["AT"] * cfg["BT"] > 32:
+            return
+        seen.add(key)
+        out.append(cfg)
+
+    add(base)
+    m16 = -(-M // 16)
+    for wm in (1, 2, 4):
+        at = -(-m16 // wm)
+        if at > 8:
+            at = 4
+        for bt in (1, 2, 4):
+            for wn in (1, 2, 4):
+                for wk in (1, 2, 4):
+                    add({"AT": at, "BT": bt, "WM": wm, "WN": wn, "WK": wk})
+    return out
+
+
+def mfma_cfg_string(problem, t, decode_strategy, nt_b):
+    b = lambda x: "true" if x else "false"
+    return (f"qf::MfmaCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
+            f"{t['AT']}, {t['BT']}, {t['WM']}, {t['WN']}, {t['WK']}, {b(nt_b)}>")

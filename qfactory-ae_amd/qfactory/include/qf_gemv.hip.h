@@ -78,49 +78,17 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
     const int m0 = blockIdx.y * MT;
     const int row_base = blockIdx.x * C::RPB + team * C::RPT;
 
-    // ---- per-lane chunk bookkeeping and the stationary activations ----
+    // ---- per-lane chunk bookkeeping ----
     int coff[IT];            // byte offset of the chunk inside a packed weight row
     int goff[IT];            // group index of the chunk
-    uint32_t a[MT][IT][AR];
-    float c1[MT][IT];        // sum over classes of 1024 * 2^-o * (sum of a in that class)
-    float sa[MT][IT];        // sum of a over the chunk
-
+    bool cvalid[IT];
 #pragma unroll
     for (int it = 0; it < IT; it++) {
         const int c = tt + T * it;
-        const bool valid = c < NCH;
-        const int cc = valid ? c : 0;
+        cvalid[it] = c < NCH;
+        const int cc = cvalid[it] ? c : 0;
         coff[it] = cc * C::VB;
         goff[it] = C::QPARAM ? (cc * EPC) / (C::GS > 0 ? C::GS : 1) : 0;
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const int mm = min(m0 + m, m_total - 1);
-            const uint16_t* ap = A + (size_t)mm * C::K + (size_t)cc * EPC;
-            float cls_sum[NCLS];
-#pragma unroll
-            for (int c2 = 0; c2 < NCLS; c2++) cls_sum[c2] = 0.0f;
-#pragma unroll
-            for (int r = 0; r < AR; r += (AR >= 4 ? 4 : AR)) {
-                constexpr int LW = AR >= 4 ? 4 : AR;
-                uint32_t tmp[LW];
-                load_words<LW, false>(ap + 2 * r, tmp);
-#pragma unroll
-                for (int j = 0; j < LW; j++) {
-                    const uint32_t val = valid ? tmp[j] : 0u;
-                    a[m][it][r + j] = val;
-                    const f16x2 h = as_f16x2(val);
-                    cls_sum[D::cls((r + j) % PAIRS)] += (float)h.x + (float)h.y;
-                }
-            }
-            float c1v = 0.0f, sav = 0.0f;
-#pragma unroll
-            for (int c2 = 0; c2 < NCLS; c2++) {
-                c1v += 1024.0f * D::inv_scale(c2) * cls_sum[c2];
-                sav += cls_sum[c2];
-            }
-            c1[m][it] = c1v;
-            sa[m][it] = sav;
-        }
     }
 
     // ---- streaming stages ----
@@ -145,6 +113,48 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
             }
         }
     };
+
+    // The first stage of weights goes out before anything else so that its HBM latency overlaps
+    // the activation loads and their bookkeeping.
+    Stage st0, st1;
+    load_stage(st0, 0);
+
+    // ---- the stationary activations and their per-chunk sums ----
+    uint32_t a[MT][IT][AR];
+    float c1[MT][IT];        // sum over classes of 1024 * 2^-o * (sum of a in that class)
+    float sa[MT][IT];        // sum of a over the chunk
+#pragma unroll
+    for (int it = 0; it < IT; it++) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const int mm = min(m0 + m, m_total - 1);
+            const uint16_t* ap = A + (size_t)mm * C::K + (size_t)(coff[it] / C::VB) * EPC;
+            float cls_sum[NCLS];
+#pragma unroll
+            for (int c2 = 0; c2 < NCLS; c2++) cls_sum[c2] = 0.0f;
+#pragma unroll
+            for (int r = 0; r < AR; r += (AR >= 4 ? 4 : AR)) {
+                constexpr int LW = AR >= 4 ? 4 : AR;
+                uint32_t tmp[LW];
+                load_words<LW, false>(ap + 2 * r, tmp);
+#pragma unroll
+                for (int j = 0; j < LW; j++) {
+                    const uint32_t val = cvalid[it] ? tmp[j] : 0u;
+                    a[m][it][r + j] = val;
+                    const f16x2 h = as_f16x2(val);
+                    cls_sum[D::cls((r + j) % PAIRS)] += (float)h.x + (float)h.y;
+                }
+            }
+            float c1v = 0.0f, sav = 0.0f;
+#pragma unroll
+            for (int c2 = 0; c2 < NCLS; c2++) {
+                c1v += 1024.0f * D::inv_scale(c2) * cls_sum[c2];
+                sav += cls_sum[c2];
+            }
+            c1[m][it] = c1v;
+            sa[m][it] = sav;
+        }
+    }
 
     auto compute_stage = [&](const Stage& st, int step) {
         float part[V];
@@ -195,11 +205,19 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
             }
         }
         wave_reduce_many<V>(part, lane);
-        if (reduce_owner<V>(lane)) red[team][wk][step * V + reduce_index<V>(lane)] = part[0];
+        if (reduce_owner<V>(lane)) {
+            const int v = reduce_index<V>(lane);
+            if constexpr (WK == 1) {          // one wave owns the rows: store straight from the lane
+                const int u = v / MT, m = v % MT;
+                const int row = row_base + step * U + u;
+                if (row < C::N && m0 + m < m_total)
+                    Cout[(size_t)(m0 + m) * C::N + row] = f32_to_f16_bits(part[0]);
+            } else {
+                red[team][wk][step * V + v] = part[0];
+            }
+        }
     };
 
-    Stage st0, st1;
-    load_stage(st0, 0);
 #pragma unroll
     for (int step = 0; step < STEPS; step += 2) {
         if (step + 1 < STEPS) load_stage(st1, step + 1);
@@ -210,6 +228,7 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
         }
     }
 
+    if constexpr (WK == 1) return;
     __syncthreads();
 
     // ---- cross-wave sum and the single store of every output element ----

@@ -57,6 +57,28 @@ def test_qlinear_matches_oracle(qf, oracle, case):
     assert_close(oracle, got if rows is None else got[:, rows], ref, _id(case))
 
 
+@pytest.mark.parametrize("case", prebuild.large_parity_cases(), ids=_id)
+def test_large_gemm_matches_oracle_on_sampled_columns(qf, oracle, case):
+    """Llama-3-70B-style shapes at M = 32..256: packed tensors are filled directly with seeded
+    random bytes (any byte pattern is a valid packed weight / zero tensor); 1024 seeded output
+    columns are checked against the oracle -- every output column is an independent dot product."""
+    M, N, K, nbits, GS = (case[k] for k in ("M", "N", "K", "NBITS", "GS"))
+    print(f"[case] {_id(case)}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(N + K + M)
+    layer = qf.empty(M, K, N, nbits, GS, sym=False, compile_flags=NO_SEARCH)
+    layer.w.copy_(torch.randint(-128, 128, layer.w.shape, dtype=torch.int8, device="cuda", generator=g))
+    layer.s.copy_((torch.rand(layer.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
+    layer.z.copy_(torch.randint(-128, 128, layer.z.shape, dtype=torch.int8, device="cuda", generator=g))
+    A = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
+    out = layer(A)
+    torch.cuda.synchronize()
+    rows = np.sort(np.random.default_rng(N + M).choice(N, size=1024, replace=False))
+    rows_t = torch.from_numpy(rows).cuda()
+    ref = oracle.qlinear_np(A.cpu().numpy(), layer.w[rows_t].cpu().numpy(), layer.s[rows_t].cpu().numpy(),
+                            layer.z[rows_t].cpu().numpy(), nbits, GS)
+    assert_close(oracle, out[:, rows_t].cpu().numpy(), ref, _id(case))
+
+
 def test_output_is_fully_overwritten_and_deterministic(qf, oracle):
     M, N, K, nbits, GS = 1, 100, 256, 4, 128
     A, weight, scale, zero = make_problem(99, M, N, K, nbits, GS)
