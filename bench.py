@@ -30,6 +30,8 @@ os.environ.setdefault("QFACTORY_CACHE_DIR", os.path.join(PKG_PARENT, "jit_cache"
 os.environ.setdefault("QFACTORY_LOG_LEVEL", "WARNING")
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2516.6          # 256 CUs x 4096 FLOP/clk x 2.4 GHz, dense fp16
+GEMM_SHAPES = [("qkv70b", 10240, 8192), ("o70b", 8192, 8192), ("gate_up70b", 57344, 8192), ("down70b", 8192, 28672)]
 SHAPES = [("qkv", 12288, 4096), ("o", 4096, 4096), ("gate_up", 22016, 4096), ("down", 4096, 11008)]  # (name, N, K)
 NBITS, GS = 4, 128
 DOMINANT = "gate_up"
@@ -126,6 +128,37 @@ def kernel_event_time_us(lins, x, reps=64):
     return best[len(best) // 2]
 
 
+def gemm_report(M=256, copies_bytes=600e6):
+    """BASELINE.json configs[3] at M = 256: W4A16 g128 GEMM on Llama-3-70B-style shapes, per shape
+    microseconds, TFLOP/s and the fraction of the dense fp16 MFMA peak."""
+    import torch
+    from qfactory import QLinear
+    flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
+    g = torch.Generator(device="cuda").manual_seed(1)
+    report = []
+    for name, N, K in GEMM_SHAPES:
+        n_copies = max(2, min(8, int(copies_bytes // (N * K // 2))))
+        lins = []
+        for _ in range(n_copies):
+            lin = QLinear.empty(M, K, N, NBITS, GS, sym=False, compile_flags=flags)
+            lin.w.copy_(torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=g))
+            lin.s.copy_((torch.rand(lin.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
+            lin.z.copy_(torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=g))
+            lins.append(lin)
+        x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
+        us = kernel_event_time_us(lins, x, reps=2 * n_copies)
+        flops = 2.0 * M * N * K
+        rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1),
+               "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
+               "GB/s": round(algorithmic_bytes(M, N, K) / us / 1e3, 1), "kernel": lins[0].func.runtime.description}
+        report.append(rec)
+        log(f"[bench] GEMM M={M} {name:11s} N={N:6d} K={K:6d} {us:8.2f} us {rec['TFLOP/s']:7.1f} TFLOP/s "
+            f"{100 * rec['mfma_frac']:5.1f}% of fp16 MFMA peak")
+        del lins
+        torch.cuda.empty_cache()
+    return report
+
+
 def cpu_baseline(budget_s=15.0):
     """torch-CPU dequant + fp32 matmul over the same four shapes, bounded to about `budget_s`."""
     import torch
@@ -166,6 +199,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--layers", type=int, default=8, help="distinct resident weight copies cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the M=256 GEMM report")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -242,6 +276,8 @@ def main():
         "shapes": shapes_report,
         "parity": parity,
     }
+    if not args.no_gemm:
+        result["gemm_m256"] = {"peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS, "shapes": gemm_report(256)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
         log(f"[bench] cpu baseline: {result['cpu_baseline']}")
