@@ -103,6 +103,8 @@ class QMatmulQFunc(QFunc):
         nbits, gs = self.qtile_b.nbits, self.qtile_b.quant_granularity[1]
         if regime == "gemv":
             return tiling.gemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
+        if regime == "mgemv":
+            return tiling.mgemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
         return tiling.mfma_tiling(p["M"], p["N"], p["K"], nbits, gs)
 
     def arg_name_type(self):
@@ -114,9 +116,9 @@ class QMatmulQFunc(QFunc):
 
     # -- search space -------------------------------------------------------------------------
     def transform(self) -> List[QFunc]:
-        if self.regime == "gemv":
-            return [self.clone(decode_strategy="deferred")]
-        return [self.clone(decode_strategy=d) for d in ("eager", "deferred")]
+        # one decode strategy per kernel family today: the dot2 GEMV defers scale/zero to fp32,
+        # the matrix-core kernels dequantise eagerly (bit-identical weights to the reference)
+        return [self.clone()]
 
     def schedule(self) -> List[QFunc]:
         return [self.clone(l2cache_a=True, l2cache_b=b) for b in (False, True)]
@@ -125,6 +127,8 @@ class QMatmulQFunc(QFunc):
         p = self.problem
         if self.regime == "gemv":
             cands = tiling.gemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
+        elif self.regime == "mgemv":
+            cands = tiling.mgemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         else:
             cands = tiling.mfma_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         return [self.clone(tiling_configs=c) for c in cands]
@@ -135,11 +139,17 @@ class QMatmulQFunc(QFunc):
         t = self.tiling_configs
         b = lambda x: "true" if x else "false"
         code = "// QFactory-HIP generated translation unit\n\n"
+        for name, value in sorted(getattr(self, "defines", {}).items()):   # kernel-header tuning knobs
+            code += f"#define {name} {value}\n"
         if self.regime == "gemv":
             code += '#include "qf_gemv.hip.h"\n'
             cfg = (f"qf::GemvCfg<{p['NBITS']}, {p['GS']}, {b(p['SYM'])}, true, {p['N']}, {p['K']}, "
                    f"{t['MT']}, {t['WK']}, {t['WN']}, {t['U']}, {t['STEPS']}, {t['VB']}, {b(not self.l2cache_b)}>")
             call = "qf::gemv_launch<Cfg>"
+        elif self.regime == "mgemv":
+            code += '#include "qf_mgemv.hip.h"\n'
+            cfg = tiling.mgemv_cfg_string(p, t, not self.l2cache_b)
+            call = "qf::mgemv_launch<Cfg>"
         elif self.regime == "mfma":
             code += '#include "qf_mfma.hip.h"\n'
             cfg = tiling.mfma_cfg_string(p, t, self.decode_strategy, not self.l2cache_b)

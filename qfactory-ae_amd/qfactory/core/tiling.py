@@ -18,10 +18,18 @@ GEMV_MAX_M = 4          # largest M served by the dot2 GEMV before the MFMA kern
 MFMA_AVAILABLE = True
 
 
+MGEMV_MIN_M = 3         # below: dot2 GEMV; [MGEMV_MIN_M, MGEMV_MAX_M]: A-stationary MFMA kernel
+MGEMV_MAX_M = 32
+
+
 def regime_for(M, K=None, nbits=None, group_size=None):
-    if M <= GEMV_MAX_M or not MFMA_AVAILABLE:
+    if M < MGEMV_MIN_M or not MFMA_AVAILABLE:
         return "gemv"
-    if K is not None and not mfma_supported(K, nbits, group_size):
+    if K is None or not mfma_supported(K, nbits, group_size):
+        return "gemv"
+    if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
+        return "mgemv"
+    if M <= GEMV_MAX_M:
         return "gemv"
     return "mfma"
 
@@ -186,3 +194,82 @@ def mfma_cfg_string(problem, t, decode_strategy, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::MfmaCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
             f"{t['AT']}, {t['BT']}, {t['WM']}, {t['WN']}, {t['WK']}, {b(nt_b)}>")
+
+
+# --------------------------------------------------------------------------------------------
+# A-stationary MFMA regime (2 <= M <= 64)
+# --------------------------------------------------------------------------------------------
+
+def mgemv_regs(mt16, ch, pf, nbits):
+    """Rough VGPR need of qf::mgemv_kernel: resident activations, the ring of weight stages and
+    the fragment copy of the tile being consumed."""
+    ksteps = (128 // nbits) // 8
+    return mt16 * ch * ksteps * 4 + pf * (ch * 4 + 4) + ch * 4 + 48
+
+
+def mgemv_reg_limit(wk):
+    waves_per_simd = -(-wk // 4)
+    return min(512, 512 // waves_per_simd)
+
+
+def mgemv_tiling(M, N, K, nbits, group_size, max_waves=16, **pins):
+    """MT16 activation tiles resident per wave, WK waves x CH chunks covering K, PF weight tiles in
+    flight; None if the activations do not fit the register file of one block."""
+    if not mfma_supported(K, nbits, group_size):
+        return None
+    chunk = 4 * (128 // nbits)
+    if group_size % chunk and chunk % group_size:
+        return None
+    mt16 = -(-M // 16)
+    nchunk = K // chunk
+    best = None
+    for ch in (16, 8, 4, 2, 1):
+        if ch > nchunk:
+            continue
+        wk = -(-nchunk // ch)
+        if wk > max_waves or (wk - 1) * ch >= nchunk:
+            continue
+        for pf in (2, 4, 1):
+            if mgemv_regs(mt16, ch, pf, nbits) > mgemv_reg_limit(wk):
+                continue
+            waste = wk * ch - nchunk
+            key = (waste > ch // 2, -wk, pf != 2, waste)      # more, thinner waves measured best on MI355X
+            if best is None or key < best[0]:
+                best = (key, wk, ch, pf)
+    if best is None:
+        return None
+    _, wk, ch, pf = best
+    cfg = {"MT16": mt16, "WK": wk, "CH": ch, "PB": NUM_CUS, "PF": pf}
+    cfg.update(pins)
+    return cfg
+
+
+def mgemv_candidates(M, N, K, nbits, group_size):
+    base = mgemv_tiling(M, N, K, nbits, group_size)
+    if base is None:
+        return []
+    seen, out = set(), []
+    nchunk = K // (4 * (128 // nbits))
+
+    def add(cfg):
+        key = tuple(sorted(cfg.items()))
+        ok = (cfg["WK"] <= 16 and cfg["WK"] * cfg["CH"] >= nchunk and (cfg["WK"] - 1) * cfg["CH"] < nchunk
+              and cfg["CH"] <= nchunk
+              and mgemv_regs(cfg["MT16"], cfg["CH"], cfg["PF"], nbits) <= mgemv_reg_limit(cfg["WK"]))
+        if ok and key not in seen:
+            seen.add(key)
+            out.append(cfg)
+
+    add(base)
+    for ch in (1, 2, 4, 8, 16):
+        wk = -(-nchunk // ch)
+        for pb in (NUM_CUS // 2, NUM_CUS, 2 * NUM_CUS):
+            for pf in (1, 2, 4):
+                add({"MT16": base["MT16"], "WK": wk, "CH": ch, "PB": pb, "PF": pf})
+    return out
+
+
+def mgemv_cfg_string(problem, t, nt_b):
+    b = lambda x: "true" if x else "false"
+    return (f"qf::MGemvCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
+            f"{t['MT16']}, {t['WK']}, {t['CH']}, {t['PB']}, {t['PF']}, {b(nt_b)}>")

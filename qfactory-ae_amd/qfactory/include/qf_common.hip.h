@@ -11,7 +11,33 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// Scheduling fence between "issue the loads" and "consume earlier loads" regions.  0: none,
+// 1: full scheduling barrier.
+#ifndef QF_SCHED_FENCE_MODE
+#define QF_SCHED_FENCE_MODE 0
+#endif
+#if QF_SCHED_FENCE_MODE == 1
+#define QF_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define QF_SCHED_FENCE() ((void)0)
+#endif
+
+// Register holders of prefetched scale / zero-point loads.  1: 32-bit (the zero-extended load
+// result stays untouched until its use), 0: 16- and 8-bit members (the compiler may pack them,
+// which touches a load result right after its issue).
+#ifndef QF_WIDE_HOLDERS
+#define QF_WIDE_HOLDERS 1
+#endif
+
 namespace qf {
+
+#if QF_WIDE_HOLDERS
+typedef uint32_t scale_holder_t;
+typedef uint32_t zero_holder_t;
+#else
+typedef uint16_t scale_holder_t;
+typedef uint8_t zero_holder_t;
+#endif
 
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));

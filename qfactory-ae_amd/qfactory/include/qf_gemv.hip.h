@@ -94,8 +94,8 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
     // ---- streaming stages ----
     struct Stage {
         uint32_t w[U][IT][NW];
-        uint16_t s[U][IT];
-        uint8_t z[U][IT];
+        scale_holder_t s[U][IT];
+        zero_holder_t z[U][IT];
     };
 
     auto load_stage = [&](Stage& st, int step) {
@@ -118,6 +118,7 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
     // the activation loads and their bookkeeping.
     Stage st0, st1;
     load_stage(st0, 0);
+    QF_SCHED_FENCE();      // keep every stage-0 load ahead of the activation loads
 
     // ---- the stationary activations and their per-chunk sums ----
     uint32_t a[MT][IT][AR];
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
                 }
                 float sc = 1.0f, zf = 0.0f;
                 if constexpr (C::QPARAM) {
-                    sc = f16_bits_to_f32(st.s[u][it]);
+                    sc = f16_bits_to_f32((uint16_t)st.s[u][it]);
                     if constexpr (C::SYM) {
                         zf = (float)(1 << (C::NBITS - 1));
                     } else {
@@ -218,12 +219,19 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
         }
     };
 
+    QF_SCHED_FENCE();
 #pragma unroll
     for (int step = 0; step < STEPS; step += 2) {
-        if (step + 1 < STEPS) load_stage(st1, step + 1);
+        if (step + 1 < STEPS) {
+            load_stage(st1, step + 1);
+            QF_SCHED_FENCE();  // the prefetch is issued before any compute of this step
+        }
         compute_stage(st0, step);
         if (step + 1 < STEPS) {
-            if (step + 2 < STEPS) load_stage(st0, step + 2);
+            if (step + 2 < STEPS) {
+                load_stage(st0, step + 2);
+                QF_SCHED_FENCE();
+            }
             compute_stage(st1, step + 1);
         }
     }

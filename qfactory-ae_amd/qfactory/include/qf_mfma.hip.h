@@ -172,8 +172,8 @@ __global__ __launch_bounds__(C::THREADS) void mfma_kernel(
 
     struct WStage {
         uint32_t w[BT][4];
-        uint16_t s[BT];
-        uint8_t z[BT];
+        scale_holder_t s[BT];
+        zero_holder_t z[BT];
     };
     auto load_w = [&](WStage& st, int it) {
         const int itc = min(it, C::IT_TOTAL - 1);
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(C::THREADS) void mfma_kernel(
             for (int j = 0; j < BT; j++) {
                 const int zero = C::SYM ? (1 << (C::NBITS - 1))
                                         : (int)((wcur.z[j] >> ((g % P8) * C::NBITS)) & ZMASK);
-                qc[j] = make_qconst<C::NBITS>(wcur.s[j], zero);
+                qc[j] = make_qconst<C::NBITS>((uint16_t)wcur.s[j], zero);
             }
             const uint16_t* abase = As + ((size_t)(buf * WK + wk) * C::BM + wm * AT * 16 + r) * PITCH + kb * EPL;
 #pragma unroll

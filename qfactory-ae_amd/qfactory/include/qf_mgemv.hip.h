@@ -1,0 +1,398 @@
+// Dequant-fused low-bit "skinny GEMM" on the gfx950 matrix cores for 2 <= M <= 32, HBM-bound.
+//
+//   C[m][n] = fp16( sum_g s[n][g] * sum_{k in g} A[m][k] * (q[n][k] - Z[n][g]) )
+//
+// Same operands as the reference's kernel_gptq (qfactory/include/gptq_gemv.h:14-154) in its
+// deferred-decode form (utils.h:193-213): the integer part is summed first, the scale is applied
+// once per group -- here in fp32 and on the matrix cores.  Organised like qf::gemv_kernel: the
+// packed weights are read exactly once, straight from the reference layout.
+//
+//   * Persistent blocks: at most PB blocks, each sweeping SLOTS 16-row weight tiles, so the
+//     activations are fetched once per block and not once per tile.
+//   * A team of WK waves splits K; wave wk owns CH consecutive "chunks" (a chunk is the 4*128/NBITS
+//     elements that one 16-byte load per lane covers for 16 weight rows).  The activations of a
+//     wave's chunks stay in VGPRs in MFMA fragment order (A-stationary): no LDS staging and no
+//     barrier in the main loop.
+//   * Per tile: CH 16-byte loads per lane (next tile prefetched); fields are masked in place
+//     (1024 + 2^o*q) and brought to the exact integer q - Z with one packed fp16 add or fma;
+//     v_mfma_f32_16x16x32_f16 with the activations as source A (rows m) and the weights as source
+//     B (columns n), so a lane holds one n and needs one scale: acc += s * group_sum in fp32.
+//   * Each wave parks its partial 16x16 tiles in its own LDS slots; one barrier at the end of the
+//     block, then the partials of the WK waves are summed and every output is written once.
+#pragma once
+
+#include <cstdio>
+#include "qf_common.hip.h"
+
+namespace qf {
+
+template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_>
+struct MGemvCfg {
+    static constexpr int NBITS = NBITS_, GS = GS_, N = N_, K = K_;
+    static constexpr bool SYM = SYM_, NT_B = NT_B_;
+    static constexpr int MT16 = MT16_;             // 16-row activation tiles held per wave
+    static constexpr int WK = WK_;                 // waves along K per team
+    static constexpr int CH = CH_;                 // chunks per wave
+    static constexpr int PB = PB_;                 // upper bound on blocks along N
+    static constexpr int EPL = 128 / NBITS;        // fields per lane and 16-byte load
+    static constexpr int KSTEPS = EPL / 8;         // MFMA k-steps per chunk
+    static constexpr int CHUNK = 4 * EPL;          // elements of K per chunk
+    static constexpr int NCHUNK = K / CHUNK;
+    static constexpr int THREADS = 64 * WK;
+    static constexpr int BM = 16 * MT16;
+    static constexpr int NT = (N + 15) / 16;       // 16-row weight tiles
+    static constexpr int GRID_X = NT < PB ? NT : PB;
+    static constexpr int SLOTS = (NT + GRID_X - 1) / GRID_X;               // tiles per block
+    static constexpr int PF = PF_;                 // weight tiles in flight per wave (ring of stages): 2 or 4
+    static constexpr int SB = 4;                   // tiles per batch: partials are reduced and stored per batch
+    static constexpr int NBATCH = (SLOTS + SB - 1) / SB;
+    static constexpr int RB = K * NBITS / 8;
+    static constexpr int G = K / GS;
+    static constexpr int ZRB = G * NBITS / 8;
+    static constexpr bool DEFERRED = (GS % CHUNK == 0);      // a chunk lies inside one group
+    static constexpr int LPR = CH * 4;             // lanes covering one row's K-slice (CH*64 bytes)
+    static constexpr int RPI = 64 / LPR;           // rows per coalesced weight load
+    // groups and zero-point bytes of one row inside a wave's K-slice
+    // (upper bounds when a slice may start inside a group / inside a byte; indices are clamped to the row)
+    static constexpr int GWN = (GS <= CHUNK) ? CH * CHUNK / GS : (CH * CHUNK) / GS + 2;
+    static constexpr int ZB = (GWN * NBITS + 7) / 8 + 1;
+    static constexpr int WBUF_W = 16 * (CH * 64 + 16);
+    static constexpr int WBUF_A = 16 * (CHUNK * 2 + 16);
+    static constexpr int WBUF = WBUF_W > WBUF_A ? WBUF_W : WBUF_A;    // per-wave transposition buffer
+    static constexpr size_t LDS_BYTES = (size_t)WK * SB * MT16 * 1024 + (size_t)WK * WBUF;
+};
+
+// ---- masked fields of one k-step (8 fields of one lane) -> exact fp16 integers q - Z ----
+struct ZConst {
+    f16x2 off[4];   // per class: -(1024 * 2^-o + Z), both halves
+};
+
+template <int NBITS>
+__device__ __forceinline__ ZConst make_zconst(uint32_t zero) {
+    // -(B + Z) for B = 1024 * 2^-o is representable and its bit pattern is linear in Z:
+    // 0xE400 + Z, 0xDC00 + 4Z, 0xD400 + 16Z, 0xCC00 + 64Z for o = 0, 2, 4, 6
+    ZConst c;
+    using D = Decode<NBITS>;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int cls = k < D::NCLS ? k : 0;
+        const int o = (NBITS == 4) ? 4 * cls : (NBITS == 2 ? 2 * cls : 0);
+        const uint32_t base = 0xE400u - 0x0400u * (uint32_t)o;          // exponent drops by one per factor 2
+        const uint32_t h = base + (zero << o);
+        c.off[k] = as_f16x2(h * 0x00010001u);
+    }
+    return c;
+}
+
+template <int NBITS> struct IntStep;
+
+template <> struct IntStep<4> {
+    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const ZConst& c) {
+        uint32_t x[4];
+        Decode<4>::word(w[t], x);
+        const f16x2 sixteenth = f16x2{(_Float16)0.0625f, (_Float16)0.0625f};
+        const f16x2 v0 = as_f16x2(x[0]) + c.off[0];
+        const f16x2 v1 = __builtin_elementwise_fma(as_f16x2(x[1]), sixteenth, c.off[1]);
+        const f16x2 v2 = as_f16x2(x[2]) + c.off[0];
+        const f16x2 v3 = __builtin_elementwise_fma(as_f16x2(x[3]), sixteenth, c.off[1]);
+        return f16x8{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+    }
+};
+
+template <> struct IntStep<2> {
+    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const ZConst& c) {
+        const uint32_t word = (t & 1) ? (w[t >> 1] >> 8) : w[t >> 1];
+        f16x2 v[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t x = (word & (0x00030003u << (2 * p))) | kMagic;
+            const float inv = Decode<2>::inv_scale(p);
+            v[p] = __builtin_elementwise_fma(as_f16x2(x), f16x2{(_Float16)inv, (_Float16)inv}, c.off[p]);
+        }
+        return f16x8{v[0].x, v[0].y, v[1].x, v[1].y, v[2].x, v[2].y, v[3].x, v[3].y};
+    }
+};
+
+template <> struct IntStep<8> {
+    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const ZConst& c) {
+        uint32_t x[2], y[2];
+        Decode<8>::word(w[2 * t], x);
+        Decode<8>::word(w[2 * t + 1], y);
+        const f16x2 v0 = as_f16x2(x[0]) + c.off[0];
+        const f16x2 v1 = as_f16x2(x[1]) + c.off[0];
+        const f16x2 v2 = as_f16x2(y[0]) + c.off[0];
+        const f16x2 v3 = as_f16x2(y[1]) + c.off[0];
+        return f16x8{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+    }
+};
+
+template <class C>
+__global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
+    const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
+    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
+    constexpr int MT16 = C::MT16, WK = C::WK, CH = C::CH, SLOTS = C::SLOTS, PF = C::PF, SB = C::SB;
+    constexpr int EPL = C::EPL, KSTEPS = C::KSTEPS, CHUNK = C::CHUNK;
+    constexpr int P8 = 8 / C::NBITS;
+    constexpr uint32_t ZMASK = (1u << C::NBITS) - 1u;
+    constexpr bool DEFERRED = C::DEFERRED;
+    constexpr int LPR = C::LPR, RPI = C::RPI;            // lanes per row and rows per coalesced weight load
+    constexpr int GWN = C::GWN, ZB = C::ZB;              // scales / zero bytes per row in a wave's K-slice
+    constexpr int NSI = (16 * GWN + 63) / 64;            // load instructions for the scales of one tile
+    constexpr int NZI = (16 * ZB + 63) / 64;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    f32x4* red = reinterpret_cast<f32x4*>(smem);                                    // [WK][SB][MT16][64]
+    uint8_t* wbuf = smem + (size_t)WK * SB * MT16 * 1024 + (size_t)(threadIdx.x >> 6) * C::WBUF;   // private to the wave
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wk = tid >> 6;
+    const int r = lane & 15, kb = lane >> 4;
+    const int m0 = blockIdx.y * C::BM;
+    const int team_id = blockIdx.x;
+    constexpr int TEAM_STRIDE = C::GRID_X;
+
+    // chunks [lo, lo + CH) are read by this wave; it owns [own_from, own_from + CH) (a clamped last
+    // wave re-reads chunks of its neighbours with zeroed activations: every address stays in bounds)
+    const int own_from = wk * CH;
+    const int lo = min(own_from, C::NCHUNK - CH);
+    const int gw_lo = (lo * CHUNK) / C::GS;              // first group of the wave's K-slice
+
+    // ---- coalesced loads: LPR consecutive lanes cover one row's K-slice (CH*64 bytes) ----
+    struct WStage {
+        u32x4 w[CH];                 // load i: row i*RPI + lane/LPR, bytes (lane%LPR)*16 of the slice
+        uint32_t s[NSI];             // lane -> (row, group) = (idx / GWN, idx % GWN), idx = lane + 64*j
+        uint32_t z[NZI];             // lane -> (row, byte)  = (idx / ZB,  idx % ZB)
+    };
+    auto load_tile = [&](WStage& st, int tile) {
+        const int n_base = tile * 16;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int n = min(n_base + i * RPI + lane / LPR, C::N - 1);
+            const uint8_t* wp = W + (size_t)n * C::RB + (size_t)lo * 64 + (lane % LPR) * 16;
+            st.w[i] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)wp) : *(const u32x4*)wp;
+        }
+#pragma unroll
+        for (int j = 0; j < NSI; j++) {
+            const int idx = lane + 64 * j;
+            const int n = min(n_base + min(idx / GWN, 15), C::N - 1);
+            st.s[j] = S[(size_t)n * C::G + min(gw_lo + idx % GWN, C::G - 1)];
+        }
+        if constexpr (!C::SYM) {
+#pragma unroll
+            for (int j = 0; j < NZI; j++) {
+                const int idx = lane + 64 * j;
+                const int n = min(n_base + min(idx / ZB, 15), C::N - 1);
+                st.z[j] = Zp[(size_t)n * C::ZRB + min((gw_lo * C::NBITS) / 8 + idx % ZB, C::ZRB - 1)];
+            }
+        }
+    };
+
+    // ring of PF stages: tiles slot .. slot+PF-1 of this team are in flight
+    WStage ring[PF];
+#pragma unroll
+    for (int p = 0; p < PF - 1; p++)
+        if (p < SLOTS) load_tile(ring[p], min(team_id + p * TEAM_STRIDE, C::NT - 1));
+
+    // ---- resident activations, brought into MFMA fragment order through the wave's LDS buffer:
+    //      fragment (mt, c, t) = A[m0 + 16*mt + r][(lo+c)*CHUNK + kb*EPL + 8t .. +8] ----
+    f16x8 af[MT16][CH][KSTEPS];
+    {
+        constexpr int ROWB = CHUNK * 2;                  // bytes of one chunk of one activation row
+        constexpr int PITCH_A = ROWB + 16;
+        constexpr int LPRA = ROWB / 16;                  // lanes per row
+        constexpr int RPIA = 64 / LPRA;                  // rows per load (LPRA <= 64)
+#pragma unroll
+        for (int mt = 0; mt < MT16; mt++) {
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                const bool own = (lo + c >= own_from) && (lo + c < own_from + CH);
+#pragma unroll
+                for (int i = 0; i < 16 / RPIA; i++) {
+                    const int row = i * RPIA + lane / LPRA;
+                    const int m = m0 + 16 * mt + row;
+                    const uint16_t* ap = A + (size_t)min(m, m_total - 1) * C::K + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8;
+                    u32x4 v = *reinterpret_cast<const u32x4*>(ap);
+                    if (!(own && m < m_total)) v = u32x4{0, 0, 0, 0};
+                    *reinterpret_cast<u32x4*>(wbuf + row * PITCH_A + (lane % LPRA) * 16) = v;
+                }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int t = 0; t < KSTEPS; t++)
+                    af[mt][c][t] = *reinterpret_cast<const f16x8*>(wbuf + r * PITCH_A + kb * EPL * 2 + t * 16);
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+
+    const float* redf = reinterpret_cast<const float*>(smem);
+    static_assert(SB % PF == 0, "ring index must be static inside a batch");
+    constexpr int PITCH_W = CH * 64 + 16;
+#pragma unroll 1
+    for (int batch = 0; batch < C::NBATCH; batch++) {
+#pragma unroll
+        for (int sb = 0; sb < SB; sb++) {
+            const int slot = batch * SB + sb;
+            const int tile = team_id + slot * TEAM_STRIDE;
+            WStage& cur = ring[sb % PF];
+            // refill the stage consumed in the previous iteration with the tile PF-1 ahead
+            if (slot + PF - 1 < SLOTS)
+                load_tile(ring[(sb + PF - 1) % PF], min(tile + (PF - 1) * TEAM_STRIDE, C::NT - 1));
+            f32x4 acc[MT16];
+#pragma unroll
+            for (int mt = 0; mt < MT16; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (slot < SLOTS && tile < C::NT) {               // wave-uniform
+                // coalesced registers -> LDS -> fragment registers: lane (r, kb) takes the 16 bytes
+                // of row r at chunk c, k-block kb
+#pragma unroll
+                for (int i = 0; i < CH; i++)
+                    *reinterpret_cast<u32x4*>(wbuf + (i * RPI + lane / LPR) * PITCH_W + (lane % LPR) * 16) = cur.w[i];
+                __builtin_amdgcn_wave_barrier();
+                u32x4 wfrag[CH];
+#pragma unroll
+                for (int c = 0; c < CH; c++)
+                    wfrag[c] = *reinterpret_cast<const u32x4*>(wbuf + r * PITCH_W + c * 64 + kb * 16);
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int c = 0; c < CH; c++) {
+                    const int g = ((lo + c) * CHUNK + kb * EPL) / C::GS;     // group of this lane's fields
+                    // scale and zero-point of (row r, group g) sit in lane/register (idx % 64, idx / 64)
+                    const int sidx = r * GWN + (g - gw_lo);
+                    uint32_t sraw = 0;
+#pragma unroll
+                    for (int j = 0; j < NSI; j++) {
+                        const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((sidx & 63) << 2, (int)cur.s[j]);
+                        sraw = (NSI == 1 || (sidx >> 6) == j) ? v : sraw;
+                    }
+                    uint32_t zero = 1u << (C::NBITS - 1);
+                    if constexpr (!C::SYM) {
+                        const int zbyte = (g * C::NBITS) / 8 - (gw_lo * C::NBITS) / 8;
+                        const int zidx = r * ZB + zbyte;
+                        uint32_t zraw = 0;
+#pragma unroll
+                        for (int j = 0; j < NZI; j++) {
+                            const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((zidx & 63) << 2, (int)cur.z[j]);
+                            zraw = (NZI == 1 || (zidx >> 6) == j) ? v : zraw;
+                        }
+                        zero = (zraw >> ((g % P8) * C::NBITS)) & ZMASK;
+                    }
+                    const ZConst zc = make_zconst<C::NBITS>(zero);
+                    const uint32_t w4[4] = {wfrag[c].x, wfrag[c].y, wfrag[c].z, wfrag[c].w};
+                    if constexpr (DEFERRED) {
+                        // the whole chunk lies in one group: integer sum on the matrix core, one fp32 scale
+                        f32x4 gsum[MT16];
+#pragma unroll
+                        for (int t = 0; t < KSTEPS; t++) {
+                            const f16x8 wf = IntStep<C::NBITS>::run(w4, t, zc);
+#pragma unroll
+                            for (int mt = 0; mt < MT16; mt++)
+                                gsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                    af[mt][c][t], wf, t == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : gsum[mt], 0, 0, 0);
+                        }
+                        const float sc = f16_bits_to_f32((uint16_t)sraw);
+#pragma unroll
+                        for (int mt = 0; mt < MT16; mt++)
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[mt][e] = __builtin_fmaf(sc, gsum[mt][e], acc[mt][e]);
+                    } else {
+                        // a chunk spans several groups (the four lanes of a row may sit in different
+                        // ones): scale every element before the contraction
+                        const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)sraw);
+                        const f16x8 s8 = f16x8{sh, sh, sh, sh, sh, sh, sh, sh};
+#pragma unroll
+                        for (int t = 0; t < KSTEPS; t++) {
+                            const f16x8 wf = IntStep<C::NBITS>::run(w4, t, zc) * s8;
+#pragma unroll
+                            for (int mt = 0; mt < MT16; mt++)
+                                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][c][t], wf, acc[mt], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT16; mt++)
+                red[(((size_t)wk * SB + sb) * MT16 + mt) * 64 + lane] = acc[mt];
+        }
+
+        __syncthreads();
+
+        // ---- sum the WK partial tiles of this batch and store.  A partial tile sits in LDS as
+        //      [lane = n + 16*(m/4)][e = m%4]; the storing lane takes (m = lane/4, n = 4*(lane%4) .. +3):
+        //      one 8-byte store per lane. ----
+        for (int p = wk; p < SB * MT16; p += WK) {
+            const int sb = p / MT16, mt = p % MT16;
+            const int slot = batch * SB + sb;
+            const int tile = team_id + slot * TEAM_STRIDE;
+            if (slot >= SLOTS || tile >= C::NT) continue;
+            const int ml = lane >> 2, nq = (lane & 3) * 4;
+            float total[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int k2 = 0; k2 < WK; k2++) {
+                const float* base = redf + ((((size_t)k2 * SB + sb) * MT16 + mt) * 64) * 4;
+#pragma unroll
+                for (int j = 0; j < 4; j++) total[j] += base[((nq + j) + 16 * (ml >> 2)) * 4 + (ml & 3)];
+            }
+            const int m = m0 + 16 * mt + ml;
+            const int n = tile * 16 + nq;
+            if (m < m_total) {
+                uint16_t h[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) h[e] = f32_to_f16_bits(total[e]);
+                uint16_t* dst = Cout + (size_t)m * C::N + n;
+                if constexpr (C::N % 4 == 0) {
+                    if (n < C::N) *reinterpret_cast<u32x2*>(dst) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < C::N) dst[e] = h[e];
+                }
+            }
+        }
+        if (batch + 1 < C::NBATCH) __syncthreads();           // LDS slots are reused by the next batch
+    }
+}
+
+template <class C>
+int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m, hipStream_t stream) {
+    const char* why = nullptr;
+    if (C::NBITS != 2 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 4 or 8 for this kernel";
+    else if (C::K % C::CHUNK != 0) why = "K must be a multiple of 4*128/NBITS";
+    else if (C::GS <= 0 || C::K % C::GS != 0) why = "GS must divide K";
+    else if (C::GS % C::EPL != 0) why = "a lane's 16 bytes of fields must lie inside one group";
+    else if (!C::SYM && (C::G % (8 / C::NBITS)) != 0) why = "K/GS must fill whole zero-point bytes";
+    else if (C::CH > C::NCHUNK) why = "more chunks per wave than the row has";
+    else if (C::WK * C::CH < C::NCHUNK) why = "WK*CH must cover K";
+    else if ((C::WK - 1) * C::CH >= C::NCHUNK) why = "a wave would own no chunk";
+    else if (C::THREADS > 1024) why = "block too large";
+    else if (C::CH != 1 && C::CH != 2 && C::CH != 4 && C::CH != 8 && C::CH != 16) why = "CH must be 1, 2, 4, 8 or 16";
+    else if (C::GS % C::CHUNK != 0 && C::CHUNK % C::GS != 0) why = "GS must divide the chunk or be a multiple of it";
+    else if (C::PF != 1 && C::PF != 2 && C::PF != 4) why = "PF must be 1, 2 or 4";
+    else if (C::LDS_BYTES > 160 * 1024) why = "partial tiles exceed the 160 KB of LDS";
+    if (why) {
+        fprintf(stderr, "qfactory mgemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT16=%d WK=%d CH=%d PB=%d PF=%d)\n",
+                why, C::NBITS, C::GS, C::N, C::K, C::MT16, C::WK, C::CH, C::PB, C::PF);
+        return 1;
+    }
+    if (m <= 0) return 0;
+    static bool attr_set = false;
+    if (!attr_set && C::LDS_BYTES > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mgemv_kernel<C>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES);
+        if (e != hipSuccess) {
+            fprintf(stderr, "qfactory mgemv: cannot reserve %zu bytes of LDS: %s\n", C::LDS_BYTES, hipGetErrorString(e));
+            return 2;
+        }
+        attr_set = true;
+    }
+    dim3 grid(C::GRID_X, (m + C::BM - 1) / C::BM);
+    hipLaunchKernelGGL(mgemv_kernel<C>, grid, dim3(C::THREADS), C::LDS_BYTES, stream, (const uint16_t*)A,
+                       (const uint8_t*)W, (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        fprintf(stderr, "qfactory mgemv: launch failed: %s\n", hipGetErrorString(err));
+        return 2;
+    }
+    return 0;
+}
+
+}  // namespace qf

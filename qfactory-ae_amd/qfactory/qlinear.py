@@ -20,7 +20,7 @@ from .core import tiling
 
 def _m_bucket(m):
     """Row count a specialisation is compiled for when ``m`` rows arrive."""
-    if m <= tiling.GEMV_MAX_M:
+    if m < tiling.MGEMV_MIN_M:
         return m
     if m <= 16:
         return 16
