@@ -105,6 +105,8 @@ class QMatmulQFunc(QFunc):
             return tiling.gemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "mgemv":
             return tiling.mgemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
+        if regime == "gemm":
+            return tiling.gemm_tiling(p["M"], p["N"], p["K"], nbits, gs)
         return tiling.mfma_tiling(p["M"], p["N"], p["K"], nbits, gs)
 
     def arg_name_type(self):
@@ -129,6 +131,8 @@ class QMatmulQFunc(QFunc):
             cands = tiling.gemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         elif self.regime == "mgemv":
             cands = tiling.mgemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
+        elif self.regime == "gemm":
+            cands = tiling.gemm_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         else:
             cands = tiling.mfma_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         return [self.clone(tiling_configs=c) for c in cands]
@@ -150,6 +154,10 @@ class QMatmulQFunc(QFunc):
             code += '#include "qf_mgemv.hip.h"\n'
             cfg = tiling.mgemv_cfg_string(p, t, not self.l2cache_b)
             call = "qf::mgemv_launch<Cfg>"
+        elif self.regime == "gemm":
+            code += '#include "qf_gemm.hip.h"\n'
+            cfg = tiling.gemm_cfg_string(p, t, not self.l2cache_b)
+            call = "qf::gemm_launch<Cfg>"
         elif self.regime == "mfma":
             code += '#include "qf_mfma.hip.h"\n'
             cfg = tiling.mfma_cfg_string(p, t, self.decode_strategy, not self.l2cache_b)

@@ -31,6 +31,8 @@ def regime_for(M, K=None, nbits=None, group_size=None):
         return "mgemv"
     if M <= GEMV_MAX_M:
         return "gemv"
+    if M > MGEMV_MAX_M and gemm_supported(K, nbits, group_size):
+        return "gemm"
     return "mfma"
 
 
@@ -273,3 +275,75 @@ def mgemv_cfg_string(problem, t, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::MGemvCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
             f"{t['MT16']}, {t['WK']}, {t['CH']}, {t['PB']}, {t['PF']}, {b(nt_b)}>")
+
+
+# --------------------------------------------------------------------------------------------
+# Large-M GEMM regime (LDS-staged operands, 32x32x16 MFMA, optional split-K over blocks)
+# --------------------------------------------------------------------------------------------
+GEMM_BK = 64
+
+
+def gemm_supported(K, nbits, group_size):
+    if nbits not in (2, 4, 8):
+        return False
+    epl = 128 // nbits
+    return K % GEMM_BK == 0 and GEMM_BK % epl == 0 and group_size % epl == 0
+
+
+def _split_k(tiles, K, bk, target_blocks=NUM_CUS, max_ks=8, min_iters=8):
+    best = 1
+    for ks in range(1, max_ks + 1):
+        if K % (ks * bk) or K // (ks * bk) < min_iters:
+            continue
+        best = ks
+        if tiles * ks >= target_blocks:
+            break
+    return best
+
+
+def gemm_tiling(M, N, K, nbits, group_size, **pins):
+    bm = 256 if M > 128 else (128 if M > 64 else 64)
+    bn = 128
+    wm, wn = (2, 2) if bm >= 128 else (1, 4)
+    tiles = -(-N // bn) * -(-M // bm)
+    # split-K over blocks costs a fenced round trip through memory (tens of microseconds on
+    # MI355X): only worth it when the tiles alone would leave most of the machine idle
+    ks = _split_k(tiles, K, GEMM_BK) if tiles < NUM_CUS // 8 else 1
+    cfg = {"BM": bm, "BN": bn, "BK": GEMM_BK, "WM": wm, "WN": wn, "KS": ks, "PA": 2, "PW": 8}
+    cfg.update(pins)
+    return cfg
+
+
+def gemm_candidates(M, N, K, nbits, group_size):
+    seen, out = set(), []
+
+    def add(cfg):
+        key = tuple(sorted(cfg.items()))
+        tm, tn = cfg["BM"] // cfg["WM"], cfg["BN"] // cfg["WN"]
+        lds = 2 * (cfg["BM"] + cfg["BN"]) * (cfg["BK"] + 8) * 2
+        ok = (tm % 32 == 0 and tn % 32 == 0 and (tm // 32) * (tn // 32) * 16 <= 256 and lds <= 160 * 1024
+              and K % (cfg["KS"] * cfg["BK"]) == 0 and cfg["BK"] % (128 // nbits) == 0
+              and 64 * cfg["WM"] * cfg["WN"] <= 1024
+              and (cfg["BN"] * cfg["BK"] // (128 // nbits)) % (64 * cfg["WM"] * cfg["WN"]) == 0
+              and (cfg["BM"] * cfg["BK"] // 8) % (64 * cfg["WM"] * cfg["WN"]) == 0)
+        if ok and key not in seen:
+            seen.add(key)
+            out.append(cfg)
+
+    add(gemm_tiling(M, N, K, nbits, group_size))
+    for bm in (64, 128, 256):
+        if bm >= 2 * M and bm > 64:
+            continue
+        for bn in (64, 128, 256):
+            for wm, wn in ((1, 4), (2, 2), (4, 1), (2, 4), (4, 2)):
+                for bk in (32, 64):
+                    for ks in (1, 2, 4):
+                        for pa, pw in ((2, 4), (2, 8), (4, 8)):
+                            add({"BM": bm, "BN": bn, "BK": bk, "WM": wm, "WN": wn, "KS": ks, "PA": pa, "PW": pw})
+    return out
+
+
+def gemm_cfg_string(problem, t, nt_b):
+    b = lambda x: "true" if x else "false"
+    return (f"qf::GemmCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
+            f"{t['BM']}, {t['BN']}, {t['BK']}, {t['WM']}, {t['WN']}, {t['KS']}, {t['PA']}, {t['PW']}, {b(nt_b)}>")

@@ -25,7 +25,7 @@
 #pragma once
 
 #include <cstdio>
-#include "qf_common.hip.h"
+#include "qf_dequant.hip.h"
 
 namespace qf {
 
@@ -54,81 +54,6 @@ struct MfmaCfg {
     static constexpr int GRID_X = (N + BN - 1) / BN;
     static constexpr size_t LDS_BYTES = (size_t)2 * WK * BM * PITCH * 2 +
                                         (WK > 1 ? (size_t)(WK - 1) * WM * WN * AT * BT * 256 * 4 : 0);
-};
-
-// ---- dequantise one k-step (8 fields of one lane) to fp16: returns fp16_rn((q - Z) * s) ----
-template <int NBITS> struct DequantStep;
-
-// constants per (lane, n-tile, group): packed scale, and the packed offsets that turn the masked
-// magic-number encodings into q - Z exactly
-struct QConst {
-    f16x2 s2;       // (s, s)
-    f16x2 off[4];   // per class: -(1024 * 2^-o + Z)
-};
-
-__device__ __forceinline__ f16x2 splat(float v) {
-    const _Float16 h = (_Float16)v;
-    return f16x2{h, h};
-}
-
-template <int NBITS>
-__device__ __forceinline__ QConst make_qconst(uint16_t s_bits, int zero) {
-    QConst c;
-    const _Float16 s = __builtin_bit_cast(_Float16, s_bits);
-    c.s2 = f16x2{s, s};
-    using D = Decode<NBITS>;
-#pragma unroll
-    for (int k = 0; k < 4; k++)
-        c.off[k] = splat(-(1024.0f * D::inv_scale(k < D::NCLS ? k : 0) + (float)zero));   // exact: integers below 2048
-    return c;
-}
-
-__device__ __forceinline__ f16x2 pk_fma(f16x2 a, f16x2 b, f16x2 c) {
-    return __builtin_elementwise_fma(a, b, c);
-}
-
-template <> struct DequantStep<4> {
-    // word t of the lane's four words holds the 8 fields of k-step t
-    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const QConst& c) {
-        uint32_t x[4];
-        Decode<4>::word(w[t], x);
-        const f16x2 sixteenth = f16x2{(_Float16)0.0625f, (_Float16)0.0625f};
-        f16x2 v0 = as_f16x2(x[0]) + c.off[0];
-        f16x2 v1 = pk_fma(as_f16x2(x[1]), sixteenth, c.off[1]);
-        f16x2 v2 = as_f16x2(x[2]) + c.off[0];
-        f16x2 v3 = pk_fma(as_f16x2(x[3]), sixteenth, c.off[1]);
-        v0 *= c.s2; v1 *= c.s2; v2 *= c.s2; v3 *= c.s2;
-        return f16x8{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
-    }
-};
-
-template <> struct DequantStep<2> {
-    // a word holds 16 fields = two k-steps: pairs 0..3 then pairs 4..7
-    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const QConst& c) {
-        const uint32_t word = (t & 1) ? (w[t >> 1] >> 8) : w[t >> 1];
-        f16x2 v[4];
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const uint32_t x = (word & (0x00030003u << (2 * p))) | kMagic;
-            const float inv = Decode<2>::inv_scale(p);
-            v[p] = pk_fma(as_f16x2(x), f16x2{(_Float16)inv, (_Float16)inv}, c.off[p]) * c.s2;
-        }
-        return f16x8{v[0].x, v[0].y, v[1].x, v[1].y, v[2].x, v[2].y, v[3].x, v[3].y};
-    }
-};
-
-template <> struct DequantStep<8> {
-    // a k-step is two words of four byte fields
-    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const QConst& c) {
-        uint32_t x[2], y[2];
-        Decode<8>::word(w[2 * t], x);
-        Decode<8>::word(w[2 * t + 1], y);
-        const f16x2 v0 = (as_f16x2(x[0]) + c.off[0]) * c.s2;
-        const f16x2 v1 = (as_f16x2(x[1]) + c.off[0]) * c.s2;
-        const f16x2 v2 = (as_f16x2(y[0]) + c.off[0]) * c.s2;
-        const f16x2 v3 = (as_f16x2(y[1]) + c.off[0]) * c.s2;
-        return f16x8{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
-    }
 };
 
 template <class C>
@@ -236,8 +161,8 @@ __global__ __launch_bounds__(C::THREADS) void mfma_kernel(
             const int g = (it * BK + kb * EPL) / C::GS;
 #pragma unroll
             for (int j = 0; j < BT; j++) {
-                const int zero = C::SYM ? (1 << (C::NBITS - 1))
-                                        : (int)((wcur.z[j] >> ((g % P8) * C::NBITS)) & ZMASK);
+                const uint32_t zero = C::SYM ? (1u << (C::NBITS - 1))
+                                             : ((uint32_t)(wcur.z[j] >> ((g % P8) * C::NBITS)) & ZMASK);
                 qc[j] = make_qconst<C::NBITS>((uint16_t)wcur.s[j], zero);
             }
             const uint16_t* abase = As + ((size_t)(buf * WK + wk) * C::BM + wm * AT * 16 + r) * PITCH + kb * EPL;

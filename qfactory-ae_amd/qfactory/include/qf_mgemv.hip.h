@@ -22,7 +22,7 @@
 #pragma once
 
 #include <cstdio>
-#include "qf_common.hip.h"
+#include "qf_dequant.hip.h"
 
 namespace qf {
 
@@ -60,70 +60,6 @@ struct MGemvCfg {
     static constexpr int WBUF_A = 16 * (CHUNK * 2 + 16);
     static constexpr int WBUF = WBUF_W > WBUF_A ? WBUF_W : WBUF_A;    // per-wave transposition buffer
     static constexpr size_t LDS_BYTES = (size_t)WK * SB * MT16 * 1024 + (size_t)WK * WBUF;
-};
-
-// ---- masked fields of one k-step (8 fields of one lane) -> exact fp16 integers q - Z ----
-struct ZConst {
-    f16x2 off[4];   // per class: -(1024 * 2^-o + Z), both halves
-};
-
-template <int NBITS>
-__device__ __forceinline__ ZConst make_zconst(uint32_t zero) {
-    // -(B + Z) for B = 1024 * 2^-o is representable and its bit pattern is linear in Z:
-    // 0xE400 + Z, 0xDC00 + 4Z, 0xD400 + 16Z, 0xCC00 + 64Z for o = 0, 2, 4, 6
-    ZConst c;
-    using D = Decode<NBITS>;
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const int cls = k < D::NCLS ? k : 0;
-        const int o = (NBITS == 4) ? 4 * cls : (NBITS == 2 ? 2 * cls : 0);
-        const uint32_t base = 0xE400u - 0x0400u * (uint32_t)o;          // exponent drops by one per factor 2
-        const uint32_t h = base + (zero << o);
-        c.off[k] = as_f16x2(h * 0x00010001u);
-    }
-    return c;
-}
-
-template <int NBITS> struct IntStep;
-
-template <> struct IntStep<4> {
-    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const ZConst& c) {
-        uint32_t x[4];
-        Decode<4>::word(w[t], x);
-        const f16x2 sixteenth = f16x2{(_Float16)0.0625f, (_Float16)0.0625f};
-        const f16x2 v0 = as_f16x2(x[0]) + c.off[0];
-        const f16x2 v1 = __builtin_elementwise_fma(as_f16x2(x[1]), sixteenth, c.off[1]);
-        const f16x2 v2 = as_f16x2(x[2]) + c.off[0];
-        const f16x2 v3 = __builtin_elementwise_fma(as_f16x2(x[3]), sixteenth, c.off[1]);
-        return f16x8{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
-    }
-};
-
-template <> struct IntStep<2> {
-    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const ZConst& c) {
-        const uint32_t word = (t & 1) ? (w[t >> 1] >> 8) : w[t >> 1];
-        f16x2 v[4];
-#pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const uint32_t x = (word & (0x00030003u << (2 * p))) | kMagic;
-            const float inv = Decode<2>::inv_scale(p);
-            v[p] = __builtin_elementwise_fma(as_f16x2(x), f16x2{(_Float16)inv, (_Float16)inv}, c.off[p]);
-        }
-        return f16x8{v[0].x, v[0].y, v[1].x, v[1].y, v[2].x, v[2].y, v[3].x, v[3].y};
-    }
-};
-
-template <> struct IntStep<8> {
-    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], int t, const ZConst& c) {
-        uint32_t x[2], y[2];
-        Decode<8>::word(w[2 * t], x);
-        Decode<8>::word(w[2 * t + 1], y);
-        const f16x2 v0 = as_f16x2(x[0]) + c.off[0];
-        const f16x2 v1 = as_f16x2(x[1]) + c.off[0];
-        const f16x2 v2 = as_f16x2(y[0]) + c.off[0];
-        const f16x2 v3 = as_f16x2(y[1]) + c.off[0];
-        return f16x8{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
-    }
 };
 
 template <class C>

@@ -73,7 +73,16 @@ class GPTQLinear(torch.nn.Module):
     def _compile(self, m, compile_flags):
         matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
                          torch.float16, torch.int8, self.group_size, base_impl=self.base_impl)
-        return matmul.compile_profile(**compile_flags)
+        func = matmul.compile_profile(**compile_flags)
+        # One launch now: a specialisation may allocate scratch on its first call (split-K
+        # partial tiles), which must not happen later inside a HIP-graph capture.
+        if self.w.is_cuda:
+            x = torch.zeros(m, self.in_features, dtype=torch.float16, device=self.w.device)
+            out = torch.empty(m, self.out_features, dtype=torch.float16, device=self.w.device)
+            rc = func(x, self.w, out, self.s, self.z) if self.z is not None else func(x, self.w, out, self.s)
+            if rc != 0:
+                raise RuntimeError(f"quantized linear launch failed with return code {rc}")
+        return func
 
     def func_for(self, m):
         bucket = _m_bucket(m)
