@@ -283,17 +283,44 @@ def mgemv_cfg_string(problem, t, nt_b):
 GEMM_BK = 64
 
 
-def gemm_supported(K, nbits, group_size):
+def gemm_valid(cfg, K, nbits, group_size):
+    """Mirror of the static checks in gemm_launch (qf_gemm.hip.h)."""
     if nbits not in (2, 4, 8):
         return False
     epl = 128 // nbits
-    return K % GEMM_BK == 0 and GEMM_BK % epl == 0 and group_size % epl == 0
+    supk = 1024 // nbits
+    bm, bn, bk, wm, wn, ks, pa = (cfg[k] for k in ("BM", "BN", "BK", "WM", "WN", "KS", "PA"))
+    threads = 64 * wm * wn
+    tm, tn = bm // wm, bn // wn
+    if bm % (32 * wm) or bn % (32 * wn) or threads > 1024 or (tm // 32) * (tn // 32) * 16 > 256:
+        return False
+    if bk % 16 or bk % epl or K % (ks * bk) or K % group_size or group_size % epl:
+        return False
+    if supk % bk or supk // bk < 2 or pa < 2 or (2 * supk // bk) % pa:
+        return False
+    if (group_size < supk and supk % group_size) or (group_size > supk and group_size % supk):
+        return False
+    if ks > 1 and (K // ks) % min(group_size, supk):
+        return False
+    rb = K * nbits // 8
+    if rb % 16 or rb < 128 or (bn * 8) % threads:
+        return False
+    if (bn * bk // epl) % threads or (bm * bk // 8) % threads:
+        return False
+    ngs = max(1, supk // group_size)
+    lds = 2 * (bm + bn) * (bk + 8) * 2 + 2 * bn * 144 + 2 * bn * ngs * 3 + 16
+    return lds <= 160 * 1024
 
 
-def _split_k(tiles, K, bk, target_blocks=NUM_CUS, max_ks=8, min_iters=8):
+def gemm_supported(K, nbits, group_size):
+    probe = {"BM": 128, "BN": 128, "BK": GEMM_BK, "WM": 2, "WN": 2, "KS": 1, "PA": 2}
+    return gemm_valid(probe, K, nbits, group_size)
+
+
+def _split_k(tiles, K, bk, align, target_blocks=NUM_CUS, max_ks=8, min_iters=8):
     best = 1
     for ks in range(1, max_ks + 1):
-        if K % (ks * bk) or K // (ks * bk) < min_iters:
+        if K % (ks * bk) or K // (ks * bk) < min_iters or (K // ks) % align:
             continue
         best = ks
         if tiles * ks >= target_blocks:
@@ -308,8 +335,8 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     tiles = -(-N // bn) * -(-M // bm)
     # split-K over blocks costs a fenced round trip through memory (tens of microseconds on
     # MI355X): only worth it when the tiles alone would leave most of the machine idle
-    ks = _split_k(tiles, K, GEMM_BK) if tiles < NUM_CUS // 8 else 1
-    cfg = {"BM": bm, "BN": bn, "BK": GEMM_BK, "WM": wm, "WN": wn, "KS": ks, "PA": 2, "PW": 8}
+    ks = _split_k(tiles, K, GEMM_BK, min(group_size, 1024 // nbits)) if tiles < NUM_CUS // 8 else 1
+    cfg = {"BM": bm, "BN": bn, "BK": GEMM_BK, "WM": wm, "WN": wn, "KS": ks, "PA": 2}
     cfg.update(pins)
     return cfg
 
@@ -319,14 +346,7 @@ def gemm_candidates(M, N, K, nbits, group_size):
 
     def add(cfg):
         key = tuple(sorted(cfg.items()))
-        tm, tn = cfg["BM"] // cfg["WM"], cfg["BN"] // cfg["WN"]
-        lds = 2 * (cfg["BM"] + cfg["BN"]) * (cfg["BK"] + 8) * 2
-        ok = (tm % 32 == 0 and tn % 32 == 0 and (tm // 32) * (tn // 32) * 16 <= 256 and lds <= 160 * 1024
-              and K % (cfg["KS"] * cfg["BK"]) == 0 and cfg["BK"] % (128 // nbits) == 0
-              and 64 * cfg["WM"] * cfg["WN"] <= 1024
-              and (cfg["BN"] * cfg["BK"] // (128 // nbits)) % (64 * cfg["WM"] * cfg["WN"]) == 0
-              and (cfg["BM"] * cfg["BK"] // 8) % (64 * cfg["WM"] * cfg["WN"]) == 0)
-        if ok and key not in seen:
+        if key not in seen and gemm_valid(cfg, K, nbits, group_size):
             seen.add(key)
             out.append(cfg)
 
@@ -338,12 +358,12 @@ def gemm_candidates(M, N, K, nbits, group_size):
             for wm, wn in ((1, 4), (2, 2), (4, 1), (2, 4), (4, 2)):
                 for bk in (32, 64):
                     for ks in (1, 2, 4):
-                        for pa, pw in ((2, 4), (2, 8), (4, 8)):
-                            add({"BM": bm, "BN": bn, "BK": bk, "WM": wm, "WN": wn, "KS": ks, "PA": pa, "PW": pw})
+                        for pa in (2, 4):
+                            add({"BM": bm, "BN": bn, "BK": bk, "WM": wm, "WN": wn, "KS": ks, "PA": pa})
     return out
 
 
 def gemm_cfg_string(problem, t, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::GemmCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
-            f"{t['BM']}, {t['BN']}, {t['BK']}, {t['WM']}, {t['WN']}, {t['KS']}, {t['PA']}, {t['PW']}, {b(nt_b)}>")
+            f"{t['BM']}, {t['BN']}, {t['BK']}, {t['WM']}, {t['WN']}, {t['KS']}, {t['PA']}, {b(nt_b)}>")
