@@ -53,7 +53,6 @@ __global__ __launch_bounds__(256) void pack_plane_kernel(const int32_t* __restri
     const int64_t n = (int64_t)blockIdx.x * 32 + (threadIdx.x & 31);
     const int64_t wi = (int64_t)blockIdx.y * 8 + (threadIdx.x >> 5);
     if (n >= N || wi >= K / P) return;
-    // stage through LDS so that the row-major writes are coalesced along the word index
     out[n * row_words + word_offset + wi] = build_word<B>(weight, N, n, wi * P, shift, mask);
 }
 

@@ -3,8 +3,8 @@
 Drop-in for the reference's ``qfactory/convert.py`` (``convert_params`` at convert.py:84-97): the
 same entry point, argument dictionaries, validation and -- bit for bit -- the same packed tensors
 for 2/4/8-bit weights.  The reference builds the layout with Python loops over K (convert.py:58-66,
-77-79); here every step is a whole-tensor integer operation, so the routine runs unchanged on CPU
-or GPU tensors and stays usable on 70B-sized layers.
+77-79); here every step is a whole-tensor integer operation (CPU tensors) or one HIP kernel of
+libqfactory_hip.so (device tensors), so the routine stays usable on 70B-sized layers.
 
 Layout produced (reference file:line in brackets):
 
@@ -107,7 +107,17 @@ def _pack_fields(fields_nk, nbits):
     return words.contiguous().view(torch.int8)             # little-endian bytes of every word
 
 
+def _on_device(t):
+    """Device tensors whose K fills whole 32-element words take the HIP packers of
+    libqfactory_hip.so (one pass over the tensor); everything else the whole-tensor torch ops below,
+    on whatever device the tensor lives.  Both produce identical bytes."""
+    return t.is_cuda
+
+
 def _transform_weight_basic(K, N, weight, nbits):
+    if _on_device(weight) and K % 32 == 0:
+        from . import native
+        return native.pack_weight(weight.contiguous(), nbits)
     wt = weight.T
     if nbits == 3:
         lo = _pack_fields(wt & 3, 2)
@@ -117,6 +127,9 @@ def _transform_weight_basic(K, N, weight, nbits):
 
 
 def _transform_scale(K, N, GS, scale):
+    if _on_device(scale):
+        from . import native
+        return native.transpose_scale(scale.contiguous())
     return scale.T.contiguous()
 
 
@@ -125,6 +138,9 @@ def _transform_zero(K, N, GS, zero, nbits):
     pack_factor = 8 // fb
     G = zero.shape[0]
     assert G % pack_factor == 0, f"K/GS ({G}) must fill whole bytes of {pack_factor} zero-points"
+    if _on_device(zero):
+        from . import native
+        return native.pack_zero(zero.contiguous(), nbits)
     zp = (zero + 1).clamp(max=(2 ** nbits - 1)).T.to(torch.int64)           # (N, G)
     shifts = torch.arange(pack_factor, device=zero.device, dtype=torch.int64) * fb
     packed = (zp.reshape(zp.shape[0], G // pack_factor, pack_factor) << shifts).sum(dim=2)

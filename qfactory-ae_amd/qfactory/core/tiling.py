@@ -329,8 +329,14 @@ def _split_k(tiles, K, bk, align, target_blocks=NUM_CUS, max_ks=8, min_iters=8):
 
 
 def gemm_tiling(M, N, K, nbits, group_size, **pins):
-    bm = 256 if M > 128 else (128 if M > 64 else 64)
     bn = 128
+    # the largest block tile that still gives every CU a block: at M = 256 and N = 8192 a 256- or
+    # 128-row tile would leave half of the 256 CUs idle
+    bm = 64
+    for cand in (256, 128):
+        if M > cand // 2 and -(-N // bn) * -(-M // cand) >= NUM_CUS:
+            bm = cand
+            break
     wm, wn = (2, 2) if bm >= 128 else (1, 4)
     tiles = -(-N // bn) * -(-M // bm)
     # split-K over blocks costs a fenced round trip through memory (tens of microseconds on

@@ -1,0 +1,113 @@
+"""ctypes binding of libqfactory_hip.so, the ahead-of-time HIP library (device-side repacking and
+the stream read / copy calibration kernels).  Its C ABI is declared in include/qfactory_hip.h.
+
+The library is built in-tree with hipcc (``build()``; no GPU needed) and loaded lazily.  There is
+no substitute path: calling an entry point without the built library raises.
+"""
+import ctypes
+import os
+import subprocess
+import threading
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.join(os.path.dirname(PKG_DIR), "csrc")
+REPO_INCLUDE = os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include")
+SOURCE = os.path.join(CSRC_DIR, "qfactory_hip.hip")
+LIBRARY = os.path.join(CSRC_DIR, "libqfactory_hip.so")
+
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-std=c++20", "-shared", "-fPIC", "-O3",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+# name -> (restype, argtypes); mirrors include/qfactory_hip.h
+_P, _I64, _INT, _SZ = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+SIGNATURES = {
+    "qf_version": (_INT, []),
+    "qf_pack_weight": (_INT, [_P, _P, _I64, _I64, _INT, _P]),
+    "qf_pack_zero": (_INT, [_P, _P, _I64, _I64, _INT, _P]),
+    "qf_transpose_scale": (_INT, [_P, _P, _I64, _I64, _P]),
+    "qf_stream_read": (_INT, [_P, _SZ, _P, _P]),
+    "qf_stream_copy": (_INT, [_P, _P, _SZ, _P]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+def build(force=False):
+    """Compile csrc/qfactory_hip.hip for gfx950 into csrc/libqfactory_hip.so."""
+    hipcc = os.environ.get("QFACTORY_HIPCC", "/opt/rocm/bin/hipcc")
+    if not force and os.path.exists(LIBRARY) and os.path.getmtime(LIBRARY) >= os.path.getmtime(SOURCE):
+        return LIBRARY
+    tmp = f"{LIBRARY}.tmp.{os.getpid()}"
+    cmd = [hipcc, "-x", "hip", SOURCE, "-o", tmp, *HIPCC_FLAGS, f"-I{REPO_INCLUDE}"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {SOURCE}:\n{proc.stderr}")
+    os.replace(tmp, LIBRARY)
+    return LIBRARY
+
+
+def load():
+    """The loaded library with argument types set; raises if it has not been built."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIBRARY):
+                raise RuntimeError(f"{LIBRARY} is missing: build it with qfactory.native.build() "
+                                   "(hipcc, no GPU needed); there is no CPU substitute for the device packers")
+            lib = ctypes.CDLL(LIBRARY)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype, fn.argtypes = res, args
+            _lib = lib
+    return _lib
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed with return code {rc}")
+
+
+def pack_weight(weight, nbits):
+    """(K, N) int32 device tensor -> (N, K*nbits/8) int8, bit-identical to convert._transform_weight_basic."""
+    import torch
+    assert weight.is_cuda and weight.dtype == torch.int32 and weight.is_contiguous() and weight.dim() == 2
+    K, N = weight.shape
+    out = torch.empty(N, K * nbits // 8, dtype=torch.int8, device=weight.device)
+    _check(load().qf_pack_weight(weight.data_ptr(), out.data_ptr(), K, N, nbits, _stream()), "qf_pack_weight")
+    return out
+
+
+def pack_zero(zero, nbits):
+    """(G, N) int32 device tensor -> (N, G*fb/8) int8 holding min(zero + 1, 2^nbits - 1)."""
+    import torch
+    assert zero.is_cuda and zero.dtype == torch.int32 and zero.is_contiguous() and zero.dim() == 2
+    G, N = zero.shape
+    fb = 4 if nbits == 3 else nbits
+    out = torch.empty(N, G * fb // 8, dtype=torch.int8, device=zero.device)
+    _check(load().qf_pack_zero(zero.data_ptr(), out.data_ptr(), G, N, nbits, _stream()), "qf_pack_zero")
+    return out
+
+
+def transpose_scale(scale):
+    """(G, N) fp16 device tensor -> (N, G) fp16 contiguous."""
+    import torch
+    assert scale.is_cuda and scale.dtype == torch.float16 and scale.is_contiguous() and scale.dim() == 2
+    G, N = scale.shape
+    out = torch.empty(N, G, dtype=torch.float16, device=scale.device)
+    _check(load().qf_transpose_scale(scale.data_ptr(), out.data_ptr(), G, N, _stream()), "qf_transpose_scale")
+    return out
+
+
+def stream_read(src, sink):
+    _check(load().qf_stream_read(src.data_ptr(), src.numel() * src.element_size(), sink.data_ptr(), _stream()), "qf_stream_read")
+
+
+def stream_copy(dst, src):
+    assert dst.numel() * dst.element_size() == src.numel() * src.element_size()
+    _check(load().qf_stream_copy(dst.data_ptr(), src.data_ptr(), src.numel() * src.element_size(), _stream()), "qf_stream_copy")

@@ -1,0 +1,74 @@
+"""The C-ABI shared objects load without a GPU and export every symbol the headers in include/
+declare.  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+
+INCLUDE = os.path.join(ROOT, "include")
+
+
+def _declared_functions(header, guard=None):
+    """Names of the function prototypes in a header (optionally only those under `#if defined(guard)`)."""
+    text = open(os.path.join(INCLUDE, header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    if guard is not None:
+        m = re.search(r"#(?:el)?if defined\(%s\)(.*?)#(?:elif|endif)" % guard, text, flags=re.S)
+        assert m, f"{guard} block not found in {header}"
+        text = m.group(1)
+    else:
+        text = re.sub(r"#if defined\(.*?#endif", "", text, flags=re.S)
+    text = "\n".join(l for l in text.splitlines() if not l.lstrip().startswith(("#", "typedef")))
+    return sorted(set(re.findall(r"\b([A-Za-z_]\w*)\s*\([^;{]*\)\s*;", text)))
+
+
+def test_header_parsers_see_the_expected_prototypes():
+    assert _declared_functions("qfactory_hip.h") == sorted(
+        ["qf_version", "qf_pack_weight", "qf_pack_zero", "qf_transpose_scale", "qf_stream_read", "qf_stream_copy"])
+    assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_GROUPED") == ["launch", "launch_m", "qf_describe"]
+    assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_PLAIN") == ["launch", "qf_describe"]
+
+
+def test_aot_library_exports_every_declared_symbol():
+    from qfactory import native
+    native.build()
+    lib = ctypes.CDLL(native.LIBRARY)
+    for name in _declared_functions("qfactory_hip.h"):
+        assert hasattr(lib, name), f"{name} missing from {native.LIBRARY}"
+    assert sorted(native.SIGNATURES) == _declared_functions("qfactory_hip.h")
+    lib.qf_version.restype = ctypes.c_int
+    assert lib.qf_version() == 100          # host-only call: no device work
+
+
+@pytest.mark.parametrize("gs,guard", [(128, "QF_LAUNCH_GROUPED"), (-1, "QF_LAUNCH_PLAIN")])
+def test_jit_object_exports_the_launch_abi(gs, guard):
+    from qfactory.core.qfunc import MatmulQFunc, QMatmulQFunc
+    from qfactory.core.qtile import AsymQTile, QTile
+    from qfactory.jit import jit
+    a = QTile((1, 512), torch.float16, 16)
+    if gs == -1:
+        qfunc = MatmulQFunc(a, QTile((64, 512), torch.int8, 4), "nt")
+    else:
+        qfunc = QMatmulQFunc(a, AsymQTile((64, 512), torch.int8, 4, (1, gs)), "nt")
+    runtime = jit.compile(qfunc)
+    lib = ctypes.CDLL(os.path.join(runtime.path, "kernel.so"))
+    for name in _declared_functions("qfactory_launch.h", guard):
+        assert hasattr(lib, name), f"{name} missing from {runtime.path}"
+    lib.qf_describe.restype = ctypes.c_char_p
+    text = lib.qf_describe().decode()
+    assert "N=64" in text and "K=512" in text and "NBITS=4" in text
+    # the generated translation unit includes the ABI header and implements the matching variant
+    src = open(os.path.join(runtime.path, "kernel.hip")).read()
+    assert f"#define {guard}" in src and '#include "qfactory_launch.h"' in src
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from qfactory import native
+    monkeypatch.setattr(native, "_lib", None)
+    monkeypatch.setattr(native, "LIBRARY", str(tmp_path / "absent.so"))
+    with pytest.raises(RuntimeError, match="missing"):
+        native.load()
