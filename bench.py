@@ -159,6 +159,30 @@ def gemm_report(M=256, copies_bytes=600e6):
     return report
 
 
+COPY_BYTES = 64 << 20
+
+# HBM traffic per launch of the dominant kernel, from hardware counters: rocprofv3 --pmc FETCH_SIZE
+# and --pmc WRITE_SIZE over `bench.py --counter-pass`, each scaled by what the same counter reads
+# for the 64 MiB stream copy of that run (which moves COPY_BYTES each way).  Keyed by the kernel's
+# description so that a different specialisation reports null instead of a stale figure.
+MEASURED_TRAFFIC = {}
+
+
+def counter_pass(layers, acts, reps=5):
+    import torch
+    from qfactory import native
+    src = torch.randint(-128, 128, (COPY_BYTES,), dtype=torch.int8, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for r in range(reps):
+        for name, N, K in SHAPES:
+            layers[r % len(layers)][name](acts[K])
+        native.stream_copy(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    log(f"[bench] counter pass: {reps} launches of each kernel and of a {COPY_BYTES} byte stream copy")
+
+
 def cpu_baseline(budget_s=15.0):
     """torch-CPU dequant + fp32 matmul over the same four shapes, bounded to about `budget_s`."""
     import torch
@@ -201,6 +225,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=256 GEMM report")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
+    ap.add_argument("--counter-pass", action="store_true",
+                    help="only launch each of the four kernels (cold weights) and a 64 MiB stream copy a few times, "
+                         "eagerly: the run to put under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the path; this build runs on exactly one GPU (--gpus 1)")
@@ -214,6 +241,10 @@ def main():
     log(f"[bench] parity of benchmark data vs oracle: {parity}")
 
     step_bytes = sum(algorithmic_bytes(M, N, K) for _, N, K in SHAPES)
+
+    if args.counter_pass:
+        counter_pass(layers, acts)
+        return
 
     for i in range(args.warmup):
         run_step(layers[i % len(layers)], acts)
@@ -270,7 +301,8 @@ def main():
                    "bytes_per_step": int(step_bytes), "timed_with": "eager" if args.no_graph else "one HIP graph of all steps"},
         "hbm_frac_whole_step": round(value / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "achieved": dominant["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(dominant["GB/s"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(dominant["GB/s"] / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(dominant["kernel"]),
                      "kernel": f"qf::gemv_kernel {DOMINANT} N=22016 K=4096 M=1", "avg_launch_us": dominant["us"],
                      "algorithmic_bytes_per_launch": dominant["bytes"]},
         "shapes": shapes_report,

@@ -24,9 +24,12 @@
  * 3-bit has no counterpart in the reference (PERMUTE_ORDER has keys 8/4/2 only,
  * convert.py:49-53).  The layout restated here is this project's own:
  * per row, a 2-bit plane (low two bits, packed exactly like the reference's
- * 2-bit layout) of K/4 bytes followed by a 1-bit plane (high bit; per 32-bit
- * word: even-indexed elements in bits 0..15, odd-indexed in bits 16..31) of K/8
- * bytes.  Zero-points for 3-bit are stored one per nibble (two groups per byte).
+ * 2-bit layout) of K/4 bytes followed by a 1-bit plane (high bit) of K/8 bytes.
+ * A 32-bit word of the 1-bit plane serves the two 2-bit words of the same 32
+ * elements; element e sits at the bit that, after one shift of the whole word,
+ * lands directly above that element's 2-bit field (hi_plane_pos below), so a
+ * kernel merges the planes with one AND-OR per element pair.
+ * Zero-points for 3-bit are stored one per nibble (two groups per byte).
  * PARITY UNPINNED by the reference for NBITS == 3: only round trips, the
  * dequant+matmul identity and the special cases in tests/ pin it.
  *
@@ -98,6 +101,15 @@ static int perm_index(int nbits, int j) {
     return (j < p32 / 2) ? 2 * j : 2 * (j - p32 / 2) + 1;
 }
 
+/* Bit of a 1-bit-plane word that holds the high bit of element e (0..31) of its 32 elements.
+   r: which of the two 2-bit words, i: pair inside it, h: half-word (even / odd element),
+   p: pair inside its byte, upper: which byte of the half-word. */
+static int hi_plane_pos(int e) {
+    int r = e / 16, ep = e % 16, i = ep / 2, h = ep % 2, p = i % 4, upper = i / 4;
+    int base = (p % 2 == 0) ? 2 * p + 2 : 2 * p - 2;
+    return base + 8 * upper + r + 16 * h;
+}
+
 /* bytes per packed weight row */
 int64_t qfo_row_bytes(int64_t K, int nbits) { return K * nbits / 8; }
 
@@ -116,10 +128,8 @@ int qfo_pack_weight(int64_t K, int64_t N, int nbits, const int32_t *weight, int8
             }
             for (int64_t i = 0; i < K / 32; i++) {       /* 1-bit plane, 32 elements per word */
                 uint32_t u = 0;
-                for (int j = 0; j < 32; j++) {
-                    int src = (j < 16) ? 2 * j : 2 * (j - 16) + 1;
-                    u |= (((uint32_t)weight[(i * 32 + src) * N + n] >> 2) & 1u) << j;
-                }
+                for (int e = 0; e < 32; e++)
+                    u |= (((uint32_t)weight[(i * 32 + e) * N + n] >> 2) & 1u) << hi_plane_pos(e);
                 for (int t = 0; t < 4; t++) row[lo_bytes + i * 4 + t] = (uint8_t)(u >> (8 * t));
             }
         }
@@ -189,10 +199,8 @@ int qfo_unpack_weight(int64_t K, int64_t N, int nbits, const int8_t *w, int32_t 
             for (int64_t i = 0; i < K / 32; i++) {
                 uint32_t u;
                 memcpy(&u, row + lo_bytes + i * 4, 4);
-                for (int p = 0; p < 16; p++) {
-                    q[n * K + i * 32 + 2 * p] |= (int32_t)(((u >> p) & 1u) << 2);
-                    q[n * K + i * 32 + 2 * p + 1] |= (int32_t)(((u >> (p + 16)) & 1u) << 2);
-                }
+                for (int e = 0; e < 32; e++)
+                    q[n * K + i * 32 + e] |= (int32_t)(((u >> hi_plane_pos(e)) & 1u) << 2);
             }
         }
         return 0;

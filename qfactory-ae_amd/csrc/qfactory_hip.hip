@@ -29,8 +29,15 @@ int launched(const char* fn) {
 // block are arranged 32 (rows n) x 8 (words): the reads of weight[k][n] are contiguous over n
 // (128 B per k), the 4-byte writes of a row are contiguous over the 8 words.
 // Position j of a word holds element (j < P/2 ? 2j : 2(j - P/2) + 1) of its P = 32/b elements
-// (identity for 8-bit): evens in the low half-word, odds in the high half-word.
+// (identity for 8-bit): evens in the low half-word, odds in the high half-word.  The 1-bit plane
+// of the 3-bit layout has its own order (hi_plane_pos): every high bit sits where one shift of
+// the word drops it directly above the element's field in the 2-bit plane.
 // ---------------------------------------------------------------------------------------------
+__host__ __device__ constexpr int hi_plane_pos(int e) {
+    const int r = e / 16, ep = e % 16, i = ep / 2, h = ep % 2, p = i % 4, upper = i / 4;
+    return ((p % 2 == 0) ? 2 * p + 2 : 2 * p - 2) + 8 * upper + r + 16 * h;
+}
+
 template <int B>   // field width of the plane being written: 1, 2, 4 or 8
 __device__ __forceinline__ uint32_t build_word(const int32_t* __restrict__ weight, int64_t N, int64_t n,
                                                int64_t k0, int shift, uint32_t mask) {
@@ -38,7 +45,8 @@ __device__ __forceinline__ uint32_t build_word(const int32_t* __restrict__ weigh
     uint32_t word = 0;
 #pragma unroll
     for (int j = 0; j < P; j++) {
-        const int src = (B == 8) ? j : (j < P / 2 ? 2 * j : 2 * (j - P / 2) + 1);
+        // hi_plane_pos is its own inverse: bit j holds element hi_plane_pos(j)
+        const int src = (B == 8) ? j : (B == 1) ? hi_plane_pos(j) : (j < P / 2 ? 2 * j : 2 * (j - P / 2) + 1);
         const uint32_t v = ((uint32_t)weight[(k0 + src) * N + n] >> shift) & mask;
         word |= v << (j * B);
     }

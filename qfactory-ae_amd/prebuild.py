@@ -32,15 +32,17 @@ def parity_cases():
         for M in (1, 4, 16):
             cases.append(_case(M, N, K))
     for M in (1, 16):                                        # bit-width scaling at N = K = 8192
-        for nbits in (2, 4, 8):
+        for nbits in (2, 3, 4, 8):
             for sym in (False, True):
                 cases.append(_case(M, 8192, 8192, nbits, 128, sym))
     # ragged / small shapes: N not a multiple of the rows per block, odd M, other group sizes
     cases += [_case(1, 100, 256, 4, 128), _case(2, 100, 256, 4, 64), _case(3, 130, 512, 4, 32),
               _case(5, 77, 1024, 4, 128), _case(7, 1000, 2048, 8, 128), _case(2, 64, 512, 2, 64),
               _case(1, 48, 4096, 2, 128, True), _case(3, 48, 1024, 8, 256, True),
-              _case(1, 256, 11008, 4, 128)]
-    for nbits in (2, 4, 8):                                  # group_size == -1: raw integer weights
+              _case(1, 256, 11008, 4, 128),
+              _case(1, 100, 256, 3, 64), _case(2, 77, 1024, 3, 128, True), _case(5, 130, 512, 3, 32),
+              _case(33, 64, 2048, 3, 128), _case(1, 50, 11008, 3, 128)]
+    for nbits in (2, 3, 4, 8):                                  # group_size == -1: raw integer weights
         cases += [_case(1, 4096, 4096, nbits, -1), _case(3, 100, 256, nbits, -1)]
     # matrix-core regime: ragged M and N, M above one block tile, other widths and group sizes
     cases += [_case(33, 100, 512, 4, 128), _case(100, 1000, 1024, 4, 64), _case(300, 256, 2048, 4, 128),

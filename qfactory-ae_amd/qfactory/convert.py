@@ -19,9 +19,11 @@ Layout produced (reference file:line in brackets):
 
 Extension with no counterpart in the reference: ``NBITS == 3``.  A row is a 2-bit plane (the low two
 bits of every element, in exactly the 2-bit layout above, K/4 bytes) followed by a 1-bit plane (the
-high bit; per 32-bit word even-indexed elements in bits 0..15, odd-indexed in bits 16..31, K/8
-bytes): 3*K/8 bytes per row, both planes loadable with aligned vector loads.  3-bit zero-points are
-stored one per nibble.
+high bits, K/8 bytes): 3*K/8 bytes per row, both planes loadable with aligned vector loads.  One
+32-bit word of the 1-bit plane serves the two 2-bit words of the same 32 elements; its bit order
+(``_hi_plane_order``) puts every high bit where one shift of the whole word drops it directly above
+the element's 2-bit field, so the kernels merge the planes with one AND-OR per element pair.
+3-bit zero-points are stored one per nibble.
 """
 import torch
 
@@ -70,13 +72,26 @@ def _evens_then_odds(n):
     return list(range(0, n, 2)) + list(range(1, n, 2))
 
 
+def _hi_plane_order():
+    """Element held by each bit of a 1-bit-plane word.  Element e = 16*r + 2*i + h (r: which 2-bit
+    word, i: pair, h: even/odd element = low/high half-word), with p = i % 4 the pair inside its byte
+    and upper = i // 4 the byte, sits at bit (2p+2 if p even else 2p-2) + 8*upper + r + 16*h."""
+    pos = []
+    for e in range(32):
+        r, ep = divmod(e, 16)
+        i, h = divmod(ep, 2)
+        p, upper = i % 4, i // 4
+        pos.append((2 * p + 2 if p % 2 == 0 else 2 * p - 2) + 8 * upper + r + 16 * h)
+    return [pos.index(j) for j in range(32)]
+
+
 # Position j of a packed 32-bit word holds element PERMUTE_ORDER[b][j] (convert.py:49-53).  The
 # 1-bit entry is only used for the high-bit plane of the 3-bit layout.
 PERMUTE_ORDER = {
     8: [0, 1, 2, 3],
     4: _evens_then_odds(8),
     2: _evens_then_odds(16),
-    1: _evens_then_odds(32),
+    1: _hi_plane_order(),
 }
 
 

@@ -36,14 +36,20 @@ def regime_for(M, K=None, nbits=None, group_size=None):
     return "mfma"
 
 
+def plane_bits(nbits):
+    """Field width of the main weight plane: 3-bit rows are a 2-bit plane plus a 1-bit plane."""
+    return 2 if nbits == 3 else nbits
+
+
 def elements_per_chunk(nbits, vb):
-    return vb * 8 // nbits
+    return vb * 8 // plane_bits(nbits)
 
 
 def gemv_vec_bytes(K, nbits, group_size):
-    """Widest per-lane load (16/8/4 bytes) that divides a packed row and stays inside one group."""
-    row_bytes = K * nbits // 8
-    for vb in (16, 8, 4):
+    """Widest per-lane load (16/8/4 bytes of the main plane) that divides a packed row and stays
+    inside one group; 3-bit rows need at least 8 (one whole word of the 1-bit plane per chunk)."""
+    row_bytes = K * plane_bits(nbits) // 8
+    for vb in ((16, 8) if nbits == 3 else (16, 8, 4)):
         epc = elements_per_chunk(nbits, vb)
         if row_bytes % vb:
             continue

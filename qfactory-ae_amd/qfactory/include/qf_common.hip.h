@@ -111,6 +111,37 @@ template <> struct Decode<2> {
     }
 };
 
+// 3-bit rows are a 2-bit plane followed by a 1-bit plane (this project's layout; the reference has
+// no 3-bit).  Word `w` of the 2-bit plane holds 16 elements; word `h` of the 1-bit plane holds the
+// high bits of 32 elements, i.e. of 2-bit words 2J (r = 0) and 2J + 1 (r = 1).  The plane's bit
+// order is such that four shifts of `h` line every high bit up directly above its 2-bit field;
+// one AND-OR per pair then yields 1024 + 2^o * (lo + 4 * hi), decoded exactly like a 2-bit pair.
+template <> struct Decode<3> {
+    static constexpr int PAIRS = 8;
+    static constexpr int NCLS = 4;
+    __host__ __device__ static constexpr int cls(int pair) { return pair & 3; }
+    __host__ __device__ static constexpr float inv_scale(int c) { return Decode<2>::inv_scale(c); }
+    template <int R>
+    __device__ __forceinline__ static void word(uint32_t w, uint32_t h, uint32_t (&x)[PAIRS]) {
+        const uint32_t w8 = w >> 8;
+        const uint32_t he0 = h >> R, he1 = h >> (8 + R);           // pairs 0, 2 of the low / high byte
+        const uint32_t ho0 = h << (4 - R), ho1 = h >> (4 + R);     // pairs 1, 3 of the low / high byte
+        x[0] = (w & 0x00030003u) | (he0 & 0x00040004u) | kMagic;
+        x[1] = (w & 0x000C000Cu) | (ho0 & 0x00100010u) | kMagic;
+        x[2] = (w & 0x00300030u) | (he0 & 0x00400040u) | kMagic;
+        x[3] = (w & 0x00C000C0u) | (ho0 & 0x01000100u) | kMagic;
+        x[4] = (w8 & 0x00030003u) | (he1 & 0x00040004u) | kMagic;
+        x[5] = (w8 & 0x000C000Cu) | (ho1 & 0x00100010u) | kMagic;
+        x[6] = (w8 & 0x00300030u) | (he1 & 0x00400040u) | kMagic;
+        x[7] = (w8 & 0x00C000C0u) | (ho1 & 0x01000100u) | kMagic;
+    }
+};
+
+// Bits per field of the main weight plane and of a stored zero-point (3-bit: 2-bit main plane plus
+// a 1-bit plane; zero-points one per nibble).
+__host__ __device__ constexpr int plane_bits(int nbits) { return nbits == 3 ? 2 : nbits; }
+__host__ __device__ constexpr int zero_field_bits(int nbits) { return nbits == 3 ? 4 : nbits; }
+
 template <> struct Decode<8> {
     static constexpr int PAIRS = 2;
     static constexpr int NCLS = 1;

@@ -27,7 +27,7 @@ namespace qf {
 template <int NBITS_, int GS_, bool SYM_, bool QPARAM_, int N_, int K_, int MT_, int WK_, int WN_,
           int U_, int STEPS_, int VB_, bool NT_B_>
 struct GemvCfg {
-    static constexpr int NBITS = NBITS_;      // weight field width: 2, 4 or 8
+    static constexpr int NBITS = NBITS_;      // weight field width: 2, 3, 4 or 8
     static constexpr int GS = GS_;            // group size along K (ignored when !QPARAM)
     static constexpr bool SYM = SYM_;         // implicit zero-point 2^(b-1), no zero tensor read
     static constexpr bool QPARAM = QPARAM_;   // false: no scale / zero at all (group_size == -1 path)
@@ -40,8 +40,11 @@ struct GemvCfg {
     static constexpr int VB = VB_;            // bytes of packed weight per lane and load: 16, 8 or 4
     static constexpr bool NT_B = NT_B_;       // stream the weights with non-temporal loads
 
-    static constexpr int NW = VB / 4;                   // 32-bit words per chunk
-    static constexpr int EPC = VB * 8 / NBITS;          // elements per chunk
+    static constexpr int PB = plane_bits(NBITS);        // field width of the main plane (3-bit: 2 + 1-bit plane)
+    static constexpr int NW = VB / 4;                   // 32-bit words of the main plane per chunk
+    static constexpr int NWH = NBITS == 3 ? NW / 2 : 0; // 32-bit words of the 1-bit plane per chunk
+    static constexpr int HI_OFF = K / 4;                // byte offset of the 1-bit plane in a 3-bit row
+    static constexpr int EPC = VB * 8 / PB;             // elements per chunk
     static constexpr int NCH = K / EPC;                 // chunks per row
     static constexpr int T = 64 * WK;                   // threads per team
     static constexpr int IT = (NCH + T - 1) / T;        // chunks per lane and row
@@ -51,7 +54,8 @@ struct GemvCfg {
     static constexpr int V = U * MT;                    // partial sums per stage
     static constexpr int RB = K * NBITS / 8;            // packed weight row bytes
     static constexpr int G = QPARAM ? K / (GS > 0 ? GS : 1) : 0;   // groups per row
-    static constexpr int ZRB = G * NBITS / 8;           // packed zero row bytes
+    static constexpr int ZFB = zero_field_bits(NBITS);  // stored width of one zero-point
+    static constexpr int ZRB = G * ZFB / 8;             // packed zero row bytes
     static constexpr int GRID_X = (N + RPB - 1) / RPB;
 };
 
@@ -64,8 +68,9 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
     constexpr int MT = C::MT, U = C::U, STEPS = C::STEPS, V = C::V, WK = C::WK;
     constexpr int PAIRS = D::PAIRS, NCLS = D::NCLS;
     constexpr int AR = NW * PAIRS;                     // 32-bit activation registers per chunk
-    constexpr int P8 = 8 / C::NBITS;                   // zero-point fields per byte
-    constexpr uint32_t ZMASK = (1u << C::NBITS) - 1u;
+    constexpr int P8 = 8 / C::ZFB;                     // zero-point fields per byte
+    constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
+    constexpr int NWH = C::NWH;
 
     __shared__ float red[C::WN][WK][STEPS * V];
 
@@ -94,6 +99,7 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
     // ---- streaming stages ----
     struct Stage {
         uint32_t w[U][IT][NW];
+        uint32_t h[U][IT][NWH > 0 ? NWH : 1];
         scale_holder_t s[U][IT];
         zero_holder_t z[U][IT];
     };
@@ -106,6 +112,7 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
 #pragma unroll
             for (int it = 0; it < IT; it++) {
                 load_words<NW, C::NT_B>(wrow + coff[it], st.w[u][it]);
+                if constexpr (NWH > 0) load_words<NWH, C::NT_B>(wrow + C::HI_OFF + coff[it] / 2, st.h[u][it]);
                 if constexpr (C::QPARAM) {
                     st.s[u][it] = S[(size_t)row * C::G + goff[it]];
                     if constexpr (!C::SYM) st.z[u][it] = Zp[(size_t)row * C::ZRB + goff[it] / P8];
@@ -173,7 +180,12 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
 #pragma unroll
                 for (int j = 0; j < NW; j++) {
                     uint32_t x[PAIRS];
-                    D::word(st.w[u][it][j], x);
+                    if constexpr (C::NBITS == 3) {
+                        if (j % 2 == 0) D::template word<0>(st.w[u][it][j], st.h[u][it][j / 2], x);
+                        else D::template word<1>(st.w[u][it][j], st.h[u][it][j / 2], x);
+                    } else {
+                        D::word(st.w[u][it][j], x);
+                    }
 #pragma unroll
                     for (int p = 0; p < PAIRS; p++)
 #pragma unroll
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(C::THREADS) void gemv_kernel(
                     if constexpr (C::SYM) {
                         zf = (float)(1 << (C::NBITS - 1));
                     } else {
-                        zf = (float)((st.z[u][it] >> ((goff[it] % P8) * C::NBITS)) & ZMASK);
+                        zf = (float)((st.z[u][it] >> ((goff[it] % P8) * C::ZFB)) & ZMASK);
                     }
                 }
 #pragma unroll
@@ -256,12 +268,13 @@ template <class C>
 int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m,
                 hipStream_t stream) {
     const char* why = nullptr;
-    if (C::NBITS != 2 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 4 or 8 for this kernel";
+    if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8";
     else if (C::VB != 4 && C::VB != 8 && C::VB != 16) why = "VB must be 4, 8 or 16";
-    else if ((C::K * C::NBITS) % (8 * C::VB) != 0) why = "K*NBITS/8 must be a multiple of VB";
+    else if (C::NBITS == 3 && C::VB < 8) why = "3-bit rows need VB >= 8 (a whole word of the 1-bit plane per chunk)";
+    else if ((C::K * C::PB) % (8 * C::VB) != 0) why = "a packed row (main plane) must be a multiple of VB bytes";
     else if (C::QPARAM && (C::GS <= 0 || C::K % C::GS != 0)) why = "GS must divide K";
     else if (C::QPARAM && C::GS % C::EPC != 0) why = "a VB-byte chunk must lie inside one group";
-    else if (C::QPARAM && !C::SYM && (C::G % (8 / C::NBITS)) != 0) why = "K/GS must fill whole zero-point bytes";
+    else if (C::QPARAM && !C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if ((C::V & (C::V - 1)) != 0 || C::V > 64) why = "U*MT must be a power of two <= 64";
     else if (C::THREADS > 1024) why = "block too large";
     else if (C::WN * C::WK * C::STEPS * C::V * 4 > 64 * 1024) why = "reduction scratch exceeds LDS";

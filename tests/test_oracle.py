@@ -40,12 +40,40 @@ def test_pack_weight_kat_two_words_two_columns(oracle):
 
 def test_pack_weight_kat_3bit(oracle):
     # 3-bit layout of this project: 2-bit plane (low bits) then 1-bit plane (high bit).
-    # W[k] = k % 8 for K = 32: low bits k%4 -> two words 0xDDDD8888; high bit set for k%8 >= 4:
-    # evens 4,6,12,14,... -> positions 2,3,6,7,10,11,14,15 -> 0xCCCC, odds identical.
+    # W[k] = k % 8 for K = 32: low bits k%4 -> two words 0xDDDD8888.  High bit set for k%8 >= 4, i.e.
+    # pairs i = 2,3,6,7 of both 2-bit words: (p, upper) = (2,0),(3,0),(2,1),(3,1) -> bits 6,4,14,12 for
+    # the first word and one higher for the second, in both half-words -> 0xF0F0F0F0.
     W = (np.arange(32, dtype=np.int32) % 8).reshape(32, 1)
     w = oracle.pack_weight(W, 3).view(np.uint8)
     assert w.shape == (1, 12)
-    assert w[0].tolist() == [0x88, 0x88, 0xDD, 0xDD, 0x88, 0x88, 0xDD, 0xDD, 0xCC, 0xCC, 0xCC, 0xCC]
+    assert w[0].tolist() == [0x88, 0x88, 0xDD, 0xDD, 0x88, 0x88, 0xDD, 0xDD, 0xF0, 0xF0, 0xF0, 0xF0]
+
+
+def test_3bit_planes_merge_with_one_shift_per_class(oracle):
+    """The property the 1-bit plane's bit order exists for: after one shift of the whole plane
+    word, every high bit sits directly above its element's 2-bit field, so
+    (lo & 3<<o) | (hi_shifted & 4<<o) is the 3-bit value at offset o of each half-word."""
+    rng = np.random.default_rng(11)
+    K = 96
+    W = rng.integers(0, 8, size=(K, 1), dtype=np.int32)
+    row = oracle.pack_weight(W, 3).view(np.uint8)[0]
+    lo = row[: K // 4].copy().view("<u4").astype(np.uint64)
+    hi = row[K // 4:].copy().view("<u4").astype(np.uint64)
+    M32 = 0xFFFFFFFF
+    for j in range(K // 16):
+        w, H = int(lo[j]), int(hi[j // 2])
+        Hr = H >> (j % 2)
+        for upper in (0, 1):
+            wd = (w >> 8) if upper else w
+            for p in range(4):
+                if p % 2 == 0:
+                    hsel = (Hr >> 8) if upper else Hr
+                else:
+                    hsel = (Hr >> 4) if upper else (Hr << 4) & M32
+                x = (wd & (0x00030003 << (2 * p))) | (hsel & (0x00040004 << (2 * p)))
+                i = p + 4 * upper
+                assert (x >> (2 * p)) & 7 == W[16 * j + 2 * i, 0]
+                assert (x >> (2 * p + 16)) & 7 == W[16 * j + 2 * i + 1, 0]
 
 
 def test_pack_zero_kats(oracle):
