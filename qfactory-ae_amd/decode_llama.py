@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Single-GPU greedy decode loop of a Llama-2-7B-shaped model whose linears are W4A16 g128 QLinear.
+
+BASELINE.json configs[4]: 32 layers, hidden 4096, 32 heads, SwiGLU MLP 11008, vocab 32000, RMSNorm,
+RoPE; random-initialised weights; batch in {1, 16, 64}; 128 random prompt ids, 128 greedy output
+tokens.  It stands in for the reference's end-to-end runs through vLLM (reproduce/fig11,
+third_party/vllm-qfactory.patch), which need vLLM and model downloads.
+
+The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear modules; prefill
+(M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
+regimes through the layers' own row-count dispatch.  Everything else (embedding, RMSNorm, RoPE,
+attention over a static KV cache, SiLU, the fp16 lm_head) is plain PyTorch.  One decode step --
+including the argmax and the position update -- is captured in a HIP graph and replayed per token.
+
+Prints one JSON line per batch size: tokens/s over the decode phase, prefill time, and the share of
+a decode step spent in the quantized linears (their kernels timed separately at the same M).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from dataclasses import dataclass
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+if HERE not in sys.path:
+    sys.path.insert(0, HERE)
+os.environ.setdefault("QFACTORY_CACHE_DIR", os.path.join(HERE, "jit_cache"))
+os.environ.setdefault("QFACTORY_LOG_LEVEL", "WARNING")
+
+import torch
+import torch.nn.functional as F
+
+NO_SEARCH = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
+
+
+@dataclass
+class LlamaShape:
+    layers: int = 32
+    hidden: int = 4096
+    heads: int = 32
+    mlp: int = 11008
+    vocab: int = 32000
+    max_len: int = 256
+    rope_theta: float = 10000.0
+    eps: float = 1e-5
+    nbits: int = 4
+    group_size: int = 128
+
+
+def _random_qlinear(batch, K, N, shape, gen):
+    """A QLinear with random packed fields and scales sized so that the layer has gain ~0.5."""
+    from qfactory import QLinear
+    lin = QLinear.empty(batch, K, N, shape.nbits, shape.group_size, sym=False, compile_flags=NO_SEARCH)
+    lin.w.copy_(torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=gen))
+    lin.z.copy_(torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=gen))
+    spread = (2 ** shape.nbits) * 0.41                      # std of q - Z for independent uniform fields
+    base = 0.5 / (spread * K ** 0.5)
+    lin.s.copy_(((torch.rand(lin.s.shape, device="cuda", generator=gen) + 0.5) * base).to(torch.float16))
+    return lin
+
+
+class QuantLlama:
+    def __init__(self, shape: LlamaShape, batch: int, seed: int = 0):
+        self.shape, self.batch = shape, batch
+        gen = torch.Generator(device="cuda").manual_seed(seed)
+        h, hd = shape.hidden, shape.hidden // shape.heads
+        self.embed = (torch.randn(shape.vocab, h, device="cuda", generator=gen) * 0.5).to(torch.float16)
+        self.lm_head = (torch.randn(shape.vocab, h, device="cuda", generator=gen) / h ** 0.5).to(torch.float16)
+        self.final_norm = torch.ones(h, dtype=torch.float16, device="cuda")
+        self.layers = []
+        for _ in range(shape.layers):
+            self.layers.append({
+                "norm1": torch.ones(h, dtype=torch.float16, device="cuda"),
+                "norm2": torch.ones(h, dtype=torch.float16, device="cuda"),
+                "qkv": _random_qlinear(batch, h, 3 * h, shape, gen),
+                "o": _random_qlinear(batch, h, h, shape, gen),
+                "gate_up": _random_qlinear(batch, h, 2 * shape.mlp, shape, gen),
+                "down": _random_qlinear(batch, shape.mlp, h, shape, gen),
+            })
+        self.k_cache = torch.zeros(shape.layers, batch, shape.heads, shape.max_len, hd, dtype=torch.float16, device="cuda")
+        self.v_cache = torch.zeros_like(self.k_cache)
+        inv = 1.0 / (shape.rope_theta ** (torch.arange(0, hd, 2, device="cuda", dtype=torch.float32) / hd))
+        ang = torch.arange(shape.max_len, device="cuda", dtype=torch.float32)[:, None] * inv[None, :]
+        self.cos, self.sin = ang.cos(), ang.sin()                                   # (max_len, hd/2) fp32
+        self.linear = lambda lin, x: lin(x)                 # hook: tests swap in a dense fp32 evaluation
+
+    def _norm(self, x, w):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.shape.eps)).to(torch.float16) * w
+
+    def _rope(self, x, pos):
+        """x (B, H, T, hd), pos (T,) int64: rotate pairs (2i, 2i+1)."""
+        cos, sin = self.cos.index_select(0, pos)[None, None], self.sin.index_select(0, pos)[None, None]
+        xf = x.float()
+        x0, x1 = xf[..., 0::2], xf[..., 1::2]
+        out = torch.stack((x0 * cos - x1 * sin, x0 * sin + x1 * cos), dim=-1).flatten(-2)
+        return out.to(torch.float16)
+
+    def forward(self, tokens, pos):
+        """tokens (B, T) int64, pos (T,) int64 positions of those tokens.  Returns logits (B, vocab) of the
+        last token; the KV cache is updated in place.  Attention is masked to positions <= the query's."""
+        shape = self.shape
+        B, T = tokens.shape
+        H, hd = shape.heads, shape.hidden // shape.heads
+        x = self.embed[tokens]                                                       # (B, T, h)
+        key_pos = torch.arange(shape.max_len, device="cuda")
+        mask = (key_pos[None, :] <= pos[:, None])[None, None]                        # (1, 1, T, max_len)
+        for li, layer in enumerate(self.layers):
+            hdn = self._norm(x, layer["norm1"]).reshape(B * T, shape.hidden)
+            qkv = self.linear(layer["qkv"], hdn).reshape(B, T, 3, H, hd).permute(2, 0, 3, 1, 4)
+            q, k, v = self._rope(qkv[0], pos), self._rope(qkv[1], pos), qkv[2]
+            self.k_cache[li].index_copy_(2, pos, k)
+            self.v_cache[li].index_copy_(2, pos, v)
+            att = F.scaled_dot_product_attention(q, self.k_cache[li], self.v_cache[li], attn_mask=mask)
+            att = att.permute(0, 2, 1, 3).reshape(B * T, shape.hidden)
+            x = x + self.linear(layer["o"], att).reshape(B, T, shape.hidden)
+            hdn = self._norm(x, layer["norm2"]).reshape(B * T, shape.hidden)
+            gu = self.linear(layer["gate_up"], hdn)
+            act = F.silu(gu[:, : shape.mlp]) * gu[:, shape.mlp:]
+            x = x + self.linear(layer["down"], act.contiguous()).reshape(B, T, shape.hidden)
+        last = self._norm(x[:, -1], self.final_norm)
+        return last @ self.lm_head.T
+
+
+def linears_time_us(model, M, reps=8):
+    """Time of the quantized linears of one decode step at M rows: every layer's four kernels once,
+    back to back in a HIP graph (cold weights: the whole model is streamed), averaged over `reps`."""
+    xs = {K: torch.randn(M, K, device="cuda").to(torch.float16) for K in (model.shape.hidden, model.shape.mlp)}
+
+    def one_pass():
+        for layer in model.layers:
+            for name in ("qkv", "o", "gate_up", "down"):
+                lin = layer[name]
+                lin(xs[lin.in_features])
+
+    one_pass()
+    torch.cuda.synchronize()
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+        one_pass()
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()
+    torch.cuda.synchronize()
+    t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0.record()
+    for _ in range(reps):
+        graph.replay()
+    t1.record()
+    torch.cuda.synchronize()
+    return t0.elapsed_time(t1) * 1e3 / reps
+
+
+def run(shape, batch, prompt_len, new_tokens, seed=0):
+    assert prompt_len + new_tokens <= shape.max_len
+    model = QuantLlama(shape, batch, seed)
+    gen = torch.Generator(device="cuda").manual_seed(seed + 1)
+    prompt = torch.randint(0, shape.vocab, (batch, prompt_len), device="cuda", generator=gen)
+
+    # ---- prefill (eager; also compiles / warms the large-M specialisations on its first call) ----
+    model.forward(prompt, torch.arange(prompt_len, device="cuda"))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = model.forward(prompt, torch.arange(prompt_len, device="cuda"))
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+
+    # ---- decode: one step (forward + argmax + position update) captured in a HIP graph ----
+    tok = logits.argmax(-1, keepdim=True)                        # (B, 1) static buffers of the graph
+    pos = torch.full((1,), prompt_len, device="cuda", dtype=torch.int64)
+    tok0, pos0 = tok.clone(), pos.clone()
+
+    def step():
+        lg = model.forward(tok, pos)
+        tok.copy_(lg.argmax(-1, keepdim=True))
+        pos.add_(1)
+
+    step()                                                       # eager warm-up of the M = batch kernels
+    torch.cuda.synchronize()
+    tok.copy_(tok0), pos.copy_(pos0)
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    tok.copy_(tok0), pos.copy_(pos0)
+    torch.cuda.synchronize()
+    generated = []
+    t0 = time.perf_counter()
+    for _ in range(new_tokens):
+        graph.replay()
+        generated.append(tok.clone())
+    torch.cuda.synchronize()
+    decode_s = time.perf_counter() - t0
+    out_tokens = torch.cat(generated, dim=1)
+    assert out_tokens.shape == (batch, new_tokens) and int(pos) == prompt_len + new_tokens
+
+    step_us = decode_s / new_tokens * 1e6
+    lin_us = linears_time_us(model, batch)
+    return {"metric": "greedy decode throughput, Llama-2-7B shape, W4A16 g128 QLinear", "unit": "tokens/s",
+            "value": round(batch * new_tokens / decode_s, 1), "batch": batch, "prompt_len": prompt_len,
+            "new_tokens": new_tokens, "decode_step_us": round(step_us, 1), "prefill_ms": round(prefill_s * 1e3, 2),
+            "prefill_tokens_per_s": round(batch * prompt_len / prefill_s, 1),
+            "quantized_linears_us_per_step": round(lin_us, 1), "quantized_linear_share": round(lin_us / step_us, 3),
+            "layers": shape.layers, "hidden": shape.hidden, "data": "random weights, random prompt ids"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--batches", type=int, nargs="+", default=[1, 16, 64])
+    ap.add_argument("--prompt-len", type=int, default=128)
+    ap.add_argument("--new-tokens", type=int, default=128)
+    ap.add_argument("--layers", type=int, default=32)
+    args = ap.parse_args()
+    assert torch.cuda.is_available(), "decode_llama.py needs the MI355X"
+    shape = LlamaShape(layers=args.layers, max_len=args.prompt_len + args.new_tokens)
+    for batch in args.batches:
+        print(json.dumps(run(shape, batch, args.prompt_len, args.new_tokens)), flush=True)
+        torch.cuda.empty_cache()
+
+
+if __name__ == "__main__":
+    main()

@@ -69,12 +69,25 @@ def smoke_cases():
 
 def misc_test_cases():
     """Other modules the GPU tests construct (row-count dispatch, argument checks)."""
-    return [_case(M, 96, 512, 4, 128) for M in (1, 2, 3, 6)] + [_case(1, 64, 256, 4, 128)]
+    return ([_case(M, 96, 512, 4, 128) for M in (1, 2, 3, 6)] + [_case(1, 64, 256, 4, 128)]
+            + [_case(1, 384, 1024, 4, 128), _case(64, 384, 1024, 4, 128)])
+
+
+TINY_LLAMA = [(768, 256), (256, 256), (1024, 256), (256, 512)]      # the decode-loop test model, GS = 64
+
+
+def decode_cases():
+    """decode_llama.py: Llama-2-7B shapes at batch 1 / 16 / 64 (decode) and at prefill row counts,
+    plus the tiny model tests/test_decode_gpu.py runs."""
+    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 256)]
+    cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
+    return cases
 
 
 def all_cases():
     seen, out = set(), []
-    for c in parity_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases():
+    for c in (parity_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
+              + decode_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
