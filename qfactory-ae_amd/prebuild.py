@@ -84,6 +84,11 @@ def decode_cases():
     return cases
 
 
+def search_cases():
+    """Problems whose whole tiling search space is compiled (tests/test_tune.py searches on the device)."""
+    return [_case(1, 64, 256, 4, 128)]
+
+
 def all_cases():
     seen, out = set(), []
     for c in (parity_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
@@ -118,6 +123,14 @@ def prebuild(cases=None, force=False, workers=None, verbose=True):
             if path not in seen:
                 seen.add(path)
                 qfuncs.append(q)
+    if cases is None:
+        for case in search_cases():
+            for q in qfuncs_of(case):
+                for cand in q.lower():
+                    path, _ = jit.runtime_path_of(cand)
+                    if path not in seen:
+                        seen.add(path)
+                        qfuncs.append(cand)
     workers = workers or min(16, os.cpu_count() or 4)
     done = 0
     with ThreadPoolExecutor(max_workers=workers) as pool:
