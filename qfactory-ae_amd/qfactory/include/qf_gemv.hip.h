@@ -59,8 +59,18 @@ struct GemvCfg {
     static constexpr int GRID_X = (N + RPB - 1) / RPB;
 };
 
+// Lower bound on resident waves per SIMD the register allocator must leave room for (0: no bound).
+#ifndef QF_GEMV_WAVES_PER_EU
+#define QF_GEMV_WAVES_PER_EU 0
+#endif
+#if QF_GEMV_WAVES_PER_EU > 0
+#define QF_GEMV_OCCUPANCY __attribute__((amdgpu_waves_per_eu(QF_GEMV_WAVES_PER_EU)))
+#else
+#define QF_GEMV_OCCUPANCY
+#endif
+
 template <class C>
-__global__ __launch_bounds__(C::THREADS) void gemv_kernel(
+__global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
     const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
     using D = Decode<C::NBITS>;
