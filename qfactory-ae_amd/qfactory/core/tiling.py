@@ -284,71 +284,66 @@ def mgemv_cfg_string(problem, t, nt_b):
 
 
 # --------------------------------------------------------------------------------------------
-# Large-M GEMM regime (LDS-staged operands, 32x32x16 MFMA, optional split-K over blocks)
+# Large-M GEMM regime (qf::GemmCfg, include/qf_gemm.hip.h): weights dequantised into MFMA
+# fragment registers, activations through LDS, WK wave groups splitting K inside a block
 # --------------------------------------------------------------------------------------------
 GEMM_BK = 64
+
+
+def gemm_lds_bytes(cfg):
+    bm, nt32, wn, wk = cfg["BM"], cfg["NT32"], cfg["WN"], cfg["WK"]
+    bn = 32 * nt32 * wn
+    lds_a = wk * 2 * bm * (GEMM_BK + 8) * 2
+    lds_red = (wk - 1) * bm * bn * 4
+    return max(lds_a, lds_red) + wk * wn * 32 * nt32 * 144
 
 
 def gemm_valid(cfg, K, nbits, group_size):
     """Mirror of the static checks in gemm_launch (qf_gemm.hip.h)."""
     if nbits not in (2, 4, 8):
         return False
-    epl = 128 // nbits
     supk = 1024 // nbits
-    bm, bn, bk, wm, wn, ks, pa = (cfg[k] for k in ("BM", "BN", "BK", "WM", "WN", "KS", "PA"))
-    threads = 64 * wm * wn
-    tm, tn = bm // wm, bn // wn
-    if bm % (32 * wm) or bn % (32 * wn) or threads > 1024 or (tm // 32) * (tn // 32) * 16 > 256:
+    sup = supk // GEMM_BK
+    bm, nt32, wn, wk, pa = (cfg[k] for k in ("BM", "NT32", "WN", "WK", "PA"))
+    if bm <= 0 or bm % 32 or min(nt32, wn, wk) < 1 or 64 * wn * wk > 1024:
         return False
-    if bk % 16 or bk % epl or K % (ks * bk) or K % group_size or group_size % epl:
-        return False
-    if supk % bk or supk // bk < 2 or pa < 2 or (2 * supk // bk) % pa:
+    if K % supk or K % group_size or group_size % 32:
         return False
     if (group_size < supk and supk % group_size) or (group_size > supk and group_size % supk):
         return False
-    if ks > 1 and (K // ks) % min(group_size, supk):
-        return False
-    rb = K * nbits // 8
-    if rb % 16 or rb < 128 or (bn * 8) % threads:
-        return False
-    if (bn * bk // epl) % threads or (bm * bk // 8) % threads:
-        return False
     ngs = max(1, supk // group_size)
-    lds = 2 * (bm + bn) * (bk + 8) * 2 + 2 * bn * 144 + 2 * bn * ngs * 3 + 16
-    return lds <= 160 * 1024
+    if ngs > 8 or ngs * nbits > 32:
+        return False
+    if (bm * 8) % (64 * wn) or pa < 2 or (2 * sup) % pa:
+        return False
+    if (bm // 32) * nt32 * 16 > 256:
+        return False
+    return gemm_lds_bytes(cfg) <= 160 * 1024
 
 
 def gemm_supported(K, nbits, group_size):
-    probe = {"BM": 128, "BN": 128, "BK": GEMM_BK, "WM": 2, "WN": 2, "KS": 1, "PA": 2}
+    probe = {"BM": 64, "NT32": 1, "WN": 4, "WK": 1, "PA": 2}
     return gemm_valid(probe, K, nbits, group_size)
 
 
-def _split_k(tiles, K, bk, align, target_blocks=NUM_CUS, max_ks=8, min_iters=8):
-    best = 1
-    for ks in range(1, max_ks + 1):
-        if K % (ks * bk) or K // (ks * bk) < min_iters or (K // ks) % align:
-            continue
-        best = ks
-        if tiles * ks >= target_blocks:
-            break
-    return best
-
-
 def gemm_tiling(M, N, K, nbits, group_size, **pins):
-    bn = 128
-    # the largest block tile that still gives every CU a block: at M = 256 and N = 8192 a 256- or
-    # 128-row tile would leave half of the 256 CUs idle
-    bm = 64
-    for cand in (256, 128):
-        if M > cand // 2 and -(-N // bn) * -(-M // cand) >= NUM_CUS:
-            bm = cand
+    # the largest block tile (BM x 32*WN) that still gives every CU a block; when even the
+    # smallest leaves CUs idle, the smallest
+    choice = None
+    for bm, wn in ((128, 4), (64, 4), (64, 2), (32, 4), (32, 2)):
+        if bm >= 2 * M and bm > 32:
+            continue
+        choice = (bm, wn)
+        if -(-N // (32 * wn)) * -(-M // bm) >= NUM_CUS:
             break
-    wm, wn = (2, 2) if bm >= 128 else (1, 4)
-    tiles = -(-N // bn) * -(-M // bm)
-    # split-K over blocks costs a fenced round trip through memory (tens of microseconds on
-    # MI355X): only worth it when the tiles alone would leave most of the machine idle
-    ks = _split_k(tiles, K, GEMM_BK, min(group_size, 1024 // nbits)) if tiles < NUM_CUS // 8 else 1
-    cfg = {"BM": bm, "BN": bn, "BK": GEMM_BK, "WM": wm, "WN": wn, "KS": ks, "PA": 2}
+    bm, wn = choice
+    blocks = -(-N // (32 * wn)) * -(-M // bm)
+    # with at most one block per CU the K axis is split over wave groups inside the block, so
+    # that every SIMD still holds two waves (one dequantises while the other multiplies)
+    wk = max(1, 8 // wn) if blocks < 2 * NUM_CUS else 1
+    nsup = K // (1024 // nbits)
+    wk = max(1, min(wk, nsup))
+    cfg = {"BM": bm, "NT32": 1, "WN": wn, "WK": wk, "PA": 2}
     cfg.update(pins)
     return cfg
 
@@ -363,19 +358,18 @@ def gemm_candidates(M, N, K, nbits, group_size):
             out.append(cfg)
 
     add(gemm_tiling(M, N, K, nbits, group_size))
-    for bm in (64, 128, 256):
-        if bm >= 2 * M and bm > 64:
+    for bm in (32, 64, 128, 256):
+        if bm >= 2 * M and bm > 32:
             continue
-        for bn in (64, 128, 256):
-            for wm, wn in ((1, 4), (2, 2), (4, 1), (2, 4), (4, 2)):
-                for bk in (32, 64):
-                    for ks in (1, 2, 4):
-                        for pa in (2, 4):
-                            add({"BM": bm, "BN": bn, "BK": bk, "WM": wm, "WN": wn, "KS": ks, "PA": pa})
+        for nt32 in (1, 2):
+            for wn in (2, 4):
+                for wk in (1, 2, 4):
+                    for pa in (2, 4):
+                        add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})
     return out
 
 
 def gemm_cfg_string(problem, t, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::GemmCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
-            f"{t['BM']}, {t['BN']}, {t['BK']}, {t['WM']}, {t['WN']}, {t['KS']}, {t['PA']}, {b(nt_b)}>")
+            f"{t['BM']}, {t['NT32']}, {t['WN']}, {t['WK']}, {t['PA']}, {b(nt_b)}>")
