@@ -143,7 +143,12 @@ class QMatmulQFunc(QFunc):
         t = self.tiling_configs
         b = lambda x: "true" if x else "false"
         code = "// QFactory-HIP generated translation unit\n\n"
-        for name, value in sorted(getattr(self, "defines", {}).items()):   # kernel-header tuning knobs
+        defines = dict(getattr(self, "defines", {}))                        # kernel-header tuning knobs
+        if self.regime == "gemm":
+            # the GEMM kernel is bound by vector-instruction issue and has registers to spare: the
+            # one-instruction mask-and-merge decode pays there (it does not in the GEMV kernel)
+            defines.setdefault("QF_FUSED_AND_OR", 1)
+        for name, value in sorted(defines.items()):
             code += f"#define {name} {value}\n"
         if self.regime == "gemv":
             code += '#include "qf_gemv.hip.h"\n'

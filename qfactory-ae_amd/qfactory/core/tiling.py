@@ -293,9 +293,18 @@ GEMM_BK = 64
 def gemm_lds_bytes(cfg):
     bm, nt32, wn, wk = cfg["BM"], cfg["NT32"], cfg["WN"], cfg["WK"]
     bn = 32 * nt32 * wn
-    lds_a = wk * 2 * bm * (GEMM_BK + 8) * 2
+    lds_a = wk * 3 * bm * (GEMM_BK + 8) * 2
     lds_red = (wk - 1) * bm * bn * 4
     return max(lds_a, lds_red) + wk * wn * 32 * nt32 * 144
+
+
+def gemm_regs(cfg):
+    """Rough VGPR need of one lane: accumulators, two sets of activation fragments, the weight
+    super ring and the activation ring, plus ~80 of addresses and dequantisation temporaries.
+    A SIMD has 512 per lane to share between the waves a block puts on it (spills are ruinous)."""
+    mt32, nt32 = cfg["BM"] // 32, cfg["NT32"]
+    ua = max(1, cfg["BM"] * 8 // (64 * cfg["WN"]))
+    return mt32 * nt32 * 16 + 2 * mt32 * 16 + 2 * nt32 * 20 + cfg["PA"] * ua * 4 + 80
 
 
 def gemm_valid(cfg, K, nbits, group_size):
@@ -318,6 +327,8 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     if (bm // 32) * nt32 * 16 > 256:
         return False
+    if gemm_regs(cfg) * max(1, 64 * wn * wk // 256) > 512:
+        return False
     return gemm_lds_bytes(cfg) <= 160 * 1024
 
 
@@ -334,7 +345,9 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
         if bm >= 2 * M and bm > 32:
             continue
         choice = (bm, wn)
-        if -(-N // (32 * wn)) * -(-M // bm) >= NUM_CUS:
+        # measured on MI355X: a 128-row tile on 160 of the 256 CUs (N = 10240, M = 256) beats
+        # 64-row tiles on all of them (84 vs 108 us), on 128 CUs (N = 8192) it does not (67 vs 57 us)
+        if -(-N // (32 * wn)) * -(-M // bm) >= (0.6 if bm == 128 else 1.0) * NUM_CUS:
             break
     bm, wn = choice
     blocks = -(-N // (32 * wn)) * -(-M // bm)
@@ -343,7 +356,18 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     wk = max(1, 8 // wn) if blocks < 2 * NUM_CUS else 1
     nsup = K // (1024 // nbits)
     wk = max(1, min(wk, nsup))
-    cfg = {"BM": bm, "NT32": 1, "WN": wn, "WK": wk, "PA": 2}
+    pa = 4
+    while not gemm_valid({"BM": bm, "NT32": 1, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
+        if pa == 4:
+            pa = 2                                    # a shallower activation ring frees registers
+        elif wk > 1:
+            wk, pa = wk // 2, 4
+        else:
+            break
+    # two 32-row tiles per wave halve the activation reads per MFMA; worth it while the blocks
+    # still outnumber the CUs comfortably
+    nt32 = 2 if (bm == 128 and wn == 4 and blocks >= 3 * NUM_CUS) else 1
+    cfg = {"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}
     cfg.update(pins)
     return cfg
 
@@ -364,7 +388,7 @@ def gemm_candidates(M, N, K, nbits, group_size):
         for nt32 in (1, 2):
             for wn in (2, 4):
                 for wk in (1, 2, 4):
-                    for pa in (2, 4):
+                    for pa in (2, 4, 8):
                         add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})
     return out
 

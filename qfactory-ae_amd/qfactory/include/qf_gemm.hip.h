@@ -21,14 +21,28 @@
 //     share a row: fully coalesced), two supers ahead of use, into a buffer private to the wave
 //     (no block barrier on that path); a lane then picks its 4*NBITS bytes per K-iteration with
 //     one LDS read.  The scales and zero-points of a super are loaded with it and stay in registers.
-//   * Activations go global -> register ring -> LDS tile (double-buffered per group, one block
+//   * Activations go global -> register ring -> LDS tile (three buffers per group, one block
 //     barrier per K-iteration) and are read in fragment order with ds_read_b128 (rows padded by
-//     16 bytes: conflict-free).  Weights are MFMA source A (rows = n), activations source B
-//     (columns = m): a lane ends with groups of four consecutive n of one m -> 8-byte stores.
+//     16 bytes: conflict-free) one whole iteration before their MFMAs, so that no wave waits on
+//     LDS right behind a barrier (measured: the barrier-then-read stall was half of the kernel).
+//     Weights are MFMA source A (rows = n), activations source B (columns = m): a lane ends with
+//     groups of four consecutive n of one m -> 8-byte stores.
 #pragma once
 
 #include <cstdio>
 #include "qf_dequant.hip.h"
+
+// Timing experiments (results are wrong when non-zero): bit 0 skips the dequantisation arithmetic,
+// bit 1 the activation fragment reads, bit 2 the MFMAs, bit 3 the per-iteration barrier, bit 4 the
+// global activation loads, bit 5 the global weight / scale / zero loads.
+#ifndef QF_GEMM_EXPERIMENT
+#define QF_GEMM_EXPERIMENT 0
+#endif
+
+// 1: XCD-aware block -> tile map (see the kernel), 0: plain blockIdx order.
+#ifndef QF_GEMM_XCD_MAP
+#define QF_GEMM_XCD_MAP 0
+#endif
 
 namespace qf {
 
@@ -64,7 +78,8 @@ struct GemmCfg {
     static constexpr int G = K / GS;
     static constexpr int ZRB = G * NBITS / 8;
     static constexpr int GRID_X = (N + BN - 1) / BN;
-    static constexpr size_t LDS_A = (size_t)WK * 2 * BM * PITCH * 2;
+    static constexpr int NBUF = 3;                             // activation tiles in LDS per group
+    static constexpr size_t LDS_A = (size_t)WK * NBUF * BM * PITCH * 2;
     static constexpr size_t LDS_W = (size_t)WK * WN * TN * WPP;
     static constexpr size_t LDS_RED = WK > 1 ? (size_t)(WK - 1) * BM * BN * 4 : 0;
     static constexpr size_t LDS_FRONT = LDS_A > LDS_RED ? LDS_A : LDS_RED;
@@ -84,17 +99,26 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // wave-uniform indices live in scalar registers: every global address below is then a scalar
+    // base (advanced with scalar adds) plus a 32-bit per-lane offset computed once
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave % WN, grp = wave / WN;
     const int tg = tid - grp * C::TG;                          // thread index inside the group
     const int li = lane & 31, kb = lane >> 5;
 
     // activation tiles live at the start of LDS (the final cross-group sum reuses that space)
-    uint16_t* as = reinterpret_cast<uint16_t*>(smem) + (size_t)grp * 2 * BM * PITCH;    // [2][BM][PITCH]
+    uint16_t* as = reinterpret_cast<uint16_t*>(smem) + (size_t)grp * C::NBUF * BM * PITCH;   // [NBUF][BM][PITCH]
     uint8_t* wp = smem + C::LDS_FRONT + (size_t)wave * TN * WPP;                         // [TN][WPP]
 
-    const int n_blk = blockIdx.x * C::BN;
-    const int m_blk = blockIdx.y * BM;
+    // Block -> tile map.  The hardware deals workgroups round-robin to the 8 XCDs (linear id % 8),
+    // each with its own L2.  Tiles are numbered M-slab by M-slab and every XCD gets a contiguous
+    // range of that numbering, so one XCD re-reads one (or few) BM-row activation slab(s), which
+    // stay in its L2, instead of all of them.
+    const int linear = blockIdx.x + gridDim.x * blockIdx.y;
+    const int total = gridDim.x * gridDim.y;
+    const int tile = (QF_GEMM_XCD_MAP && total % 8 == 0) ? (linear % 8) * (total / 8) + linear / 8 : linear;
+    const int n_blk = (tile % C::GRID_X) * C::BN;
+    const int m_blk = (tile / C::GRID_X) * BM;
     const int n_wave = n_blk + wn * TN;
 
     // K offset of the group's iteration `it`: supers are dealt round-robin to the groups; a group
@@ -106,15 +130,19 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 
     // ---- activations: UA 16-byte units per thread and iteration, register ring of depth PA ----
     struct AStage { u32x4 a[UA]; };
-    auto load_a = [&](AStage& st, int it) {
-        const int k0 = k_of(it);
+    uint32_t a_off[UA];                                        // byte offset of this thread's units inside the slab
 #pragma unroll
-        for (int p = 0; p < UA; p++) {
-            const int u = tg + p * C::TG;
-            const int row = u / (BK / 8), col = (u % (BK / 8)) * 8;
-            const int m = min(m_blk + row, m_total - 1);
-            st.a[p] = *reinterpret_cast<const u32x4*>(A + (size_t)m * C::K + k0 + col);
-        }
+    for (int p = 0; p < UA; p++) {
+        const int u = tg + p * C::TG;
+        const int row = min(u / (BK / 8), m_total - 1 - m_blk);   // rows past the end re-read the last one
+        a_off[p] = ((uint32_t)row * C::K + (u % (BK / 8)) * 8) * 2u;
+    }
+    const uint8_t* a_slab = reinterpret_cast<const uint8_t*>(A + (size_t)m_blk * C::K);
+    auto load_a = [&](AStage& st, int it) {
+        const uint8_t* base = a_slab + (size_t)k_of(it) * 2;
+#pragma unroll
+        for (int p = 0; p < UA; p++)
+            if (!(QF_GEMM_EXPERIMENT & 16)) st.a[p] = *reinterpret_cast<const u32x4*>(base + a_off[p]);
     };
     auto store_a = [&](const AStage& st, int buf) {
 #pragma unroll
@@ -128,22 +156,39 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     // ---- one super of this wave's TN weight rows: packed fields, scales, zero-points ----
     struct Quant { uint32_t s[NT32][SREGS]; uint32_t z[NT32]; };
     struct WStage { u32x4 w[UPS]; Quant q; };
+    uint32_t w_off[UPS], s_off[NT32], z_off[NT32];             // per-lane byte offsets from the wave's first row
+    const int n_base = min(n_wave, C::N - 1);                  // a wave wholly past the last row re-reads it
+#pragma unroll
+    for (int p = 0; p < UPS; p++) {
+        const int u = lane + 64 * p;
+        w_off[p] = (uint32_t)min(u / 8, C::N - 1 - n_base) * C::RB + (u % 8) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < NT32; j++) {
+        const uint32_t row = (uint32_t)min(j * 32 + li, C::N - 1 - n_base);
+        s_off[j] = row * C::G * 2u;
+        z_off[j] = row * C::ZRB;
+    }
+    const uint8_t* w_rows = W + (size_t)n_base * C::RB;
+    const uint8_t* s_rows = reinterpret_cast<const uint8_t*>(S + (size_t)n_base * C::G);
+    const uint8_t* z_rows = Zp + (size_t)n_base * C::ZRB;
     auto load_super = [&](WStage& st, int sup_local) {
+        if (QF_GEMM_EXPERIMENT & 32) return;
         const int sup = min(sup_local * WK + grp, C::NSUP - 1);
+        const uint8_t* wb = w_rows + (size_t)sup * 128;
 #pragma unroll
         for (int p = 0; p < UPS; p++) {
-            const int u = lane + 64 * p;
-            const int n = min(n_wave + u / 8, C::N - 1);
-            const uint8_t* src = W + (size_t)n * C::RB + (size_t)sup * 128 + (u % 8) * 16;
+            const uint8_t* src = wb + w_off[p];
             st.w[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
         }
         const int g0 = sup * C::SUPK / C::GS;                  // first group of the super
+        const uint8_t* sb = s_rows + (size_t)g0 * 2;
+        const uint8_t* zb = z_rows + (g0 * C::NBITS) / 8;
 #pragma unroll
         for (int j = 0; j < NT32; j++) {
-            const int n = min(n_wave + j * 32 + li, C::N - 1);
-            const uint16_t* sp = S + (size_t)n * C::G + g0;
+            const uint8_t* sp = sb + s_off[j];
             if constexpr (NGS == 1) {
-                st.q.s[j][0] = *sp;
+                st.q.s[j][0] = *reinterpret_cast<const uint16_t*>(sp);
             } else if constexpr (NGS == 2) {
                 st.q.s[j][0] = *reinterpret_cast<const uint32_t*>(sp);
             } else if constexpr (NGS == 4) {
@@ -155,7 +200,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             }
             st.q.z[j] = 0;
             if constexpr (!C::SYM) {
-                const uint8_t* zp = Zp + (size_t)n * C::ZRB + (g0 * C::NBITS) / 8;
+                const uint8_t* zp = zb + z_off[j];
                 if constexpr (C::ZBITS >= 32) st.q.z[j] = *reinterpret_cast<const uint32_t*>(zp);
                 else if constexpr (C::ZBITS == 16) st.q.z[j] = *reinterpret_cast<const uint16_t*>(zp);
                 else if constexpr (C::ZBITS == 8) st.q.z[j] = *zp;
@@ -215,20 +260,36 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[j][i][v] = 0.0f;
 
-    // activation fragment of k-step ks: row li of tile i, columns 32*kb + 8*ks .. + 7
+    // activation fragments of one tile: k-step ks of 32-row block i is row li, columns 32*kb + 8*ks .. + 7
     const uint16_t* a_frag_base = as + (size_t)li * PITCH + 32 * kb;
+    struct AFrags { f16x8 f[MT32][4]; };
+    auto read_frags = [&](AFrags& fr, int buf) {
+#pragma unroll
+        for (int i = 0; i < MT32; i++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                if (QF_GEMM_EXPERIMENT & 2) fr.f[i][ks] = __builtin_bit_cast(f16x8, u32x4{(uint32_t)buf, 1u, 2u, 3u});
+                else fr.f[i][ks] = *reinterpret_cast<const f16x8*>(a_frag_base + ((size_t)buf * BM + i * 32) * PITCH + ks * 8);
+            }
+    };
 
-    AStage ringA[C::PA];
+    AStage ringA[C::PA];        // slot t % PA holds activation tile t on its way to LDS
     WStage ringW[2];
     Packed cur, nxt;
     Quant qcur;
+    AFrags fcur, fnxt;
 
-    // One K-iteration; s = it % (2*SUP) is a compile-time constant at every call site.
-    auto iteration = [&](int it, int s) {
-        const int buf = it & 1;
+    // One K-iteration; s = it % (2*SUP) is a compile-time constant at every call site; b1 and b2
+    // are the LDS buffers (of NBUF = 3) of tiles it+1 and it+2.
+    //   * the fragments of tile it+1 (complete in LDS since the last barrier) are fetched now and
+    //     used in the next iteration: no wave waits on LDS right after a barrier;
+    //   * tile it+2 goes from its ring slot to LDS, and the slot takes the load of tile it+2+PA;
+    //   * the MFMAs of tile it run on registers filled one iteration ago, interleaved with the
+    //     dequantisation of their weight fragments.
+    auto iteration = [&](int it, int s, int b1, int b2) {
         const int q = s % SUP, pslot = (s / SUP) & 1;
         const int P = it / SUP;                                 // super index inside the group
-        load_a(ringA[s % C::PA], min(it + C::PA, C::ITERS - 1));
+        read_frags(fnxt, b1);
         // every read of the current super has been issued one iteration ago: the next super
         // (loaded two supers back) takes its place in LDS
         if (q == SUP - 1) store_super(ringW[pslot ^ 1]);
@@ -237,14 +298,13 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         if (live) {
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                f16x8 wf[NT32], af[MT32];
-#pragma unroll
-                for (int i = 0; i < MT32; i++)
-                    af[i] = *reinterpret_cast<const f16x8*>(a_frag_base + ((size_t)buf * BM + i * 32) * PITCH + ks * 8);
+                f16x8 wf[NT32];
 #pragma unroll
                 for (int j = 0; j < NT32; j++) {
                     const QConst qc = qconst_of(qcur, j, q);
-                    if constexpr (C::NBITS == 8) {
+                    if constexpr ((QF_GEMM_EXPERIMENT & 1) != 0) {
+                        wf[j] = __builtin_bit_cast(f16x8, u32x4{cur.w[j][0], cur.w[j][1], cur.w[j][2], cur.w[j][3] + (uint32_t)ks});
+                    } else if constexpr (C::NBITS == 8) {
                         const int h = 4 * (ks / 2);
                         const uint32_t w4[4] = {cur.w[j][h], cur.w[j][h + 1], cur.w[j][h + 2], cur.w[j][h + 3]};
                         wf[j] = DequantStep<8>::run(w4, ks % 2, qc);
@@ -257,20 +317,23 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 for (int j = 0; j < NT32; j++)
 #pragma unroll
                     for (int i = 0; i < MT32; i++)
-                        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[j][i], 0, 0, 0);
+                        if (QF_GEMM_EXPERIMENT & 4) acc[j][i][ks] += (float)wf[j][0] * (float)fcur.f[i][ks][0];
+                        else acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], fcur.f[i][ks], acc[j][i], 0, 0, 0);
             }
         }
-        store_a(ringA[(s + 1) % C::PA], buf ^ 1);
+        store_a(ringA[(s + 2) % C::PA], b2);
+        load_a(ringA[(s + 2) % C::PA], min(it + 2 + C::PA, C::ITERS - 1));
         cur = nxt;
+        fcur = fnxt;
         if (q == SUP - 1) {
             // its register slot goes to the super two after it
             qcur = ringW[pslot ^ 1].q;
             load_super(ringW[pslot ^ 1], P + 3);
         }
-        __syncthreads();
+        if (!(QF_GEMM_EXPERIMENT & 8)) __syncthreads();
     };
 
-    // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 in flight ----
+    // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA+1 in flight, tiles 0 and 1 in LDS ----
     load_super(ringW[0], 0);
     load_super(ringW[1], 1);
 #pragma unroll
@@ -280,13 +343,22 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     load_super(ringW[0], 2);
     read_packed(cur, 0);
     store_a(ringA[0], 0);
+    store_a(ringA[1 % C::PA], 1);
+    load_a(ringA[0], min(C::PA, C::ITERS - 1));
+    load_a(ringA[1 % C::PA], min(C::PA + 1, C::ITERS - 1));
     __syncthreads();
+    read_frags(fcur, 0);
 
+    int b1 = 1, b2 = 2;
 #pragma unroll 1
     for (int it0 = 0; it0 < C::ITERS; it0 += 2 * SUP) {
 #pragma unroll
         for (int s = 0; s < 2 * SUP; s++)
-            if (it0 + s < C::ITERS) iteration(it0 + s, s);
+            if (it0 + s < C::ITERS) {
+                iteration(it0 + s, s, b1, b2);
+                b1 = b2;
+                b2 = b2 == C::NBUF - 1 ? 0 : b2 + 1;
+            }
     }
 
     // ---- the groups' partial sums meet in LDS (the activation tiles are no longer needed) ----
