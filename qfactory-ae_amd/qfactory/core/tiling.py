@@ -97,14 +97,15 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
     else:
         it = -(-(K // elements_per_chunk(nbits, vb)) // (64 * wk))
     if u is None:
-        # keep about 8 x 16 bytes of weight in flight per lane and stage, U*MT a power of two <= 64
-        u = max(1, min(8 // it if it <= 8 else 1, 64 // mt, 8))
+        # four rows (4 x 16 bytes per lane) in flight per wave and no second stage measured best on
+        # MI355X once the kernel's address arithmetic had moved to scalar registers: many small
+        # waves (61 registers, 8 per SIMD) beat fewer waves with deeper stages
+        u = max(1, min(4 // it if it <= 4 else 1, 64 // mt, 4))
         u = _pow2_floor(u)
     if wn is None:
         wn = 2 if wk * 2 <= 16 else 1                 # two teams per block measured best on MI355X
     if steps is None:
-        # a team amortises its activation load over about 8 rows
-        steps = max(1, 8 // u)
+        steps = 1
     return {"MT": mt, "WK": wk, "WN": wn, "U": u, "STEPS": steps, "VB": vb}
 
 

@@ -86,7 +86,9 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // wave-uniform indices in scalar registers: row pointers are then scalar bases advanced with
+    // scalar adds, and every load is base + one 32-bit lane offset (no 64-bit vector arithmetic)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wk = wave % WK;
     const int team = wave / WK;
     const int tt = wk * 64 + lane;
@@ -119,13 +121,15 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         for (int u = 0; u < U; u++) {
             const int row = min(row_base + step * U + u, C::N - 1);
             const uint8_t* wrow = W + (size_t)row * C::RB;
+            const uint8_t* srow = reinterpret_cast<const uint8_t*>(S) + (size_t)row * C::G * 2;
+            const uint8_t* zrow = Zp + (size_t)row * C::ZRB;
 #pragma unroll
             for (int it = 0; it < IT; it++) {
-                load_words<NW, C::NT_B>(wrow + coff[it], st.w[u][it]);
-                if constexpr (NWH > 0) load_words<NWH, C::NT_B>(wrow + C::HI_OFF + coff[it] / 2, st.h[u][it]);
+                load_words<NW, C::NT_B>(wrow + (uint32_t)coff[it], st.w[u][it]);
+                if constexpr (NWH > 0) load_words<NWH, C::NT_B>(wrow + (uint32_t)(C::HI_OFF + coff[it] / 2), st.h[u][it]);
                 if constexpr (C::QPARAM) {
-                    st.s[u][it] = S[(size_t)row * C::G + goff[it]];
-                    if constexpr (!C::SYM) st.z[u][it] = Zp[(size_t)row * C::ZRB + goff[it] / P8];
+                    st.s[u][it] = *reinterpret_cast<const uint16_t*>(srow + (uint32_t)(goff[it] * 2));
+                    if constexpr (!C::SYM) st.z[u][it] = zrow[(uint32_t)(goff[it] / P8)];
                 }
             }
         }
@@ -159,8 +163,9 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 for (int j = 0; j < LW; j++) {
                     const uint32_t val = cvalid[it] ? tmp[j] : 0u;
                     a[m][it][r + j] = val;
-                    const f16x2 h = as_f16x2(val);
-                    cls_sum[D::cls((r + j) % PAIRS)] += (float)h.x + (float)h.y;
+                    // sum of the pair in one instruction: dot2 with (1, 1)
+                    cls_sum[D::cls((r + j) % PAIRS)] = __builtin_amdgcn_fdot2(
+                        as_f16x2(val), as_f16x2(0x3C003C00u), cls_sum[D::cls((r + j) % PAIRS)], false);
                 }
             }
             float c1v = 0.0f, sav = 0.0f;
