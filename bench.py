@@ -165,7 +165,10 @@ COPY_BYTES = 64 << 20
 # and --pmc WRITE_SIZE over `bench.py --counter-pass`, each scaled by what the same counter reads
 # for the 64 MiB stream copy of that run (which moves COPY_BYTES each way).  Keyed by the kernel's
 # description so that a different specialisation reports null instead of a stale figure.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # FETCH_SIZE 22938.4 KiB x (65536 / 32807.5, the copy's read of 64 MiB) + WRITE_SIZE 86 KiB x (65536 / 65536)
+    "regime=gemv M=1 N=22016 K=4096 NBITS=4 GS=128 SYM=0 decode=deferred nt_b=1 MT=1 STEPS=1 U=4 VB=16 WK=2 WN=2": 47009000,
+}
 
 
 def counter_pass(layers, acts, reps=5):
