@@ -102,7 +102,7 @@ def kernel_event_time_us(lins, x, reps=64):
     def launches():
         for i in range(reps):
             lin, out = lins[i % len(lins)], outs[i % len(lins)]
-            rc = lin.func(x, lin.w, out, lin.s, lin.z)
+            rc = lin.func(x, lin.w, out, lin.s, lin.z) if lin.z is not None else lin.func(x, lin.w, out, lin.s)
             assert rc == 0
 
     launches()
@@ -186,6 +186,54 @@ def counter_pass(layers, acts, reps=5):
     log(f"[bench] counter pass: {reps} launches of each kernel and of a {COPY_BYTES} byte stream copy")
 
 
+def _timed_layers(M, N, K, nbits, sym, total_bytes=600e6):
+    """A few QLinear copies of one problem with random packed tensors (enough bytes to defeat the caches)."""
+    import torch
+    from qfactory import QLinear
+    flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
+    g = torch.Generator(device="cuda").manual_seed(2)
+    n_copies = max(2, min(8, int(total_bytes // (N * K * nbits // 8))))
+    lins = []
+    for _ in range(n_copies):
+        lin = QLinear.empty(M, K, N, nbits, GS, sym=sym, compile_flags=flags)
+        lin.w.copy_(torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=g))
+        lin.s.copy_((torch.rand(lin.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
+        if not sym:
+            lin.z.copy_(torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=g))
+        lins.append(lin)
+    x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
+    return lins, x
+
+
+def small_m_report():
+    """BASELINE.json configs[1] at M in {4, 16} and configs[2] (N = K = 8192, M in {1, 16}, 2/3/4/8-bit,
+    symmetric and asymmetric): per shape microseconds and the fraction of the 8 TB/s HBM roofline."""
+    import torch
+    report = []
+
+    def one(tag, M, N, K, nbits, sym):
+        lins, x = _timed_layers(M, N, K, nbits, sym)
+        us = kernel_event_time_us(lins, x, reps=8 * len(lins))
+        b = algorithmic_bytes(M, N, K, nbits, GS, sym)
+        rec = {"config": tag, "M": M, "N": N, "K": K, "bits": nbits, "sym": sym, "us": round(us, 3),
+               "GB/s": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
+               "TFLOP/s": round(2.0 * M * N * K / us / 1e6, 2), "kernel": lins[0].func_for(M).runtime.description}
+        report.append(rec)
+        log(f"[bench] {tag} M={M:3d} N={N:6d} K={K:6d} b={nbits} {'sym ' if sym else 'asym'} {us:8.2f} us "
+            f"{rec['GB/s']:7.1f} GB/s {100 * rec['hbm_frac']:5.1f}% of HBM peak")
+        del lins
+        torch.cuda.empty_cache()
+
+    for M in (4, 16):
+        for name, N, K in SHAPES:
+            one("configs[1]", M, N, K, NBITS, False)
+    for M in (1, 16):
+        for nbits in (2, 3, 4, 8):
+            for sym in (False, True):
+                one("configs[2]", M, 8192, 8192, nbits, sym)
+    return report
+
+
 def cpu_baseline(budget_s=15.0):
     """torch-CPU dequant + fp32 matmul over the same four shapes, bounded to about `budget_s`."""
     import torch
@@ -227,6 +275,8 @@ def main():
     ap.add_argument("--layers", type=int, default=8, help="distinct resident weight copies cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=256 GEMM report")
+    ap.add_argument("--small-m", action="store_true",
+                    help="also report configs[1] at M = 4, 16 and the configs[2] bit-width sweep (not part of `value`)")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
     ap.add_argument("--counter-pass", action="store_true",
                     help="only launch each of the four kernels (cold weights) and a 64 MiB stream copy a few times, "
@@ -313,6 +363,8 @@ def main():
     }
     if not args.no_gemm:
         result["gemm_m256"] = {"peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS, "shapes": gemm_report(256)}
+    if args.small_m:
+        result["small_m"] = small_m_report()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
         log(f"[bench] cpu baseline: {result['cpu_baseline']}")

@@ -31,7 +31,9 @@ def regime_for(M, K=None, nbits=None, group_size=None):
         return "mgemv"
     if M <= GEMV_MAX_M:
         return "gemv"
-    if M > MGEMV_MAX_M and gemm_supported(K, nbits, group_size):
+    # above 32 rows, or when the A-stationary kernel cannot hold the activations of this K in
+    # registers: the LDS-staged GEMM (with a 32-row tile for small M)
+    if gemm_supported(K, nbits, group_size):
         return "gemm"
     return "mfma"
 
@@ -342,7 +344,7 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     # the largest block tile (BM x 32*WN) that still gives every CU a block; when even the
     # smallest leaves CUs idle, the smallest
     choice = None
-    for bm, wn in ((128, 4), (64, 4), (64, 2), (32, 4), (32, 2)):
+    for bm, wn in ((128, 4), (64, 4), (64, 2), (32, 4), (32, 2), (32, 1)):
         if bm >= 2 * M and bm > 32:
             continue
         choice = (bm, wn)
@@ -387,8 +389,8 @@ def gemm_candidates(M, N, K, nbits, group_size):
         if bm >= 2 * M and bm > 32:
             continue
         for nt32 in (1, 2):
-            for wn in (2, 4):
-                for wk in (1, 2, 4):
+            for wn in (1, 2, 4):
+                for wk in (1, 2, 4, 8):
                     for pa in (2, 4, 8):
                         add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})
     return out
