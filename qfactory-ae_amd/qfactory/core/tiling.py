@@ -102,7 +102,9 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
         # four rows (4 x 16 bytes per lane) in flight per wave and no second stage measured best on
         # MI355X once the kernel's address arithmetic had moved to scalar registers: many small
         # waves (61 registers, 8 per SIMD) beat fewer waves with deeper stages
-        u = max(1, min(4 // it if it <= 4 else 1, 64 // mt, 4))
+        # (2- and 3-bit rows are short in bytes and heavy in decode work: eight rows measured best)
+        rows = 8 if nbits <= 3 else 4
+        u = max(1, min(rows // it if it <= rows else 1, 64 // mt, rows))
         u = _pow2_floor(u)
     if wn is None:
         wn = 2 if wk * 2 <= 16 else 1                 # two teams per block measured best on MI355X
