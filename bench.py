@@ -128,6 +128,27 @@ def kernel_event_time_us(lins, x, reps=64):
     return best[len(best) // 2]
 
 
+def dense_fp16_time_us(M, N, K, total_bytes=600e6):
+    """The vendor library's dense fp16 GEMM of the same shape (torch.matmul on hipBLASLt / rocBLAS), cold
+    weights: the comparison the reference's own evaluation makes against cuBLAS
+    (qfactory/testing.py:36-41).  A reported yardstick, not part of the path."""
+    import torch
+    n = max(2, min(8, int(total_bytes // (N * K * 2))))
+    ws = [torch.randn(N, K, device="cuda", dtype=torch.float16) for _ in range(n)]
+    x = torch.randn(M, K, device="cuda", dtype=torch.float16)
+    for w in ws:
+        torch.matmul(x, w.T)
+    torch.cuda.synchronize()
+    reps = 4 * n
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(reps):
+        torch.matmul(x, ws[i % n].T)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
 def gemm_report(M=256, copies_bytes=600e6):
     """BASELINE.json configs[3] at M = 256: W4A16 g128 GEMM on Llama-3-70B-style shapes, per shape
     microseconds, TFLOP/s and the fraction of the dense fp16 MFMA peak."""
@@ -147,15 +168,20 @@ def gemm_report(M=256, copies_bytes=600e6):
             lins.append(lin)
         x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
         us = kernel_event_time_us(lins, x, reps=2 * n_copies)
+        description = lins[0].func.runtime.description
+        del lins
+        torch.cuda.empty_cache()
+        dense_us = dense_fp16_time_us(M, N, K)
         flops = 2.0 * M * N * K
         rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1),
                "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
-               "GB/s": round(algorithmic_bytes(M, N, K) / us / 1e3, 1), "kernel": lins[0].func.runtime.description}
+               "GB/s": round(algorithmic_bytes(M, N, K) / us / 1e3, 1),
+               "dense_fp16_us": round(dense_us, 2), "speedup_over_dense_fp16": round(dense_us / us, 3),
+               "kernel": description}
         report.append(rec)
         log(f"[bench] GEMM M={M} {name:11s} N={N:6d} K={K:6d} {us:8.2f} us {rec['TFLOP/s']:7.1f} TFLOP/s "
-            f"{100 * rec['mfma_frac']:5.1f}% of fp16 MFMA peak")
-        del lins
-        torch.cuda.empty_cache()
+            f"{100 * rec['mfma_frac']:5.1f}% of fp16 MFMA peak; dense fp16 torch.matmul {dense_us:8.2f} us "
+            f"(x{rec['speedup_over_dense_fp16']:.2f})")
     return report
 
 
@@ -365,6 +391,8 @@ def main():
         result["gemm_m256"] = {"peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS, "shapes": gemm_report(256)}
     if args.small_m:
         result["small_m"] = small_m_report()
+        if not args.no_gemm:
+            result["gemm_m32_m64_m128"] = [rec for M in (32, 64, 128) for rec in gemm_report(M)]
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
         log(f"[bench] cpu baseline: {result['cpu_baseline']}")

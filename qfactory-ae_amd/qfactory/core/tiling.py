@@ -343,35 +343,39 @@ def gemm_supported(K, nbits, group_size):
 
 
 def gemm_tiling(M, N, K, nbits, group_size, **pins):
-    # the largest block tile (BM x 32*WN) that still gives every CU a block; when even the
-    # smallest leaves CUs idle, the smallest
-    choice = None
-    for bm, wn in ((128, 4), (64, 4), (64, 2), (32, 4), (32, 2), (32, 1)):
+    """Default GEMM tiling from a small cost model fitted to on-device sweeps: a launch takes
+    ceil(blocks / CUs) rounds of one tile's work, and a tile costs its area plus a fixed overhead
+    (pipeline fill, reduction, barriers) worth about 2048 outputs.  It reproduces the measured
+    winners: 64 x 128 tiles on 8192-wide, 128 x 128 on 10240-wide (160 tiles in one round beat 320
+    in two) and 128 x 256 on 57344-wide layers at M = 256; 32 x 32 ... 64 x 64 tiles for M <= 128."""
+    import math
+    best = None
+    for bm in (128, 64, 32):
         if bm >= 2 * M and bm > 32:
             continue
-        choice = (bm, wn)
-        # measured on MI355X: a 128-row tile on 160 of the 256 CUs (N = 10240, M = 256) beats
-        # 64-row tiles on all of them (84 vs 108 us), on 128 CUs (N = 8192) it does not (67 vs 57 us)
-        if -(-N // (32 * wn)) * -(-M // bm) >= (0.6 if bm == 128 else 1.0) * NUM_CUS:
-            break
-    bm, wn = choice
-    blocks = -(-N // (32 * wn)) * -(-M // bm)
+        for wn in (4, 2, 1):
+            for nt32 in ((1, 2) if (bm, wn) == (128, 4) else (1,)):
+                bn = 32 * wn * nt32
+                blocks = -(-N // bn) * -(-M // bm)
+                rounds = -(-blocks // NUM_CUS)
+                cost = rounds * (bm * bn + 2048)
+                key = (cost, abs(math.log2(bm / bn)), -bn)
+                if best is None or key < best[0]:
+                    best = (key, bm, wn, nt32, blocks)
+    _, bm, wn, nt32, blocks = best
     # with at most one block per CU the K axis is split over wave groups inside the block, so
     # that every SIMD still holds two waves (one dequantises while the other multiplies)
     wk = max(1, 8 // wn) if blocks < 2 * NUM_CUS else 1
     nsup = K // (1024 // nbits)
     wk = max(1, min(wk, nsup))
     pa = 4
-    while not gemm_valid({"BM": bm, "NT32": 1, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
+    while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
         if pa == 4:
             pa = 2                                    # a shallower activation ring frees registers
         elif wk > 1:
             wk, pa = wk // 2, 4
         else:
             break
-    # two 32-row tiles per wave halve the activation reads per MFMA; worth it while the blocks
-    # still outnumber the CUs comfortably
-    nt32 = 2 if (bm == 128 and wn == 4 and blocks >= 3 * NUM_CUS) else 1
     cfg = {"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}
     cfg.update(pins)
     return cfg
