@@ -309,7 +309,8 @@ def gemm_regs(cfg):
     A SIMD has 512 per lane to share between the waves a block puts on it (spills are ruinous)."""
     mt32, nt32 = cfg["BM"] // 32, cfg["NT32"]
     ua = max(1, cfg["BM"] * 8 // (64 * cfg["WN"]))
-    return mt32 * nt32 * 16 + 2 * mt32 * 16 + 2 * nt32 * 20 + cfg["PA"] * ua * 4 + 80
+    frag_sets = 2 if mt32 <= 4 else 0.25               # tall tiles keep one k-step of fragments, not two tiles
+    return int(mt32 * nt32 * 16 + frag_sets * mt32 * 16 + 2 * nt32 * 20 + cfg["PA"] * ua * 4 + 80)
 
 
 def gemm_valid(cfg, K, nbits, group_size):
@@ -358,6 +359,8 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
                 bn = 32 * wn * nt32
                 blocks = -(-N // bn) * -(-M // bm)
                 rounds = -(-blocks // NUM_CUS)
+                # (256-row tiles, which dequantise every weight once, measured no faster: the
+                # kernel is bound by load waits, not by the dequantisation)
                 cost = rounds * (bm * bn + 2048)
                 key = (cost, abs(math.log2(bm / bn)), -bn)
                 if best is None or key < best[0]:
@@ -365,7 +368,7 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     _, bm, wn, nt32, blocks = best
     # with at most one block per CU the K axis is split over wave groups inside the block, so
     # that every SIMD still holds two waves (one dequantises while the other multiplies)
-    wk = max(1, 8 // wn) if blocks < 2 * NUM_CUS else 1
+    wk = max(1, 8 // wn) if blocks <= NUM_CUS else 1
     nsup = K // (1024 // nbits)
     wk = max(1, min(wk, nsup))
     pa = 4

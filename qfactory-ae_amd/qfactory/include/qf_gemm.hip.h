@@ -79,6 +79,9 @@ struct GemmCfg {
     static constexpr int ZRB = G * NBITS / 8;
     static constexpr int GRID_X = (N + BN - 1) / BN;
     static constexpr int NBUF = 3;                             // activation tiles in LDS per group
+    // fetch the activation fragments of tile it+1 during iteration it (a second register set of
+    // 16 * MT32 registers); tall tiles read each fragment just before its MFMAs instead
+    static constexpr bool PREFETCH_A = MT32 <= 4;
     static constexpr size_t LDS_A = (size_t)WK * NBUF * BM * PITCH * 2;
     static constexpr size_t LDS_W = (size_t)WK * WN * TN * WPP;
     static constexpr size_t LDS_RED = WK > 1 ? (size_t)(WK - 1) * BM * BN * 4 : 0;
@@ -286,10 +289,10 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     //   * tile it+2 goes from its ring slot to LDS, and the slot takes the load of tile it+2+PA;
     //   * the MFMAs of tile it run on registers filled one iteration ago, interleaved with the
     //     dequantisation of their weight fragments.
-    auto iteration = [&](int it, int s, int b1, int b2) {
+    auto iteration = [&](int it, int s, int b0, int b1, int b2) {
         const int q = s % SUP, pslot = (s / SUP) & 1;
         const int P = it / SUP;                                 // super index inside the group
-        read_frags(fnxt, b1);
+        if constexpr (C::PREFETCH_A) read_frags(fnxt, b1);
         // every read of the current super has been issued one iteration ago: the next super
         // (loaded two supers back) takes its place in LDS
         if (q == SUP - 1) store_super(ringW[pslot ^ 1]);
@@ -298,7 +301,13 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         if (live) {
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                f16x8 wf[NT32];
+                f16x8 wf[NT32], af[MT32];
+#pragma unroll
+                for (int i = 0; i < MT32; i++) {
+                    if constexpr (C::PREFETCH_A) af[i] = fcur.f[i][ks];
+                    else if (QF_GEMM_EXPERIMENT & 2) af[i] = __builtin_bit_cast(f16x8, u32x4{(uint32_t)b0, 1u, 2u, 3u});
+                    else af[i] = *reinterpret_cast<const f16x8*>(a_frag_base + ((size_t)b0 * BM + i * 32) * PITCH + ks * 8);
+                }
 #pragma unroll
                 for (int j = 0; j < NT32; j++) {
                     const QConst qc = qconst_of(qcur, j, q);
@@ -317,14 +326,14 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 for (int j = 0; j < NT32; j++)
 #pragma unroll
                     for (int i = 0; i < MT32; i++)
-                        if (QF_GEMM_EXPERIMENT & 4) acc[j][i][ks] += (float)wf[j][0] * (float)fcur.f[i][ks][0];
-                        else acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], fcur.f[i][ks], acc[j][i], 0, 0, 0);
+                        if (QF_GEMM_EXPERIMENT & 4) acc[j][i][ks] += (float)wf[j][0] * (float)af[i][0];
+                        else acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[j][i], 0, 0, 0);
             }
         }
         store_a(ringA[(s + 2) % C::PA], b2);
         load_a(ringA[(s + 2) % C::PA], min(it + 2 + C::PA, C::ITERS - 1));
         cur = nxt;
-        fcur = fnxt;
+        if constexpr (C::PREFETCH_A) fcur = fnxt;
         if (q == SUP - 1) {
             // its register slot goes to the super two after it
             qcur = ringW[pslot ^ 1].q;
@@ -347,15 +356,16 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     load_a(ringA[0], min(C::PA, C::ITERS - 1));
     load_a(ringA[1 % C::PA], min(C::PA + 1, C::ITERS - 1));
     __syncthreads();
-    read_frags(fcur, 0);
+    if constexpr (C::PREFETCH_A) read_frags(fcur, 0);
 
-    int b1 = 1, b2 = 2;
+    int b0 = 0, b1 = 1, b2 = 2;
 #pragma unroll 1
     for (int it0 = 0; it0 < C::ITERS; it0 += 2 * SUP) {
 #pragma unroll
         for (int s = 0; s < 2 * SUP; s++)
             if (it0 + s < C::ITERS) {
-                iteration(it0 + s, s, b1, b2);
+                iteration(it0 + s, s, b0, b1, b2);
+                b0 = b1;
                 b1 = b2;
                 b2 = b2 == C::NBUF - 1 ? 0 : b2 + 1;
             }
