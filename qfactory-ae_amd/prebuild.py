@@ -41,7 +41,8 @@ def parity_cases():
               _case(1, 48, 4096, 2, 128, True), _case(3, 48, 1024, 8, 256, True),
               _case(1, 256, 11008, 4, 128),
               _case(1, 100, 256, 3, 64), _case(2, 77, 1024, 3, 128, True), _case(5, 130, 512, 3, 32),
-              _case(33, 64, 2048, 3, 128), _case(1, 50, 11008, 3, 128)]
+              _case(33, 64, 2048, 3, 128), _case(1, 50, 11008, 3, 128),
+              _case(48, 100, 1024, 3, 64), _case(7, 130, 512, 3, 128, True), _case(100, 96, 1536, 3, 128)]
     for nbits in (2, 3, 4, 8):                                  # group_size == -1: raw integer weights
         cases += [_case(1, 4096, 4096, nbits, -1), _case(3, 100, 256, nbits, -1)]
     # matrix-core regime: ragged M and N, M above one block tile, other widths and group sizes

@@ -25,6 +25,9 @@ MGEMV_MAX_M = 32
 def regime_for(M, K=None, nbits=None, group_size=None):
     if M < MGEMV_MIN_M or not MFMA_AVAILABLE:
         return "gemv"
+    if K is not None and nbits == 3:
+        # 3-bit has two kernels: the dot2 GEMV (any M, tiled over grid.y) and the GEMM
+        return "gemm" if gemm_supported(K, nbits, group_size) else "gemv"
     if K is None or not mfma_supported(K, nbits, group_size):
         return "gemv"
     if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
@@ -295,12 +298,12 @@ def mgemv_cfg_string(problem, t, nt_b):
 GEMM_BK = 64
 
 
-def gemm_lds_bytes(cfg):
+def gemm_lds_bytes(cfg, nbits=4):
     bm, nt32, wn, wk = cfg["BM"], cfg["NT32"], cfg["WN"], cfg["WK"]
     bn = 32 * nt32 * wn
     lds_a = wk * 3 * bm * (GEMM_BK + 8) * 2
     lds_red = (wk - 1) * bm * bn * 4
-    return max(lds_a, lds_red) + wk * wn * 32 * nt32 * 144
+    return max(lds_a, lds_red) + wk * wn * 32 * nt32 * (144 + (80 if nbits == 3 else 0))
 
 
 def gemm_regs(cfg):
@@ -315,9 +318,10 @@ def gemm_regs(cfg):
 
 def gemm_valid(cfg, K, nbits, group_size):
     """Mirror of the static checks in gemm_launch (qf_gemm.hip.h)."""
-    if nbits not in (2, 4, 8):
+    if nbits not in (2, 3, 4, 8):
         return False
-    supk = 1024 // nbits
+    pb, zfb = plane_bits(nbits), (4 if nbits == 3 else nbits)
+    supk = 1024 // pb
     sup = supk // GEMM_BK
     bm, nt32, wn, wk, pa = (cfg[k] for k in ("BM", "NT32", "WN", "WK", "PA"))
     if bm <= 0 or bm % 32 or min(nt32, wn, wk) < 1 or 64 * wn * wk > 1024:
@@ -327,7 +331,9 @@ def gemm_valid(cfg, K, nbits, group_size):
     if (group_size < supk and supk % group_size) or (group_size > supk and group_size % supk):
         return False
     ngs = max(1, supk // group_size)
-    if ngs > 8 or ngs * nbits > 32:
+    if ngs > 8 or ngs * zfb > 32:
+        return False
+    if (K // group_size) % (8 // zfb):
         return False
     if (bm * 8) % (64 * wn) or pa < 2 or (2 * sup) % pa:
         return False
@@ -335,7 +341,7 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     if gemm_regs(cfg) * max(1, 64 * wn * wk // 256) > 512:
         return False
-    return gemm_lds_bytes(cfg) <= 160 * 1024
+    return gemm_lds_bytes(cfg, nbits) <= 160 * 1024
 
 
 def gemm_supported(K, nbits, group_size):
@@ -369,7 +375,7 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     # with at most one block per CU the K axis is split over wave groups inside the block, so
     # that every SIMD still holds two waves (one dequantises while the other multiplies)
     wk = max(1, 8 // wn) if blocks <= NUM_CUS else 1
-    nsup = K // (1024 // nbits)
+    nsup = K // (1024 // plane_bits(nbits))
     wk = max(1, min(wk, nsup))
     pa = 4
     while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):

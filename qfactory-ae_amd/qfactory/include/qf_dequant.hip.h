@@ -24,7 +24,7 @@ __device__ __forceinline__ ZConst make_zconst(uint32_t zero) {
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int cls = k < D::NCLS ? k : 0;
-        const int o = (NBITS == 4) ? 4 * cls : (NBITS == 2 ? 2 * cls : 0);
+        const int o = (NBITS == 4) ? 4 * cls : ((NBITS == 2 || NBITS == 3) ? 2 * cls : 0);
         const uint32_t base = 0xE400u - 0x0400u * (uint32_t)o;          // exponent drops by one per factor 2
         const uint32_t h = base + (zero << o);
         c.off[k] = as_f16x2(h * 0x00010001u);
@@ -75,6 +75,34 @@ template <> struct IntStep<8> {
 };
 
 
+// 3-bit: eight fields of k-step t of a lane's 32 come from 2-bit-plane word w[t / 2] (its low or
+// high bytes) merged with the 1-bit-plane word `h` of the same 32 fields (see Decode<3>).
+struct IntStep3 {
+    template <int T>
+    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], uint32_t h, const ZConst& c) {
+        constexpr int R = T / 2;                      // which of the two 2-bit words
+        constexpr bool UPPER = (T & 1) != 0;          // its high bytes
+        const uint32_t wd = UPPER ? (w[R] >> 8) : w[R];
+        const uint32_t he = UPPER ? (h >> (8 + R)) : (h >> R);
+        const uint32_t ho = UPPER ? (h >> (4 + R)) : (h << (4 - R));
+        const uint32_t mg = magic_register();
+        f16x2 v[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t hs = (p % 2 == 0) ? he : ho;
+            const uint32_t x = (wd & (0x00030003u << (2 * p))) | (hs & (0x00040004u << (2 * p))) | mg;
+            const float inv = Decode<2>::inv_scale(p);
+            v[p] = __builtin_elementwise_fma(as_f16x2(x), f16x2{(_Float16)inv, (_Float16)inv}, c.off[p]);
+        }
+        return f16x8{v[0].x, v[0].y, v[1].x, v[1].y, v[2].x, v[2].y, v[3].x, v[3].y};
+    }
+};
+
+struct DequantStep3 {
+    template <int T>
+    __device__ __forceinline__ static f16x8 run(const uint32_t (&w)[4], uint32_t h, const struct QConst& c);
+};
+
 // scale splat + the offsets of make_zconst
 struct QConst {
     f16x2 s2;
@@ -95,5 +123,11 @@ template <int NBITS> struct DequantStep {
         return IntStep<NBITS>::run(w, t, c.z) * s8;
     }
 };
+
+template <int T>
+__device__ __forceinline__ f16x8 DequantStep3::run(const uint32_t (&w)[4], uint32_t h, const QConst& c) {
+    const f16x8 s8 = f16x8{c.s2.x, c.s2.y, c.s2.x, c.s2.y, c.s2.x, c.s2.y, c.s2.x, c.s2.y};
+    return IntStep3::run<T>(w, h, c.z) * s8;
+}
 
 }  // namespace qf

@@ -61,29 +61,35 @@ struct GemmCfg {
     static constexpr int TG = 64 * WN;                         // threads per group
     static constexpr int T = TG * WK;
     static constexpr int MT32 = BM / 32;
-    static constexpr int SUPK = 1024 / NBITS;                  // elements of K in 128 packed bytes
+    static constexpr int PB = plane_bits(NBITS);               // 3-bit rows: a 2-bit plane plus a 1-bit plane
+    static constexpr int ZFB = zero_field_bits(NBITS);         // stored width of one zero-point
+    static constexpr bool HI = NBITS == 3;
+    static constexpr int SUPK = 1024 / PB;                     // elements of K in 128 bytes of the main plane
     static constexpr int SUP = SUPK / BK;                      // K-iterations per super
     static constexpr int NSUP = K / SUPK;
     static constexpr int SUP_PER_GROUP = (NSUP + WK - 1) / WK;
     static constexpr int ITERS = SUP_PER_GROUP * SUP;          // K-iterations of every group
     static constexpr int UPS = TN * 8 / 64;                    // 16-byte units per lane and super
     static constexpr int UA = BM * (BK / 8) / TG;              // activation units per thread and iteration
-    static constexpr int LW = NBITS;                           // packed words per lane, tile and iteration
+    static constexpr int LW = PB;                              // main-plane words per lane, tile and iteration
     static constexpr int NGS = SUPK / GS > 0 ? SUPK / GS : 1;  // groups per row and super
     static constexpr int SREGS = (NGS + 1) / 2;                // registers of fp16 scales per tile and super
-    static constexpr int ZBITS = NGS * NBITS;                  // zero-point bits per tile and super
+    static constexpr int ZBITS = NGS * ZFB;                    // zero-point bits per tile and super
     static constexpr int PITCH = BK + 8;                       // activation tile row pitch in halves
     static constexpr int WPP = 128 + 16;                       // packed super row pitch in bytes
     static constexpr int RB = K * NBITS / 8;
     static constexpr int G = K / GS;
-    static constexpr int ZRB = G * NBITS / 8;
+    static constexpr int ZRB = G * ZFB / 8;
+    static constexpr int HI_OFF = K / 4;                       // byte offset of the 1-bit plane in a 3-bit row
+    static constexpr int HPP = 64 + 16;                        // 1-bit-plane super row pitch in bytes
+    static constexpr int UPH = TN * 4 / 64;                    // its 16-byte units per lane and super
     static constexpr int GRID_X = (N + BN - 1) / BN;
     static constexpr int NBUF = 3;                             // activation tiles in LDS per group
     // fetch the activation fragments of tile it+1 during iteration it (a second register set of
     // 16 * MT32 registers); tall tiles read each fragment just before its MFMAs instead
     static constexpr bool PREFETCH_A = MT32 <= 4;
     static constexpr size_t LDS_A = (size_t)WK * NBUF * BM * PITCH * 2;
-    static constexpr size_t LDS_W = (size_t)WK * WN * TN * WPP;
+    static constexpr size_t LDS_W = (size_t)WK * WN * TN * (WPP + (HI ? HPP : 0));
     static constexpr size_t LDS_RED = WK > 1 ? (size_t)(WK - 1) * BM * BN * 4 : 0;
     static constexpr size_t LDS_FRONT = LDS_A > LDS_RED ? LDS_A : LDS_RED;
     static constexpr size_t LDS_BYTES = LDS_FRONT + LDS_W;
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     constexpr int BM = C::BM, BK = C::BK, WN = C::WN, WK = C::WK, TN = C::TN;
     constexpr int MT32 = C::MT32, NT32 = C::NT32, PITCH = C::PITCH, WPP = C::WPP;
     constexpr int SUP = C::SUP, UPS = C::UPS, UA = C::UA, LW = C::LW, NGS = C::NGS, SREGS = C::SREGS;
-    constexpr uint32_t ZMASK = (1u << C::NBITS) - 1u;
+    constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -111,7 +117,8 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 
     // activation tiles live at the start of LDS (the final cross-group sum reuses that space)
     uint16_t* as = reinterpret_cast<uint16_t*>(smem) + (size_t)grp * C::NBUF * BM * PITCH;   // [NBUF][BM][PITCH]
-    uint8_t* wp = smem + C::LDS_FRONT + (size_t)wave * TN * WPP;                         // [TN][WPP]
+    uint8_t* wp = smem + C::LDS_FRONT + (size_t)wave * TN * (WPP + (C::HI ? C::HPP : 0));  // [TN][WPP] (+ [TN][HPP])
+    uint8_t* hp = wp + TN * WPP;
 
     // Block -> tile map.  The hardware deals workgroups round-robin to the 8 XCDs (linear id % 8),
     // each with its own L2.  Tiles are numbered M-slab by M-slab and every XCD gets a contiguous
@@ -158,13 +165,20 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 
     // ---- one super of this wave's TN weight rows: packed fields, scales, zero-points ----
     struct Quant { uint32_t s[NT32][SREGS]; uint32_t z[NT32]; };
-    struct WStage { u32x4 w[UPS]; Quant q; };
-    uint32_t w_off[UPS], s_off[NT32], z_off[NT32];             // per-lane byte offsets from the wave's first row
+    struct WStage { u32x4 w[UPS]; u32x4 h[C::HI ? C::UPH : 1]; Quant q; };
+    uint32_t w_off[UPS], h_off[C::HI ? C::UPH : 1], s_off[NT32], z_off[NT32];   // per-lane byte offsets from the wave's first row
     const int n_base = min(n_wave, C::N - 1);                  // a wave wholly past the last row re-reads it
 #pragma unroll
     for (int p = 0; p < UPS; p++) {
         const int u = lane + 64 * p;
         w_off[p] = (uint32_t)min(u / 8, C::N - 1 - n_base) * C::RB + (u % 8) * 16;
+    }
+    if constexpr (C::HI) {
+#pragma unroll
+        for (int p = 0; p < C::UPH; p++) {
+            const int u = lane + 64 * p;                        // four lanes share a row: 64 bytes per super
+            h_off[p] = (uint32_t)min(u / 4, C::N - 1 - n_base) * C::RB + C::HI_OFF + (u % 4) * 16;
+        }
     }
 #pragma unroll
     for (int j = 0; j < NT32; j++) {
@@ -184,9 +198,17 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             const uint8_t* src = wb + w_off[p];
             st.w[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
         }
+        if constexpr (C::HI) {
+            const uint8_t* hb = w_rows + (size_t)sup * 64;
+#pragma unroll
+            for (int p = 0; p < C::UPH; p++) {
+                const uint8_t* src = hb + h_off[p];
+                st.h[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
+            }
+        }
         const int g0 = sup * C::SUPK / C::GS;                  // first group of the super
         const uint8_t* sb = s_rows + (size_t)g0 * 2;
-        const uint8_t* zb = z_rows + (g0 * C::NBITS) / 8;
+        const uint8_t* zb = z_rows + (g0 * C::ZFB) / 8;
 #pragma unroll
         for (int j = 0; j < NT32; j++) {
             const uint8_t* sp = sb + s_off[j];
@@ -207,7 +229,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 if constexpr (C::ZBITS >= 32) st.q.z[j] = *reinterpret_cast<const uint32_t*>(zp);
                 else if constexpr (C::ZBITS == 16) st.q.z[j] = *reinterpret_cast<const uint16_t*>(zp);
                 else if constexpr (C::ZBITS == 8) st.q.z[j] = *zp;
-                else st.q.z[j] = (uint32_t)*zp >> ((g0 * C::NBITS) % 8);       // fewer than 8 bits: inside one byte
+                else st.q.z[j] = (uint32_t)*zp >> ((g0 * C::ZFB) % 8);         // fewer than 8 bits: inside one byte
             }
         }
     };
@@ -217,13 +239,21 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             const int u = lane + 64 * p;
             *reinterpret_cast<u32x4*>(wp + (u / 8) * WPP + (u % 8) * 16) = st.w[p];
         }
+        if constexpr (C::HI) {
+#pragma unroll
+            for (int p = 0; p < C::UPH; p++) {
+                const int u = lane + 64 * p;
+                *reinterpret_cast<u32x4*>(hp + (u / 4) * C::HPP + (u % 4) * 16) = st.h[p];
+            }
+        }
     };
     // this lane's packed fields of iteration q of the super in LDS: 32 fields = 4*NBITS bytes per tile
-    struct Packed { uint32_t w[NT32][LW >= 4 ? LW : 4]; };
+    struct Packed { uint32_t w[NT32][LW >= 4 ? LW : 4]; uint32_t h[NT32]; };
     auto read_packed = [&](Packed& pk, int q) {
 #pragma unroll
         for (int j = 0; j < NT32; j++) {
-            const uint8_t* src = wp + (j * 32 + li) * WPP + (q * BK + 32 * kb) * C::NBITS / 8;
+            const uint8_t* src = wp + (j * 32 + li) * WPP + (q * BK + 32 * kb) * C::PB / 8;
+            if constexpr (C::HI) pk.h[j] = *reinterpret_cast<const uint32_t*>(hp + (j * 32 + li) * C::HPP + (q * BK + 32 * kb) / 8);
             if constexpr (LW == 2) {
                 const u32x2 v = *reinterpret_cast<const u32x2*>(src);
                 pk.w[j][0] = v.x; pk.w[j][1] = v.y; pk.w[j][2] = 0; pk.w[j][3] = 0;
@@ -246,10 +276,10 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         } else if constexpr (C::GS >= BK) {
             const int gi = q * BK / C::GS;
             sbits = (qu.s[j][gi / 2] >> (16 * (gi % 2))) & 0xFFFFu;
-            zero = (qu.z[j] >> (gi * C::NBITS)) & ZMASK;
+            zero = (qu.z[j] >> (gi * C::ZFB)) & ZMASK;
         } else {                                               // GS == 32: group 2q + kb
             sbits = kb ? (qu.s[j][q] >> 16) : (qu.s[j][q] & 0xFFFFu);
-            zero = (qu.z[j] >> ((2 * q + kb) * C::NBITS)) & ZMASK;
+            zero = (qu.z[j] >> ((2 * q + kb) * C::ZFB)) & ZMASK;
         }
         if constexpr (C::SYM) zero = 1u << (C::NBITS - 1);
         return make_qconst<C::NBITS>((uint16_t)sbits, zero);
@@ -313,6 +343,10 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                     const QConst qc = qconst_of(qcur, j, q);
                     if constexpr ((QF_GEMM_EXPERIMENT & 1) != 0) {
                         wf[j] = __builtin_bit_cast(f16x8, u32x4{cur.w[j][0], cur.w[j][1], cur.w[j][2], cur.w[j][3] + (uint32_t)ks});
+                    } else if constexpr (C::NBITS == 3) {
+                        const uint32_t w4[4] = {cur.w[j][0], cur.w[j][1], 0u, 0u};
+                        wf[j] = ks == 0 ? DequantStep3::run<0>(w4, cur.h[j], qc) : ks == 1 ? DequantStep3::run<1>(w4, cur.h[j], qc)
+                              : ks == 2 ? DequantStep3::run<2>(w4, cur.h[j], qc) : DequantStep3::run<3>(w4, cur.h[j], qc);
                     } else if constexpr (C::NBITS == 8) {
                         const int h = 4 * (ks / 2);
                         const uint32_t w4[4] = {cur.w[j][h], cur.w[j][h + 1], cur.w[j][h + 2], cur.w[j][h + 3]};
@@ -428,16 +462,16 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 template <class C>
 int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m, hipStream_t stream) {
     const char* why = nullptr;
-    if (C::NBITS != 2 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 4 or 8 for this kernel";
+    if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8";
     else if (C::BM % 32 != 0 || C::BM <= 0 || C::NT32 < 1 || C::WN < 1 || C::WK < 1) why = "BM must be a multiple of 32; NT32, WN, WK positive";
     else if (C::T > 1024) why = "block too large";
-    else if (C::K % C::SUPK != 0 || C::NSUP < 1) why = "K must be a multiple of 1024/NBITS (128 packed bytes)";
+    else if (C::K % C::SUPK != 0 || C::NSUP < 1) why = "K must be a multiple of 128 packed bytes of the main plane";
     else if (C::GS <= 0 || C::K % C::GS != 0) why = "GS must divide K";
     else if (C::GS % 32 != 0) why = "a lane's 32 fields must lie inside one group (GS multiple of 32)";
     else if (C::GS < C::SUPK && C::SUPK % C::GS != 0) why = "GS must divide 1024/NBITS or be a multiple of it";
     else if (C::GS > C::SUPK && C::GS % C::SUPK != 0) why = "GS must divide 1024/NBITS or be a multiple of it";
     else if (C::NGS > 8 || C::ZBITS > 32) why = "too many groups per 128 packed bytes";
-    else if (!C::SYM && (C::G % (8 / C::NBITS)) != 0) why = "K/GS must fill whole zero-point bytes";
+    else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if ((C::BM * (C::BK / 8)) % C::TG != 0) why = "the activation tile must split evenly over a group's threads";
     else if (C::PA < 2 || (2 * C::SUP) % C::PA != 0) why = "PA must be >= 2 and divide 2048/NBITS/64";
     else if (C::LDS_BYTES > 160 * 1024) why = "tiles exceed the 160 KB of LDS";
