@@ -24,6 +24,11 @@
 #include <cstdio>
 #include "qf_dequant.hip.h"
 
+// Tiles a block finishes between two reductions through LDS (a multiple of the ring depth PF).
+#ifndef QF_MGEMV_SB
+#define QF_MGEMV_SB 4
+#endif
+
 namespace qf {
 
 template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_>
@@ -44,7 +49,7 @@ struct MGemvCfg {
     static constexpr int GRID_X = NT < PB ? NT : PB;
     static constexpr int SLOTS = (NT + GRID_X - 1) / GRID_X;               // tiles per block
     static constexpr int PF = PF_;                 // weight tiles in flight per wave (ring of stages): 2 or 4
-    static constexpr int SB = 4;                   // tiles per batch: partials are reduced and stored per batch
+    static constexpr int SB = QF_MGEMV_SB;         // tiles per batch: partials are reduced and stored per batch
     static constexpr int NBATCH = (SLOTS + SB - 1) / SB;
     static constexpr int RB = K * NBITS / 8;
     static constexpr int G = K / GS;
@@ -124,10 +129,11 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         }
     };
 
-    // ring of PF stages: tiles slot .. slot+PF-1 of this team are in flight
+    // ring of PF stages: tiles slot .. slot+PF-1 of this team are in flight.  The first PF go out
+    // before anything else, so that their HBM latency overlaps the activation loads.
     WStage ring[PF];
 #pragma unroll
-    for (int p = 0; p < PF - 1; p++)
+    for (int p = 0; p < PF; p++)
         if (p < SLOTS) load_tile(ring[p], min(team_id + p * TEAM_STRIDE, C::NT - 1));
 
     // ---- resident activations, brought into MFMA fragment order through the wave's LDS buffer:
@@ -138,17 +144,32 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         constexpr int PITCH_A = ROWB + 16;
         constexpr int LPRA = ROWB / 16;                  // lanes per row
         constexpr int RPIA = 64 / LPRA;                  // rows per load (LPRA <= 64)
+        // every global load of the slice goes out first (they are independent; issued one by one
+        // behind the LDS round trips below they would each expose a full L2 latency), then the
+        // chunks pass through the wave's LDS buffer one after another
+        constexpr int LPC = 16 / RPIA;                   // loads per chunk
+        u32x4 raw[MT16][CH][LPC];
+#pragma unroll
+        for (int mt = 0; mt < MT16; mt++)
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+#pragma unroll
+                for (int i = 0; i < LPC; i++) {
+                    const int row = i * RPIA + lane / LPRA;
+                    const int m = m0 + 16 * mt + row;
+                    const uint16_t* ap = A + (size_t)min(m, m_total - 1) * C::K + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8;
+                    raw[mt][c][i] = *reinterpret_cast<const u32x4*>(ap);
+                }
 #pragma unroll
         for (int mt = 0; mt < MT16; mt++) {
 #pragma unroll
             for (int c = 0; c < CH; c++) {
                 const bool own = (lo + c >= own_from) && (lo + c < own_from + CH);
 #pragma unroll
-                for (int i = 0; i < 16 / RPIA; i++) {
+                for (int i = 0; i < LPC; i++) {
                     const int row = i * RPIA + lane / LPRA;
                     const int m = m0 + 16 * mt + row;
-                    const uint16_t* ap = A + (size_t)min(m, m_total - 1) * C::K + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8;
-                    u32x4 v = *reinterpret_cast<const u32x4*>(ap);
+                    u32x4 v = raw[mt][c][i];
                     if (!(own && m < m_total)) v = u32x4{0, 0, 0, 0};
                     *reinterpret_cast<u32x4*>(wbuf + row * PITCH_A + (lane % LPRA) * 16) = v;
                 }
@@ -171,9 +192,6 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             const int slot = batch * SB + sb;
             const int tile = team_id + slot * TEAM_STRIDE;
             WStage& cur = ring[sb % PF];
-            // refill the stage consumed in the previous iteration with the tile PF-1 ahead
-            if (slot + PF - 1 < SLOTS)
-                load_tile(ring[(sb + PF - 1) % PF], min(tile + (PF - 1) * TEAM_STRIDE, C::NT - 1));
             f32x4 acc[MT16];
 #pragma unroll
             for (int mt = 0; mt < MT16; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -189,6 +207,15 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                 for (int c = 0; c < CH; c++)
                     wfrag[c] = *reinterpret_cast<const u32x4*>(wbuf + r * PITCH_W + c * 64 + kb * 16);
                 __builtin_amdgcn_wave_barrier();
+                // the stage's packed words are in LDS and its scales / zero-points in `qs` / `qz`:
+                // it takes the loads of the tile PF ahead right away, one whole tile of
+                // dequantisation and MFMAs before they are needed
+                uint32_t qs[NSI], qz[NZI];
+#pragma unroll
+                for (int j = 0; j < NSI; j++) qs[j] = cur.s[j];
+#pragma unroll
+                for (int j = 0; j < NZI; j++) qz[j] = C::SYM ? 0u : cur.z[j];
+                if (slot + PF < SLOTS) load_tile(cur, min(tile + PF * TEAM_STRIDE, C::NT - 1));
 #pragma unroll
                 for (int c = 0; c < CH; c++) {
                     const int g = ((lo + c) * CHUNK + kb * EPL) / C::GS;     // group of this lane's fields
@@ -197,7 +224,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     uint32_t sraw = 0;
 #pragma unroll
                     for (int j = 0; j < NSI; j++) {
-                        const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((sidx & 63) << 2, (int)cur.s[j]);
+                        const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((sidx & 63) << 2, (int)qs[j]);
                         sraw = (NSI == 1 || (sidx >> 6) == j) ? v : sraw;
                     }
                     uint32_t zero = 1u << (C::NBITS - 1);
@@ -207,7 +234,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                         uint32_t zraw = 0;
 #pragma unroll
                         for (int j = 0; j < NZI; j++) {
-                            const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((zidx & 63) << 2, (int)cur.z[j]);
+                            const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((zidx & 63) << 2, (int)qz[j]);
                             zraw = (NZI == 1 || (zidx >> 6) == j) ? v : zraw;
                         }
                         zero = (zraw >> ((g % P8) * C::NBITS)) & ZMASK;
