@@ -144,9 +144,10 @@ class QMatmulQFunc(QFunc):
         b = lambda x: "true" if x else "false"
         code = "// QFactory-HIP generated translation unit\n\n"
         defines = dict(getattr(self, "defines", {}))                        # kernel-header tuning knobs
-        if self.regime == "gemm":
-            # the GEMM kernel is bound by vector-instruction issue and has registers to spare: the
-            # one-instruction mask-and-merge decode pays there (it does not in the GEMV kernel)
+        if self.regime in ("gemm", "mgemv"):
+            # the matrix-core kernels expose their dequantisation's vector-instruction issue and have
+            # registers to spare: the one-instruction mask-and-merge decode pays there (2 - 7 %
+            # measured); it does not in the 4-bit GEMV kernel, where it costs a resident wave
             defines.setdefault("QF_FUSED_AND_OR", 1)
         if self.regime == "gemv" and p["NBITS"] == 2:
             # sixteen fields per word make the 2-bit GEMV decode-bound: measured 7.6 -> 6.9 us at 8192 x 8192

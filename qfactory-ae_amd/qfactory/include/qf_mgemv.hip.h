@@ -29,6 +29,12 @@
 #define QF_MGEMV_SB 4
 #endif
 
+// Timing experiments (results are wrong when non-zero): bit 0 skips the activation loads, bit 1 the
+// dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores, bit 3 the weight loads.
+#ifndef QF_MGEMV_EXPERIMENT
+#define QF_MGEMV_EXPERIMENT 0
+#endif
+
 namespace qf {
 
 template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_>
@@ -106,6 +112,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         uint32_t z[NZI];             // lane -> (row, byte)  = (idx / ZB,  idx % ZB)
     };
     auto load_tile = [&](WStage& st, int tile) {
+        if (QF_MGEMV_EXPERIMENT & 8) return;
         const int n_base = tile * 16;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
@@ -158,7 +165,8 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     const int row = i * RPIA + lane / LPRA;
                     const int m = m0 + 16 * mt + row;
                     const uint16_t* ap = A + (size_t)min(m, m_total - 1) * C::K + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8;
-                    raw[mt][c][i] = *reinterpret_cast<const u32x4*>(ap);
+                    if (QF_MGEMV_EXPERIMENT & 1) raw[mt][c][i] = u32x4{(uint32_t)lane, 1u, 2u, 3u};
+                    else raw[mt][c][i] = *reinterpret_cast<const u32x4*>(ap);
                 }
 #pragma unroll
         for (int mt = 0; mt < MT16; mt++) {
@@ -195,7 +203,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             f32x4 acc[MT16];
 #pragma unroll
             for (int mt = 0; mt < MT16; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (slot < SLOTS && tile < C::NT) {               // wave-uniform
+            if (slot < SLOTS && tile < C::NT && !(QF_MGEMV_EXPERIMENT & 2)) {               // wave-uniform
                 // coalesced registers -> LDS -> fragment registers: lane (r, kb) takes the 16 bytes
                 // of row r at chunk c, k-block kb
 #pragma unroll
@@ -282,7 +290,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         // ---- sum the WK partial tiles of this batch and store.  A partial tile sits in LDS as
         //      [lane = n + 16*(m/4)][e = m%4]; the storing lane takes (m = lane/4, n = 4*(lane%4) .. +3):
         //      one 8-byte store per lane. ----
-        for (int p = wk; p < SB * MT16; p += WK) {
+        for (int p = wk; p < SB * MT16 && !(QF_MGEMV_EXPERIMENT & 4); p += WK) {
             const int sb = p / MT16, mt = p % MT16;
             const int slot = batch * SB + sb;
             const int tile = team_id + slot * TEAM_STRIDE;
