@@ -59,6 +59,16 @@ struct GemvCfg {
     static constexpr int GRID_X = (N + RPB - 1) / RPB;
 };
 
+// Timing experiments (results are wrong when non-zero): bit 0 replaces the decode + dot products by
+// an xor of the loaded words, bit 1 skips the activation loads, bit 2 the scale / zero-point loads.
+#ifndef QF_GEMV_EXPERIMENT
+#define QF_GEMV_EXPERIMENT 0
+#endif
+
+#ifndef QF_GEMV_A_FIRST
+#define QF_GEMV_A_FIRST 1
+#endif
+
 // Lower bound on resident waves per SIMD the register allocator must leave room for (0: no bound).
 #ifndef QF_GEMV_WAVES_PER_EU
 #define QF_GEMV_WAVES_PER_EU 0
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
             for (int it = 0; it < IT; it++) {
                 load_words<NW, C::NT_B>(wrow + (uint32_t)coff[it], st.w[u][it]);
                 if constexpr (NWH > 0) load_words<NWH, C::NT_B>(wrow + (uint32_t)(C::HI_OFF + coff[it] / 2), st.h[u][it]);
-                if constexpr (C::QPARAM) {
+                if constexpr (C::QPARAM && !(QF_GEMV_EXPERIMENT & 4)) {
                     st.s[u][it] = *reinterpret_cast<const uint16_t*>(srow + (uint32_t)(goff[it] * 2));
                     if constexpr (!C::SYM) st.z[u][it] = zrow[(uint32_t)(goff[it] / P8)];
                 }
@@ -135,38 +145,49 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         }
     };
 
-    // The first stage of weights goes out before anything else so that its HBM latency overlaps
-    // the activation loads and their bookkeeping.
+    // Load order (QF_GEMV_A_FIRST, default 1).  Loads complete in issue order, so whatever is issued
+    // behind the first stage of weights is only seen once those have arrived from HBM.  With the
+    // activation loads issued first (they come from L2, a few hundred ns) their per-chunk sums are
+    // computed while the weights are still in flight; issued second, that work waits for the weights.
     Stage st0, st1;
-    load_stage(st0, 0);
-    QF_SCHED_FENCE();      // keep every stage-0 load ahead of the activation loads
-
-    // ---- the stationary activations and their per-chunk sums ----
     uint32_t a[MT][IT][AR];
     float c1[MT][IT];        // sum over classes of 1024 * 2^-o * (sum of a in that class)
     float sa[MT][IT];        // sum of a over the chunk
+    if constexpr (!QF_GEMV_A_FIRST) load_stage(st0, 0);
+    // ---- the stationary activations ----
 #pragma unroll
     for (int it = 0; it < IT; it++) {
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             const int mm = min(m0 + m, m_total - 1);
             const uint16_t* ap = A + (size_t)mm * C::K + (size_t)(coff[it] / C::VB) * EPC;
-            float cls_sum[NCLS];
-#pragma unroll
-            for (int c2 = 0; c2 < NCLS; c2++) cls_sum[c2] = 0.0f;
 #pragma unroll
             for (int r = 0; r < AR; r += (AR >= 4 ? 4 : AR)) {
                 constexpr int LW = AR >= 4 ? 4 : AR;
                 uint32_t tmp[LW];
-                load_words<LW, false>(ap + 2 * r, tmp);
+                if (QF_GEMV_EXPERIMENT & 2) { for (int j = 0; j < LW; j++) tmp[j] = 0x3C003C00u; }
+                else load_words<LW, false>(ap + 2 * r, tmp);
 #pragma unroll
-                for (int j = 0; j < LW; j++) {
-                    const uint32_t val = cvalid[it] ? tmp[j] : 0u;
-                    a[m][it][r + j] = val;
-                    // sum of the pair in one instruction: dot2 with (1, 1)
-                    cls_sum[D::cls((r + j) % PAIRS)] = __builtin_amdgcn_fdot2(
-                        as_f16x2(val), as_f16x2(0x3C003C00u), cls_sum[D::cls((r + j) % PAIRS)], false);
-                }
+                for (int j = 0; j < LW; j++) a[m][it][r + j] = tmp[j];
+            }
+        }
+    }
+    if constexpr (QF_GEMV_A_FIRST) load_stage(st0, 0);
+    // ---- and their per-chunk sums ----
+#pragma unroll
+    for (int it = 0; it < IT; it++) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            float cls_sum[NCLS];
+#pragma unroll
+            for (int c2 = 0; c2 < NCLS; c2++) cls_sum[c2] = 0.0f;
+#pragma unroll
+            for (int r = 0; r < AR; r++) {
+                const uint32_t val = cvalid[it] ? a[m][it][r] : 0u;
+                a[m][it][r] = val;
+                // sum of the pair in one instruction: dot2 with (1, 1)
+                cls_sum[D::cls(r % PAIRS)] = __builtin_amdgcn_fdot2(
+                    as_f16x2(val), as_f16x2(0x3C003C00u), cls_sum[D::cls(r % PAIRS)], false);
             }
             float c1v = 0.0f, sav = 0.0f;
 #pragma unroll
@@ -192,6 +213,11 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 for (int m = 0; m < MT; m++)
 #pragma unroll
                     for (int c2 = 0; c2 < NCLS; c2++) acc[m][c2] = 0.0f;
+                if constexpr ((QF_GEMV_EXPERIMENT & 1) != 0) {
+                    uint32_t t = 0;
+                    for (int j = 0; j < NW; j++) t ^= st.w[u][it][j];
+                    acc[0][0] += (float)(t & 1u);
+                } else
 #pragma unroll
                 for (int j = 0; j < NW; j++) {
                     uint32_t x[PAIRS];
