@@ -71,7 +71,7 @@ def smoke_cases():
 def misc_test_cases():
     """Other modules the GPU tests construct (row-count dispatch, argument checks)."""
     return ([_case(M, 96, 512, 4, 128) for M in (1, 2, 3, 6)] + [_case(1, 64, 256, 4, 128)]
-            + [_case(1, 384, 1024, 4, 128), _case(64, 384, 1024, 4, 128)])
+            + [_case(1, 384, 1024, 4, 128), _case(16, 384, 1024, 4, 128), _case(64, 384, 1024, 4, 128)])
 
 
 TINY_LLAMA = [(768, 256), (256, 256), (1024, 256), (256, 512)]      # the decode-loop test model, GS = 64

@@ -118,3 +118,26 @@ def test_closure_rejects_bad_tensors(qf):
         layer.func(x, layer.w.T, out, layer.s, layer.z)                  # shape / contiguity
     with pytest.raises(NotImplementedError):
         qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), bias=True)
+
+
+@pytest.mark.parametrize("M", [1, 16, 64])
+def test_reference_launch_symbol_through_plain_ctypes(qf, oracle, M):
+    """The reference-shaped entry point `launch(act, weight, out, scale, zero, stream, &rc)` (compile-time
+    M), bound the way the reference's loader binds it (qfactory/jit/runtime.py:37-49): a bare CDLL, void
+    pointers and an int by reference -- no helper of this package between the test and the C ABI."""
+    import ctypes
+    import os
+    N, K, nbits, GS = 384, 1024, 4, 128
+    A, weight, scale, zero = make_problem(77 + M, M, N, K, nbits, GS, False)
+    layer = qf.init(M, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
+    lib = ctypes.CDLL(os.path.join(layer.func.runtime.path, "kernel.so"))
+    x = A.cuda()
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    rc = ctypes.c_int(-1)
+    args = [ctypes.c_void_p(t.data_ptr()) for t in (x, layer.w, out, layer.s, layer.z)]
+    lib.launch.restype = None
+    lib.launch(*args, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), ctypes.byref(rc))
+    torch.cuda.synchronize()
+    assert rc.value == 0
+    ref = reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS)
+    assert_close(oracle, out.cpu().numpy(), ref, f"launch M={M}")
