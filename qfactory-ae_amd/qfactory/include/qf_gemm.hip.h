@@ -39,7 +39,9 @@
 #define QF_GEMM_EXPERIMENT 0
 #endif
 
-// 1: XCD-aware block -> tile map (see the kernel), 0: plain blockIdx order.
+// 1: block -> tile map that keeps the slabs of one column of tiles together on one XCD (see the
+// kernel), 0: plain blockIdx order.  Measured no faster (358 vs 365 us on 57344 x 8192 at M = 256, slower
+// with two 32-row tiles per wave): the Infinity Cache already serves the second fetch.  Off.
 #ifndef QF_GEMM_XCD_MAP
 #define QF_GEMM_XCD_MAP 0
 #endif
@@ -121,14 +123,22 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     uint8_t* hp = wp + TN * WPP;
 
     // Block -> tile map.  The hardware deals workgroups round-robin to the 8 XCDs (linear id % 8),
-    // each with its own L2.  Tiles are numbered M-slab by M-slab and every XCD gets a contiguous
-    // range of that numbering, so one XCD re-reads one (or few) BM-row activation slab(s), which
-    // stay in its L2, instead of all of them.
+    // each with its own L2, in linear-id order.  The BM-row slabs of one column of tiles read the
+    // same weight rows: they get ids 8 apart (same XCD, dispatched together), so the weights come
+    // from HBM once and the other slabs hit in that XCD's L2.  With the plain (x, y) order the
+    // slabs of a column are gridDim.x ids apart: once there are more tiles than CUs they run at
+    // different times and every slab fetches the weights from memory again (measured with
+    // FETCH_SIZE: 552 MB instead of 240 MB on the 57344 x 8192 layer at M = 256).
     const int linear = blockIdx.x + gridDim.x * blockIdx.y;
-    const int total = gridDim.x * gridDim.y;
-    const int tile = (QF_GEMM_XCD_MAP && total % 8 == 0) ? (linear % 8) * (total / 8) + linear / 8 : linear;
-    const int n_blk = (tile % C::GRID_X) * C::BN;
-    const int m_blk = (tile / C::GRID_X) * BM;
+    int col = blockIdx.x, slab = blockIdx.y;
+    if (QF_GEMM_XCD_MAP && C::GRID_X % 8 == 0) {
+        const int per_group = 8 * gridDim.y;                    // tiles of 8 columns
+        const int grp8 = linear / per_group, rem = linear % per_group;
+        col = grp8 * 8 + rem % 8;
+        slab = rem / 8;
+    }
+    const int n_blk = col * C::BN;
+    const int m_blk = slab * BM;
     const int n_wave = n_blk + wn * TN;
 
     // K offset of the group's iteration `it`: supers are dealt round-robin to the groups; a group
