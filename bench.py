@@ -257,6 +257,9 @@ def small_m_report():
         for nbits in (2, 3, 4, 8):
             for sym in (False, True):
                 one("configs[2]", M, 8192, 8192, nbits, sym)
+    # the 28672-wide end of the "4096 - 28672-wide LLM shapes" the GEMV target names: Llama-3-70B at M = 1
+    for name, N, K in GEMM_SHAPES:
+        one("70b-gemv", 1, N, K, NBITS, False)
     return report
 
 

@@ -61,6 +61,7 @@ def large_parity_cases():
 
 def bench_cases():
     cases = [_case(1, N, K) for N, K in LLAMA2_7B]
+    cases += [_case(1, N, K) for N, K in LLAMA3_70B]          # bench.py --small-m
     return cases
 
 

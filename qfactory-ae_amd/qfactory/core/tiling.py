@@ -101,18 +101,23 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
         wk, it = gemv_wave_split(K, nbits, vb, mt)[0]
     else:
         it = -(-(K // elements_per_chunk(nbits, vb)) // (64 * wk))
+    # Loads in flight per lane (rows x chunks per row), measured on MI355X once the kernel's address
+    # arithmetic had moved to scalar registers:
+    #   * launches of at most ~2 rounds of resident waves (the 7B shapes): 4 loads, two teams per
+    #     block, one stage -- many small waves (61 registers, 8 per SIMD) beat deeper stages;
+    #   * larger launches (57344 x 8192: 7 rounds) or rows longer than one pass of the team
+    #     (K = 28672): 8 loads, one team per block, and a second stage when a lane holds two chunks
+    #     (46.6 -> 40.5 us and 37.6 -> 25.5 us);
+    #   * 2- and 3-bit rows are short in bytes and heavy in decode work: 8 loads.
+    big = it >= 2 or (N * wk) // 4 > 2 * 8 * 4 * NUM_CUS
     if u is None:
-        # four rows (4 x 16 bytes per lane) in flight per wave and no second stage measured best on
-        # MI355X once the kernel's address arithmetic had moved to scalar registers: many small
-        # waves (61 registers, 8 per SIMD) beat fewer waves with deeper stages
-        # (2- and 3-bit rows are short in bytes and heavy in decode work: eight rows measured best)
-        rows = 8 if nbits <= 3 else 4
-        u = max(1, min(rows // it if it <= rows else 1, 64 // mt, rows))
+        in_flight = 8 if (big or nbits <= 3) else 4
+        u = max(1, min(in_flight // it if it <= in_flight else 1, 64 // mt, in_flight))
         u = _pow2_floor(u)
     if wn is None:
-        wn = 2 if wk * 2 <= 16 else 1                 # two teams per block measured best on MI355X
+        wn = 1 if big else (2 if wk * 2 <= 16 else 1)
     if steps is None:
-        steps = 1
+        steps = 2 if (big and it >= 2) else 1
     return {"MT": mt, "WK": wk, "WN": wn, "U": u, "STEPS": steps, "VB": vb}
 
 
