@@ -4,13 +4,19 @@ This is the analytic half of what the reference does by brute force (``QMatmulQF
 qfactory/core/qfunc.py:110-131, enumerates BLOCK_N x BLOCK_SIZE x NUM_ELM and times all of them):
 given the problem it proposes one default tiling and a short list of neighbours worth timing.
 
-Two regimes:
+Four kernel families (``regime_for`` picks one):
 
-* ``gemv``  -- M small, HBM-bound.  Parameters of ``qf::GemvCfg`` (include/qf_gemv.hip.h):
-  ``MT`` activation rows per block, ``WK`` waves along K per team, ``WN`` teams per block, ``U`` rows
-  in flight per stage, ``STEPS`` stages per block, ``VB`` bytes per lane and load.
-* ``mfma``  -- M large enough for the matrix cores.  Parameters of ``qf::MfmaCfg``
-  (include/qf_mfma.hip.h): ``BM`` x ``BN`` block tile, ``WM`` x ``WNW`` wave grid, K-split ``KS``.
+* ``gemv``  -- M < 3 (and 3-bit M <= 2), HBM-bound, v_dot2.  Parameters of ``qf::GemvCfg``
+  (include/qf_gemv.hip.h): ``MT`` activation rows per block, ``WK`` waves along K per team, ``WN``
+  teams per block, ``U`` rows in flight per stage, ``STEPS`` stages per block, ``VB`` bytes per lane
+  and load.
+* ``mgemv`` -- 3 <= M <= 32 when the activations fit the register file: persistent A-stationary MFMA
+  kernel, ``qf::MGemvCfg`` (include/qf_mgemv.hip.h): ``MT16`` 16-row activation tiles, ``WK`` waves x
+  ``CH`` chunks covering K, ``PB`` blocks, ``PF`` weight tiles in flight.
+* ``gemm``  -- larger M (and what ``mgemv`` cannot hold): ``qf::GemmCfg`` (include/qf_gemm.hip.h):
+  ``BM`` activation rows per block, ``NT32`` 32-row weight tiles per wave, ``WN`` waves along N,
+  ``WK`` wave groups along K, ``PA`` activation tiles in flight.
+* ``mfma``  -- generic fallback, ``qf::MfmaCfg`` (include/qf_mfma.hip.h).
 """
 
 NUM_CUS = 256

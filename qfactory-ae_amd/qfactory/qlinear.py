@@ -74,8 +74,8 @@ class GPTQLinear(torch.nn.Module):
         matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
                          torch.float16, torch.int8, self.group_size, base_impl=self.base_impl)
         func = matmul.compile_profile(**compile_flags)
-        # One launch now: a specialisation may allocate scratch on its first call (split-K
-        # partial tiles), which must not happen later inside a HIP-graph capture.
+        # One launch now: the first call of a specialisation loads its code object and may raise its
+        # LDS limit (hipFuncSetAttribute), neither of which should happen inside a HIP-graph capture.
         if self.w.is_cuda:
             x = torch.zeros(m, self.in_features, dtype=torch.float16, device=self.w.device)
             out = torch.empty(m, self.out_features, dtype=torch.float16, device=self.w.device)
