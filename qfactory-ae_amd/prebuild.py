@@ -81,7 +81,7 @@ TINY_LLAMA = [(768, 256), (256, 256), (1024, 256), (256, 512)]      # the decode
 def decode_cases():
     """decode_llama.py: Llama-2-7B shapes at batch 1 / 16 / 64 (decode) and at prefill row counts,
     plus the tiny model tests/test_decode_gpu.py runs."""
-    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 256)]
+    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256)]
     cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
     return cases
 
