@@ -304,7 +304,8 @@ def mgemv_cfg_string(problem, t, nt_b):
 
 # --------------------------------------------------------------------------------------------
 # Large-M GEMM regime (qf::GemmCfg, include/qf_gemm.hip.h): weights dequantised into MFMA
-# fragment registers, activations through LDS, WK wave groups splitting K inside a block
+# fragment registers, activations loaded straight into LDS (PA tiles ahead), WK wave groups
+# splitting K inside a block
 # --------------------------------------------------------------------------------------------
 GEMM_BK = 64
 
@@ -312,19 +313,20 @@ GEMM_BK = 64
 def gemm_lds_bytes(cfg, nbits=4):
     bm, nt32, wn, wk = cfg["BM"], cfg["NT32"], cfg["WN"], cfg["WK"]
     bn = 32 * nt32 * wn
-    lds_a = wk * 3 * bm * (GEMM_BK + 8) * 2
+    nbuf = cfg["PA"] + (0 if bm // 32 <= 4 else 1)     # tiles in flight (+ the one being read when fragments are not prefetched)
+    lds_a = wk * nbuf * bm * GEMM_BK * 2
     lds_red = (wk - 1) * bm * bn * 4
     return max(lds_a, lds_red) + wk * wn * 32 * nt32 * (144 + (80 if nbits == 3 else 0))
 
 
 def gemm_regs(cfg):
     """Rough VGPR need of one lane: accumulators, two sets of activation fragments, the weight
-    super ring and the activation ring, plus ~80 of addresses and dequantisation temporaries.
-    A SIMD has 512 per lane to share between the waves a block puts on it (spills are ruinous)."""
+    super ring, plus ~80 of addresses and dequantisation temporaries.  A SIMD has 512 per lane to
+    share between the waves a block puts on it (spills are ruinous)."""
     mt32, nt32 = cfg["BM"] // 32, cfg["NT32"]
     ua = max(1, cfg["BM"] * 8 // (64 * cfg["WN"]))
     frag_sets = 2 if mt32 <= 4 else 0.25               # tall tiles keep one k-step of fragments, not two tiles
-    return int(mt32 * nt32 * 16 + frag_sets * mt32 * 16 + 2 * nt32 * 20 + cfg["PA"] * ua * 4 + 80)
+    return int(mt32 * nt32 * 16 + frag_sets * mt32 * 16 + 2 * nt32 * 20 + ua + 80)
 
 
 def gemm_valid(cfg, K, nbits, group_size):
@@ -333,7 +335,6 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     pb, zfb = plane_bits(nbits), (4 if nbits == 3 else nbits)
     supk = 1024 // pb
-    sup = supk // GEMM_BK
     bm, nt32, wn, wk, pa = (cfg[k] for k in ("BM", "NT32", "WN", "WK", "PA"))
     if bm <= 0 or bm % 32 or min(nt32, wn, wk) < 1 or 64 * wn * wk > 1024:
         return False
@@ -346,7 +347,7 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     if (K // group_size) % (8 // zfb):
         return False
-    if (bm * 8) % (64 * wn) or pa < 2 or (2 * sup) % pa:
+    if (bm * 8) % (64 * wn) or not 3 <= pa <= 12:
         return False
     if (bm // 32) * nt32 * 16 > 256:
         return False
@@ -356,7 +357,7 @@ def gemm_valid(cfg, K, nbits, group_size):
 
 
 def gemm_supported(K, nbits, group_size):
-    probe = {"BM": 64, "NT32": 1, "WN": 4, "WK": 1, "PA": 2}
+    probe = {"BM": 64, "NT32": 1, "WN": 4, "WK": 1, "PA": 3}
     return gemm_valid(probe, K, nbits, group_size)
 
 
@@ -391,7 +392,7 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     pa = 4
     while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
         if pa == 4:
-            pa = 2                                    # a shallower activation ring frees registers
+            pa = 3                                    # one activation tile less in LDS
         elif wk > 1:
             wk, pa = wk // 2, 4
         else:
@@ -417,7 +418,7 @@ def gemm_candidates(M, N, K, nbits, group_size):
         for nt32 in (1, 2):
             for wn in (1, 2, 4):
                 for wk in (1, 2, 4, 8):
-                    for pa in (2, 4, 8):
+                    for pa in (3, 4, 6):
                         add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})
     return out
 

@@ -21,10 +21,14 @@
 //     share a row: fully coalesced), two supers ahead of use, into a buffer private to the wave
 //     (no block barrier on that path); a lane then picks its 4*NBITS bytes per K-iteration with
 //     one LDS read.  The scales and zero-points of a super are loaded with it and stay in registers.
-//   * Activations go global -> register ring -> LDS tile (three buffers per group, one block
-//     barrier per K-iteration) and are read in fragment order with ds_read_b128 (rows padded by
-//     16 bytes: conflict-free) one whole iteration before their MFMAs, so that no wave waits on
-//     LDS right behind a barrier (measured: the barrier-then-read stall was half of the kernel).
+//   * Activations go from global memory straight into LDS (global_load_lds_dwordx4: no register
+//     in between, no ds_write), PA tiles of BM x 64 ahead per group.  The only wait is an explicit
+//     s_waitcnt vmcnt(n) in front of the one block barrier per K-iteration, n being the number of
+//     younger loads of the wave, which stay in flight (measured 6-12 % faster at M = 128 .. 256
+//     than a register ring with ds_write, whose waits the compiler places itself).  Tiles are read
+//     in fragment order with ds_read_b128 (XOR-swizzled columns: conflict-free) one whole
+//     iteration before their MFMAs, so that no wave waits on LDS right behind a barrier (measured:
+//     the barrier-then-read stall was half of the kernel).
 //     Weights are MFMA source A (rows = n), activations source B (columns = m): a lane ends with
 //     groups of four consecutive n of one m -> 8-byte stores.
 #pragma once
@@ -33,8 +37,7 @@
 #include "qf_dequant.hip.h"
 
 // Timing experiments (results are wrong when non-zero): bit 0 skips the dequantisation arithmetic,
-// bit 1 the activation fragment reads, bit 2 the MFMAs, bit 3 the per-iteration barrier, bit 4 the
-// global activation loads, bit 5 the global weight / scale / zero loads.
+// bit 1 the activation fragment reads, bit 2 the MFMAs, bit 5 the global weight / scale / zero loads.
 #ifndef QF_GEMM_EXPERIMENT
 #define QF_GEMM_EXPERIMENT 0
 #endif
@@ -56,7 +59,7 @@ struct GemmCfg {
     static constexpr int NT32 = NT32_;                         // 32-row weight tiles per wave
     static constexpr int WN = WN_;                             // waves along N per group
     static constexpr int WK = WK_;                             // groups along K
-    static constexpr int PA = PA_;                             // activation tiles in flight (register ring)
+    static constexpr int PA = PA_;                             // activation tiles in flight towards LDS
     static constexpr int BK = 64;                              // K-iteration
     static constexpr int TN = 32 * NT32;                       // weight rows per wave
     static constexpr int BN = TN * WN;
@@ -77,7 +80,6 @@ struct GemmCfg {
     static constexpr int NGS = SUPK / GS > 0 ? SUPK / GS : 1;  // groups per row and super
     static constexpr int SREGS = (NGS + 1) / 2;                // registers of fp16 scales per tile and super
     static constexpr int ZBITS = NGS * ZFB;                    // zero-point bits per tile and super
-    static constexpr int PITCH = BK + 8;                       // activation tile row pitch in halves
     static constexpr int WPP = 128 + 16;                       // packed super row pitch in bytes
     static constexpr int RB = K * NBITS / 8;
     static constexpr int G = K / GS;
@@ -86,11 +88,16 @@ struct GemmCfg {
     static constexpr int HPP = 64 + 16;                        // 1-bit-plane super row pitch in bytes
     static constexpr int UPH = TN * 4 / 64;                    // its 16-byte units per lane and super
     static constexpr int GRID_X = (N + BN - 1) / BN;
-    static constexpr int NBUF = 3;                             // activation tiles in LDS per group
-    // fetch the activation fragments of tile it+1 during iteration it (a second register set of
-    // 16 * MT32 registers); tall tiles read each fragment just before its MFMAs instead
-    static constexpr bool PREFETCH_A = MT32 <= 4;
-    static constexpr size_t LDS_A = (size_t)WK * NBUF * BM * PITCH * 2;
+    // PREFETCH_A: fetch the activation fragments of tile it+1 during iteration it (a second register
+    // set of 16 * MT32 registers); tall tiles read each fragment just before its MFMAs instead
+    static constexpr bool PREFETCH_A = BM / 32 <= 4;
+    // activation tiles in LDS per group: the PA tiles in flight, plus the one being read when
+    // fragments are not prefetched
+    static constexpr int NBUF = PA + (PREFETCH_A ? 0 : 1);
+    static constexpr int ROWB = BK * 2;                        // bytes of one activation tile row in LDS
+    static constexpr size_t LDS_A = (size_t)WK * NBUF * BM * ROWB;
+    // vector-memory loads of one super per wave (packed words, 1-bit plane, scales, zero-points)
+    static constexpr int SUPER_LOADS = UPS + (HI ? UPH : 0) + NT32 * (SYM ? 1 : 2);
     static constexpr size_t LDS_W = (size_t)WK * WN * TN * (WPP + (HI ? HPP : 0));
     static constexpr size_t LDS_RED = WK > 1 ? (size_t)(WK - 1) * BM * BN * 4 : 0;
     static constexpr size_t LDS_FRONT = LDS_A > LDS_RED ? LDS_A : LDS_RED;
@@ -98,12 +105,54 @@ struct GemmCfg {
     static constexpr int ACC_PER_THREAD = MT32 * NT32 * 16;
 };
 
+template <int V> struct IntTag { static constexpr int value = V; };
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(IntTag<I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// s_waitcnt immediate of gfx9: vmcnt in bits 3:0 and 15:14, expcnt (not waited for) in 6:4, lgkmcnt in 11:8
+constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
+    const int vm = vmcnt > 63 ? 63 : vmcnt;
+    return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | ((lgkmcnt & 0xF) << 8);
+}
+
+// Wait until at most ALLOWED of this wave's vector-memory loads (in issue order) and none of its
+// LDS operations are outstanding, then meet the block's other waves.  A bare s_barrier: the
+// fence of __syncthreads() would wait for every outstanding load.
+template <int ALLOWED>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(ALLOWED, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// 16 bytes per lane from global memory straight into LDS (no register in between): lane l's
+// bytes land at lds + 16*l, `lds` being the same for the whole wave; counted by vmcnt like a load.
+__device__ __forceinline__ void load_to_lds_16(const void* global, void* lds) {
+    __builtin_amdgcn_global_load_lds(global, (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
+// Vector-memory loads a wave issues in the `back` iterations that end with iteration s (s counted
+// modulo the super): UA activation loads each, plus a whole super in the last iteration of a super.
+template <class C>
+constexpr int loads_since(int s, int back) {
+    int n = 0;
+    for (int d = 0; d < back; d++)
+        n += C::UA + ((((s - d) % C::SUP + C::SUP) % C::SUP == C::SUP - 1) ? C::SUPER_LOADS : 0);
+    return n;
+}
+
 template <class C>
 __global__ __launch_bounds__(C::T) void gemm_kernel(
     const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
     const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
     constexpr int BM = C::BM, BK = C::BK, WN = C::WN, WK = C::WK, TN = C::TN;
-    constexpr int MT32 = C::MT32, NT32 = C::NT32, PITCH = C::PITCH, WPP = C::WPP;
+    constexpr int MT32 = C::MT32, NT32 = C::NT32, WPP = C::WPP;
     constexpr int SUP = C::SUP, UPS = C::UPS, UA = C::UA, LW = C::LW, NGS = C::NGS, SREGS = C::SREGS;
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
 
@@ -114,11 +163,10 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     // base (advanced with scalar adds) plus a 32-bit per-lane offset computed once
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave % WN, grp = wave / WN;
-    const int tg = tid - grp * C::TG;                          // thread index inside the group
     const int li = lane & 31, kb = lane >> 5;
 
     // activation tiles live at the start of LDS (the final cross-group sum reuses that space)
-    uint16_t* as = reinterpret_cast<uint16_t*>(smem) + (size_t)grp * C::NBUF * BM * PITCH;   // [NBUF][BM][PITCH]
+    uint8_t* as_b = smem + (size_t)grp * C::NBUF * BM * C::ROWB;                           // [NBUF][BM][ROWB]
     uint8_t* wp = smem + C::LDS_FRONT + (size_t)wave * TN * (WPP + (C::HI ? C::HPP : 0));  // [TN][WPP] (+ [TN][HPP])
     uint8_t* hp = wp + TN * WPP;
 
@@ -148,29 +196,27 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         return sup * C::SUPK + (it % SUP) * BK;
     };
 
-    // ---- activations: UA 16-byte units per thread and iteration, register ring of depth PA ----
-    struct AStage { u32x4 a[UA]; };
-    uint32_t a_off[UA];                                        // byte offset of this thread's units inside the slab
+    // ---- activations: UA 16-byte units per lane and iteration, global memory -> LDS ----
+    // Instruction p of wave wn fills the 1 KB of 16-byte slots (p*WN + wn)*64 .. +63 of the tile
+    // (the hardware writes the 64 lanes' 16 bytes back to back); slot 8*row + (c ^ (row/2 % 8))
+    // holds columns 8c .. 8c+7 of a row: an XOR swizzle instead of row padding.  A 16-byte fragment
+    // read is served 16 lanes (= 16 rows, one column slot) at a time; rows 2a and 2a+1 start 32
+    // banks apart and the eight values of a move the slot to eight different 4-bank groups: no
+    // conflicts.
+    uint32_t a_off[UA];                                        // byte offset of this lane's units inside the slab
 #pragma unroll
     for (int p = 0; p < UA; p++) {
-        const int u = tg + p * C::TG;
-        const int row = min(u / (BK / 8), m_total - 1 - m_blk);   // rows past the end re-read the last one
-        a_off[p] = ((uint32_t)row * C::K + (u % (BK / 8)) * 8) * 2u;
+        const int u = (p * WN + wn) * 64 + lane;
+        const int row = u / 8, c8 = (u % 8) ^ ((row >> 1) & 7);
+        a_off[p] = ((uint32_t)min(row, m_total - 1 - m_blk) * C::K + c8 * 8) * 2u;   // rows past the end re-read the last one
     }
     const uint8_t* a_slab = reinterpret_cast<const uint8_t*>(A + (size_t)m_blk * C::K);
-    auto load_a = [&](AStage& st, int it) {
+    // tile `it` of the group into LDS buffer `buf`, asynchronously
+    auto load_a = [&](int buf, int it) {
         const uint8_t* base = a_slab + (size_t)k_of(it) * 2;
+        uint8_t* dst = as_b + (size_t)buf * BM * C::ROWB + (size_t)wn * 1024;
 #pragma unroll
-        for (int p = 0; p < UA; p++)
-            if (!(QF_GEMM_EXPERIMENT & 16)) st.a[p] = *reinterpret_cast<const u32x4*>(base + a_off[p]);
-    };
-    auto store_a = [&](const AStage& st, int buf) {
-#pragma unroll
-        for (int p = 0; p < UA; p++) {
-            const int u = tg + p * C::TG;
-            const int row = u / (BK / 8), col = (u % (BK / 8)) * 8;
-            *reinterpret_cast<u32x4*>(as + ((size_t)buf * BM + row) * PITCH + col) = st.a[p];
-        }
+        for (int p = 0; p < UA; p++) load_to_lds_16(base + a_off[p], dst + (size_t)p * WN * 1024);
     };
 
     // ---- one super of this wave's TN weight rows: packed fields, scales, zero-points ----
@@ -304,7 +350,12 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             for (int v = 0; v < 16; v++) acc[j][i][v] = 0.0f;
 
     // activation fragments of one tile: k-step ks of 32-row block i is row li, columns 32*kb + 8*ks .. + 7
-    const uint16_t* a_frag_base = as + (size_t)li * PITCH + 32 * kb;
+    uint32_t a_frag_off[4];                                    // swizzled byte offset of k-step ks
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) a_frag_off[ks] = (uint32_t)li * C::ROWB + (((4 * kb + ks) ^ ((li >> 1) & 7)) * 16);
+    auto frag_of = [&](int buf, int i, int ks) {
+        return *reinterpret_cast<const f16x8*>(as_b + ((size_t)buf * BM + i * 32) * C::ROWB + a_frag_off[ks]);
+    };
     struct AFrags { f16x8 f[MT32][4]; };
     auto read_frags = [&](AFrags& fr, int buf) {
 #pragma unroll
@@ -312,24 +363,26 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 if (QF_GEMM_EXPERIMENT & 2) fr.f[i][ks] = __builtin_bit_cast(f16x8, u32x4{(uint32_t)buf, 1u, 2u, 3u});
-                else fr.f[i][ks] = *reinterpret_cast<const f16x8*>(a_frag_base + ((size_t)buf * BM + i * 32) * PITCH + ks * 8);
+                else fr.f[i][ks] = frag_of(buf, i, ks);
             }
     };
 
-    AStage ringA[C::PA];        // slot t % PA holds activation tile t on its way to LDS
     WStage ringW[2];
     Packed cur, nxt;
     Quant qcur;
     AFrags fcur, fnxt;
 
-    // One K-iteration; s = it % (2*SUP) is a compile-time constant at every call site; b1 and b2
-    // are the LDS buffers (of NBUF = 3) of tiles it+1 and it+2.
+    // One K-iteration; s = it % (2*SUP) is a compile-time constant at every call site; b0, b1 and
+    // b2 are the LDS buffers of tiles it, it+1 and it+PA (tile t lives in buffer t % NBUF).
     //   * the fragments of tile it+1 (complete in LDS since the last barrier) are fetched now and
     //     used in the next iteration: no wave waits on LDS right after a barrier;
-    //   * tile it+2 goes from its ring slot to LDS, and the slot takes the load of tile it+2+PA;
     //   * the MFMAs of tile it run on registers filled one iteration ago, interleaved with the
-    //     dequantisation of their weight fragments.
-    auto iteration = [&](int it, int s, int b0, int b1, int b2) {
+    //     dequantisation of their weight fragments;
+    //   * tile it+PA is requested into the buffer whose tile every wave has finished reading
+    //     before the last barrier; past the end of K the last tile is requested again, so that
+    //     the count of loads in flight stays what the waits below assume.
+    auto iteration = [&](int it, auto s_tag, int b0, int b1, int b2) {
+        constexpr int s = decltype(s_tag)::value;
         const int q = s % SUP, pslot = (s / SUP) & 1;
         const int P = it / SUP;                                 // super index inside the group
         if constexpr (C::PREFETCH_A) read_frags(fnxt, b1);
@@ -346,7 +399,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 for (int i = 0; i < MT32; i++) {
                     if constexpr (C::PREFETCH_A) af[i] = fcur.f[i][ks];
                     else if (QF_GEMM_EXPERIMENT & 2) af[i] = __builtin_bit_cast(f16x8, u32x4{(uint32_t)b0, 1u, 2u, 3u});
-                    else af[i] = *reinterpret_cast<const f16x8*>(a_frag_base + ((size_t)b0 * BM + i * 32) * PITCH + ks * 8);
+                    else af[i] = frag_of(b0, i, ks);
                 }
 #pragma unroll
                 for (int j = 0; j < NT32; j++) {
@@ -374,8 +427,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                         else acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[j][i], 0, 0, 0);
             }
         }
-        store_a(ringA[(s + 2) % C::PA], b2);
-        load_a(ringA[(s + 2) % C::PA], min(it + 2 + C::PA, C::ITERS - 1));
+        load_a(b2, min(it + C::PA, C::ITERS - 1));
         cur = nxt;
         if constexpr (C::PREFETCH_A) fcur = fnxt;
         if (q == SUP - 1) {
@@ -383,37 +435,43 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             qcur = ringW[pslot ^ 1].q;
             load_super(ringW[pslot ^ 1], P + 3);
         }
-        if (!(QF_GEMM_EXPERIMENT & 8)) __syncthreads();
+        // Publish the tile the next iteration reads (tile it+2 with fragment prefetch, else it+1):
+        // it was requested PA - W iterations ago, and every vector-memory load the wave has issued
+        // in the iterations since (activation tiles and whole supers) may stay in flight.  Loads
+        // return in order; the supers of the requesting iteration itself are not counted, wherever
+        // the compiler places them relative to the request.
+        constexpr int W = C::PREFETCH_A ? 2 : 1;
+        wait_loads_and_barrier<loads_since<C>(s, C::PA - W)>();
     };
 
-    // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA+1 in flight, tiles 0 and 1 in LDS ----
+    // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----
     load_super(ringW[0], 0);
     load_super(ringW[1], 1);
 #pragma unroll
-    for (int p = 0; p < C::PA; p++) load_a(ringA[p], min(p, C::ITERS - 1));
+    for (int p = 0; p < C::PA; p++) load_a(p, min(p, C::ITERS - 1));
     store_super(ringW[0]);
     qcur = ringW[0].q;
     load_super(ringW[0], 2);
     read_packed(cur, 0);
-    store_a(ringA[0], 0);
-    store_a(ringA[1 % C::PA], 1);
-    load_a(ringA[0], min(C::PA, C::ITERS - 1));
-    load_a(ringA[1 % C::PA], min(C::PA + 1, C::ITERS - 1));
-    __syncthreads();
+    wait_loads_and_barrier<0>();
     if constexpr (C::PREFETCH_A) read_frags(fcur, 0);
 
-    int b0 = 0, b1 = 1, b2 = 2;
+    int b0 = 0, b1 = 1, b2 = C::PA % C::NBUF;
 #pragma unroll 1
     for (int it0 = 0; it0 < C::ITERS; it0 += 2 * SUP) {
-#pragma unroll
-        for (int s = 0; s < 2 * SUP; s++)
+        static_for<0, 2 * SUP>([&](auto s_tag) {
+            constexpr int s = decltype(s_tag)::value;
             if (it0 + s < C::ITERS) {
-                iteration(it0 + s, s, b0, b1, b2);
+                iteration(it0 + s, s_tag, b0, b1, b2);
                 b0 = b1;
-                b1 = b2;
+                b1 = b1 == C::NBUF - 1 ? 0 : b1 + 1;
                 b2 = b2 == C::NBUF - 1 ? 0 : b2 + 1;
             }
+        });
     }
+    // the repeated activation requests of the last iterations still target LDS: drain them before
+    // the space is reused below or the wave ends
+    wait_loads_and_barrier<0>();
 
     // ---- the groups' partial sums meet in LDS (the activation tiles are no longer needed) ----
     if constexpr (WK > 1) {
@@ -483,7 +541,7 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::NGS > 8 || C::ZBITS > 32) why = "too many groups per 128 packed bytes";
     else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if ((C::BM * (C::BK / 8)) % C::TG != 0) why = "the activation tile must split evenly over a group's threads";
-    else if (C::PA < 2 || (2 * C::SUP) % C::PA != 0) why = "PA must be >= 2 and divide 2048/NBITS/64";
+    else if (C::PA < 3 || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12";
     else if (C::LDS_BYTES > 160 * 1024) why = "tiles exceed the 160 KB of LDS";
     else if (C::ACC_PER_THREAD > 256) why = "accumulator tile exceeds the register file";
     if (why) {
