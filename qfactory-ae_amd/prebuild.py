@@ -49,6 +49,14 @@ def parity_cases():
     cases += [_case(33, 100, 512, 4, 128), _case(100, 1000, 1024, 4, 64), _case(300, 256, 2048, 4, 128),
               _case(48, 130, 1024, 2, 64), _case(17, 96, 512, 8, 32), _case(64, 512, 1024, 4, 128, True),
               _case(128, 256, 11008, 4, 128)]
+    # streaming skinny regime (3 <= M <= 16, K too long for resident activations): ragged M and N,
+    # a last wave with dead steps (43 steps over 8 waves), group per lane / per chunk / per step, 2 and 8 bits
+    cases += [_case(5, 100, 11008, 4, 128), _case(3, 77, 11008, 4, 32), _case(7, 130, 11008, 4, 64, True),
+              _case(16, 272, 14336, 4, 256), _case(12, 48, 14336, 2, 256), _case(16, 64, 14336, 2, 512, True),
+              _case(9, 64, 8192, 8, 128), _case(4, 100, 8192, 8, 64), _case(11, 40, 11008, 8, 32, True),
+              _case(8, 8200, 11008, 4, 128)]
+    # 2-bit at K = 4096: the A-stationary kernel's 16-wave tiling does not fit LDS, 8 waves do
+    cases += [_case(16, 100, 4096, 2, 128), _case(32, 48, 4096, 2, 64, True)]
     return cases
 
 

@@ -105,6 +105,8 @@ class QMatmulQFunc(QFunc):
             return tiling.gemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "mgemv":
             return tiling.mgemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
+        if regime == "skinny":
+            return tiling.skinny_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "gemm":
             return tiling.gemm_tiling(p["M"], p["N"], p["K"], nbits, gs)
         return tiling.mfma_tiling(p["M"], p["N"], p["K"], nbits, gs)
@@ -131,6 +133,8 @@ class QMatmulQFunc(QFunc):
             cands = tiling.gemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         elif self.regime == "mgemv":
             cands = tiling.mgemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
+        elif self.regime == "skinny":
+            cands = tiling.skinny_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         elif self.regime == "gemm":
             cands = tiling.gemm_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         else:
@@ -144,7 +148,7 @@ class QMatmulQFunc(QFunc):
         b = lambda x: "true" if x else "false"
         code = "// QFactory-HIP generated translation unit\n\n"
         defines = dict(getattr(self, "defines", {}))                        # kernel-header tuning knobs
-        if self.regime in ("gemm", "mgemv"):
+        if self.regime in ("gemm", "mgemv", "skinny"):
             # the matrix-core kernels expose their dequantisation's vector-instruction issue and have
             # registers to spare: the one-instruction mask-and-merge decode pays there (2 - 7 %
             # measured); it does not in the 4-bit GEMV kernel, where it costs a resident wave
@@ -163,6 +167,10 @@ class QMatmulQFunc(QFunc):
             code += '#include "qf_mgemv.hip.h"\n'
             cfg = tiling.mgemv_cfg_string(p, t, not self.l2cache_b)
             call = "qf::mgemv_launch<Cfg>"
+        elif self.regime == "skinny":
+            code += '#include "qf_skinny.hip.h"\n'
+            cfg = tiling.skinny_cfg_string(p, t, not self.l2cache_b)
+            call = "qf::skinny_launch<Cfg>"
         elif self.regime == "gemm":
             code += '#include "qf_gemm.hip.h"\n'
             cfg = tiling.gemm_cfg_string(p, t, not self.l2cache_b)

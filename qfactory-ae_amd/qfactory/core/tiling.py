@@ -4,7 +4,7 @@ This is the analytic half of what the reference does by brute force (``QMatmulQF
 qfactory/core/qfunc.py:110-131, enumerates BLOCK_N x BLOCK_SIZE x NUM_ELM and times all of them):
 given the problem it proposes one default tiling and a short list of neighbours worth timing.
 
-Four kernel families (``regime_for`` picks one):
+Five kernel families (``regime_for`` picks one):
 
 * ``gemv``  -- M < 3 (and 3-bit M <= 2), HBM-bound, v_dot2.  Parameters of ``qf::GemvCfg``
   (include/qf_gemv.hip.h): ``MT`` activation rows per block, ``WK`` waves along K per team, ``WN``
@@ -13,6 +13,9 @@ Four kernel families (``regime_for`` picks one):
 * ``mgemv`` -- 3 <= M <= 32 when the activations fit the register file: persistent A-stationary MFMA
   kernel, ``qf::MGemvCfg`` (include/qf_mgemv.hip.h): ``MT16`` 16-row activation tiles, ``WK`` waves x
   ``CH`` chunks covering K, ``PB`` blocks, ``PF`` weight tiles in flight.
+* ``skinny`` -- 3 <= M <= 16 where ``mgemv`` cannot hold the activations (K = 11008, 8-bit K = 8192 ...):
+  ``qf::SkinnyCfg`` (include/qf_skinny.hip.h): activations streamed per K-step instead of resident,
+  ``WK`` waves splitting K, ``SB`` tiles per batch, ``D`` stages in flight, ``AST`` resident fragments.
 * ``gemm``  -- larger M (and what ``mgemv`` cannot hold): ``qf::GemmCfg`` (include/qf_gemm.hip.h):
   ``BM`` activation rows per block, ``NT32`` 32-row weight tiles per wave, ``WN`` waves along N,
   ``WK`` wave groups along K, ``PA`` activation tiles in flight.
@@ -38,6 +41,8 @@ def regime_for(M, K=None, nbits=None, group_size=None):
         return "gemv"
     if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
         return "mgemv"
+    if skinny_preferred(M, K, nbits, group_size):
+        return "skinny"
     if M <= GEMV_MAX_M:
         return "gemv"
     # above 32 rows, or when the A-stationary kernel cannot hold the activations of this K in
@@ -234,6 +239,13 @@ def mgemv_regs(mt16, ch, pf, nbits):
     return mt16 * ch * ksteps * 4 + pf * (ch * 4 + 4) + ch * 4 + 48
 
 
+def mgemv_lds_bytes(mt16, wk, ch, nbits, sb=4):
+    """LDS of qf::mgemv_kernel: SB partial tiles per wave plus the wave's transposition buffer."""
+    chunk = 4 * (128 // nbits)
+    wbuf = max(16 * (ch * 64 + 16), 16 * (chunk * 2 + 16))
+    return wk * sb * mt16 * 1024 + wk * wbuf
+
+
 def mgemv_reg_limit(wk):
     waves_per_simd = -(-wk // 4)
     return min(512, 512 // waves_per_simd)
@@ -259,6 +271,8 @@ def mgemv_tiling(M, N, K, nbits, group_size, max_waves=16, **pins):
         for pf in (2, 4, 1):
             if mgemv_regs(mt16, ch, pf, nbits) > mgemv_reg_limit(wk):
                 continue
+            if mgemv_lds_bytes(mt16, wk, ch, nbits) > 160 * 1024:
+                continue
             waste = wk * ch - nchunk
             key = (waste > ch // 2, -wk, pf != 2, waste)      # more, thinner waves measured best on MI355X
             if best is None or key < best[0]:
@@ -282,7 +296,8 @@ def mgemv_candidates(M, N, K, nbits, group_size):
         key = tuple(sorted(cfg.items()))
         ok = (cfg["WK"] <= 16 and cfg["WK"] * cfg["CH"] >= nchunk and (cfg["WK"] - 1) * cfg["CH"] < nchunk
               and cfg["CH"] <= nchunk
-              and mgemv_regs(cfg["MT16"], cfg["CH"], cfg["PF"], nbits) <= mgemv_reg_limit(cfg["WK"]))
+              and mgemv_regs(cfg["MT16"], cfg["CH"], cfg["PF"], nbits) <= mgemv_reg_limit(cfg["WK"])
+              and mgemv_lds_bytes(cfg["MT16"], cfg["WK"], cfg["CH"], nbits) <= 160 * 1024)
         if ok and key not in seen:
             seen.add(key)
             out.append(cfg)
@@ -300,6 +315,134 @@ def mgemv_cfg_string(problem, t, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::MGemvCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
             f"{t['MT16']}, {t['WK']}, {t['CH']}, {t['PB']}, {t['PF']}, {b(nt_b)}>")
+
+
+# --------------------------------------------------------------------------------------------
+# Skinny MFMA regime (3 <= M <= 32): qf::SkinnyCfg (include/qf_skinny.hip.h) -- every load lands in
+# fragment order, WK waves split K in steps of 128 packed bytes, SB tiles per batch, D stages in flight
+# --------------------------------------------------------------------------------------------
+
+def skinny_supported(K, nbits, group_size):
+    if nbits not in (2, 4, 8) or not group_size or group_size <= 0:
+        return False
+    epl = 128 // nbits
+    chunk, stepk = 4 * epl, 8 * epl
+    if K % stepk or K % group_size or group_size % epl:
+        return False
+    if (group_size % stepk) if group_size >= stepk else (chunk % group_size):
+        return False
+    return (K // group_size) % (8 // nbits) == 0
+
+
+SKINNY_MAX_M = 16
+SKINNY_MAX_K = 16384
+
+
+def skinny_preferred(M, K, nbits, group_size):
+    """The streaming kernel takes the rows-of-16 problems whose activations the A-stationary kernel
+    cannot keep in registers (K = 11008 or 14336 at 4 bits, K = 8192 or 11008 at 8 bits).  Measured at
+    M = 4 .. 16 on 4096 x 11008: 10.7 .. 13.2 us against 13.9 .. 21.7 us for the kernels that served it
+    before (8-bit: 17.4 against 28.6).  Every block streams all of the activations, M x K x 2 bytes:
+    at K = 28672 that is twice the block's weight bytes and the GEMM kernel wins (49 against 109 us),
+    as it does above 16 rows."""
+    if not (MGEMV_MIN_M <= M <= SKINNY_MAX_M) or K > SKINNY_MAX_K:
+        return False
+    return skinny_tiling(M, 16 * NUM_CUS, K, nbits, group_size) is not None
+
+
+def skinny_regs(cfg, nbits, spw):
+    """Rough VGPR need of qf::skinny_kernel: D stages (coalesced activation rows unless resident,
+    packed words), the activation fragments in use (all the wave's steps when AST), the batch's
+    scales and zero-points twice, accumulators, ~48 of addresses and temporaries."""
+    stepk = 8 * (128 // nbits)
+    a_step = cfg["MT16"] * stepk // 8                  # registers of one activation step (16 rows x STEPK halves / 64 lanes)
+    stage = (0 if cfg["AST"] else a_step) + cfg["SB"] * 8
+    quant = 2 * cfg["SB"] * 2 * spw
+    frags = spw * a_step if cfg["AST"] else a_step
+    return cfg["D"] * stage + frags + quant + cfg["SB"] * cfg["MT16"] * 8 + 48
+
+
+def skinny_lds_bytes(cfg, nbits):
+    stepk = 8 * (128 // nbits)
+    return 2 * cfg["WK"] * cfg["SB"] * cfg["MT16"] * 1024 + cfg["WK"] * cfg["MT16"] * 16 * (stepk * 2 + 16)
+
+
+def skinny_valid(cfg, N, K, nbits, group_size):
+    import math
+    if not skinny_supported(K, nbits, group_size):
+        return False
+    mt16, wk, sb, d = cfg["MT16"], cfg["WK"], cfg["SB"], cfg["D"]
+    nstep = K // (8 * (128 // nbits))
+    spw = -(-nstep // wk)
+    if not (1 <= mt16 <= 2 and 1 <= wk <= 16 and 1 <= sb <= 8 and 1 <= d <= 4):
+        return False
+    if (wk - 1) * spw >= nstep or math.lcm(spw, d) > 32:
+        return False
+    if skinny_lds_bytes(cfg, nbits) > 160 * 1024:
+        return False
+    return skinny_regs(cfg, nbits, spw) <= min(512, 512 // -(-wk // 4))
+
+
+def skinny_tiling(M, N, K, nbits, group_size, **pins):
+    """Default tiling (None if the kernel does not cover the problem), from on-device sweeps at
+    M = 16: eight waves per block; one tile per batch unless a block sweeps four or more; the
+    activation fragments stay resident when a block has several batches and they fit; two stages
+    in flight."""
+    if not skinny_supported(K, nbits, group_size) or M > 32:
+        return None
+    mt16 = -(-M // 16)
+    nstep = K // (8 * (128 // nbits))
+    nt = -(-N // 16)
+    slots = -(-nt // min(nt, NUM_CUS))
+    best = None
+    for wk in range(min(8, nstep), 0, -1):
+        spw = -(-nstep // wk)
+        if (wk - 1) * spw >= nstep:
+            continue
+        waste = (wk * spw - nstep) / nstep
+        for sb in ((2, 1) if slots >= 4 else (1,)):
+            nbatch = -(-slots // sb)
+            for ast in ((1, 0) if nbatch > 1 else (0,)):
+                for d in (2, 1):
+                    cfg = {"MT16": mt16, "WK": wk, "SB": sb, "D": d, "AST": ast, "PB": NUM_CUS}
+                    if not skinny_valid(cfg, N, K, nbits, group_size):
+                        continue
+                    key = (waste > 0.13, -wk, -ast, -sb, -d)
+                    if best is None or key < best[0]:
+                        best = (key, cfg)
+    if best is None:
+        return None
+    cfg = best[1]
+    cfg.update(pins)
+    return cfg
+
+
+def skinny_candidates(M, N, K, nbits, group_size):
+    base = skinny_tiling(M, N, K, nbits, group_size)
+    if base is None:
+        return []
+    seen, out = set(), []
+
+    def add(cfg):
+        key = tuple(sorted(cfg.items()))
+        if key not in seen and skinny_valid(cfg, N, K, nbits, group_size):
+            seen.add(key)
+            out.append(cfg)
+
+    add(base)
+    for wk in (16, 14, 12, 11, 8, 7, 6, 4):
+        for sb in (1, 2, 4):
+            for d in (1, 2, 3):
+                for ast in (0, 1):
+                    for pb in (NUM_CUS, 2 * NUM_CUS):
+                        add({"MT16": base["MT16"], "WK": wk, "SB": sb, "D": d, "AST": ast, "PB": pb})
+    return out
+
+
+def skinny_cfg_string(problem, t, nt_b):
+    b = lambda x: "true" if x else "false"
+    return (f"qf::SkinnyCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
+            f"{t['MT16']}, {t['WK']}, {t['SB']}, {t['D']}, {b(t['AST'])}, {t['PB']}, {b(nt_b)}>")
 
 
 # --------------------------------------------------------------------------------------------
