@@ -464,12 +464,13 @@ def gemm_lds_bytes(cfg, nbits=4):
 
 def gemm_regs(cfg):
     """Rough VGPR need of one lane: accumulators, two sets of activation fragments, the weight
-    super ring, plus ~80 of addresses and dequantisation temporaries.  A SIMD has 512 per lane to
+    super ring, plus ~50 of addresses and dequantisation temporaries (compiled: 192 for 64 x 32 wave
+    tiles with two groups, 250 for 256 x 32 ones).  A SIMD has 512 per lane to
     share between the waves a block puts on it (spills are ruinous)."""
     mt32, nt32 = cfg["BM"] // 32, cfg["NT32"]
     ua = max(1, cfg["BM"] * 8 // (64 * cfg["WN"]))
     frag_sets = 2 if mt32 <= 4 else 0.25               # tall tiles keep one k-step of fragments, not two tiles
-    return int(mt32 * nt32 * 16 + frag_sets * mt32 * 16 + 2 * nt32 * 20 + ua + 80)
+    return int(mt32 * nt32 * 16 + frag_sets * mt32 * 16 + 2 * nt32 * 20 + ua + 50)
 
 
 def gemm_valid(cfg, K, nbits, group_size):
@@ -490,7 +491,7 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     if (K // group_size) % (8 // zfb):
         return False
-    if (bm * 8) % (64 * wn) or not 3 <= pa <= 12:
+    if (bm * 8) % (64 * wn) or not (3 if bm // 32 <= 4 else 2) <= pa <= 12:
         return False
     if (bm // 32) * nt32 * 16 > 256:
         return False
@@ -509,19 +510,19 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     ceil(blocks / CUs) rounds of one tile's work, and a tile costs its area plus a fixed overhead
     (pipeline fill, reduction, barriers) worth about 2048 outputs.  It reproduces the measured
     winners: 64 x 128 tiles on 8192-wide, 128 x 128 on 10240-wide (160 tiles in one round beat 320
-    in two) and 128 x 256 on 57344-wide layers at M = 256; 32 x 32 ... 64 x 64 tiles for M <= 128."""
+    in two) and 256 x 256 on 57344-wide layers at M = 256; 32 x 32 ... 64 x 64 tiles for M <= 128."""
     import math
     best = None
-    for bm in (128, 64, 32):
+    for bm in (256, 128, 64, 32):
         if bm >= 2 * M and bm > 32:
             continue
-        for wn in (4, 2, 1):
+        # 256-row tiles: eight waves side by side (a 256 x 256 block tile, every weight dequantised
+        # once); measured 250 against 300 us on 57344 x 8192 at M = 256
+        for wn in ((8,) if bm == 256 else (4, 2, 1)):
             for nt32 in ((1, 2) if (bm, wn) == (128, 4) else (1,)):
                 bn = 32 * wn * nt32
                 blocks = -(-N // bn) * -(-M // bm)
                 rounds = -(-blocks // NUM_CUS)
-                # (256-row tiles, which dequantise every weight once, measured no faster: the
-                # kernel is bound by load waits, not by the dequantisation)
                 cost = rounds * (bm * bn + 2048)
                 key = (cost, abs(math.log2(bm / bn)), -bn)
                 if best is None or key < best[0]:
@@ -530,9 +531,11 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     # with at most one block per CU the K axis is split over wave groups inside the block, so
     # that every SIMD still holds two waves (one dequantises while the other multiplies)
     wk = max(1, 8 // wn) if blocks <= NUM_CUS else 1
+    if bm == 256:
+        wk = 1
     nsup = K // (1024 // plane_bits(nbits))
     wk = max(1, min(wk, nsup))
-    pa = 4
+    pa = 4 if bm <= 128 else 2                        # tall tiles: LDS holds PA + 1 of them
     while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
         if pa == 4:
             pa = 3                                    # one activation tile less in LDS
@@ -559,9 +562,9 @@ def gemm_candidates(M, N, K, nbits, group_size):
         if bm >= 2 * M and bm > 32:
             continue
         for nt32 in (1, 2):
-            for wn in (1, 2, 4):
+            for wn in (1, 2, 4, 8):
                 for wk in (1, 2, 4, 8):
-                    for pa in (3, 4, 6):
+                    for pa in (2, 3, 4, 6):
                         add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})
     return out
 

@@ -541,7 +541,7 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::NGS > 8 || C::ZBITS > 32) why = "too many groups per 128 packed bytes";
     else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if ((C::BM * (C::BK / 8)) % C::TG != 0) why = "the activation tile must split evenly over a group's threads";
-    else if (C::PA < 3 || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12";
+    else if (C::PA < (C::PREFETCH_A ? 3 : 2) || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12 (2 .. 12 for tiles taller than 128 rows)";
     else if (C::LDS_BYTES > 160 * 1024) why = "tiles exceed the 160 KB of LDS";
     else if (C::ACC_PER_THREAD > 256) why = "accumulator tile exceeds the register file";
     if (why) {
