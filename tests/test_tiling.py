@@ -1,0 +1,97 @@
+"""Host-side tiling logic (no GPU): regime routing, and that every default tiling the package would
+compile satisfies the static limits its kernel checks at launch (registers, LDS, divisibility)."""
+import math
+
+import pytest
+
+import prebuild
+from qfactory.core import tiling
+
+
+def _cases():
+    return [c for c in prebuild.all_cases() if c["GS"] != -1]
+
+
+def _id(c):
+    return f"M{c['M']}-N{c['N']}-K{c['K']}-b{c['NBITS']}-g{c['GS']}"
+
+
+@pytest.mark.parametrize("M,K,nbits,gs,expected", [
+    (1, 4096, 4, 128, "gemv"), (2, 11008, 4, 128, "gemv"),
+    (3, 4096, 4, 128, "mgemv"), (16, 8192, 4, 128, "mgemv"), (32, 4096, 4, 128, "mgemv"),
+    (16, 4096, 2, 128, "mgemv"), (16, 4096, 8, 128, "mgemv"),
+    (4, 11008, 4, 128, "skinny"), (16, 11008, 4, 128, "skinny"), (16, 14336, 4, 128, "skinny"),
+    (16, 8192, 8, 128, "skinny"), (16, 11008, 8, 128, "skinny"),
+    (17, 11008, 4, 128, "gemm"), (16, 28672, 4, 128, "gemm"), (32, 8192, 4, 128, "gemm"),
+    (64, 4096, 4, 128, "gemm"), (256, 8192, 4, 128, "gemm"),
+    (1, 8192, 3, 128, "gemv"), (2, 8192, 3, 128, "gemv"), (16, 8192, 3, 128, "gemm"),
+    (33, 2048, 3, 128, "gemm"),
+])
+def test_regime_routing(M, K, nbits, gs, expected):
+    assert tiling.regime_for(M, K, nbits, gs) == expected
+
+
+@pytest.mark.parametrize("case", _cases(), ids=_id)
+def test_default_tiling_respects_the_kernel_limits(case):
+    M, N, K, nbits, gs = (case[k] for k in ("M", "N", "K", "NBITS", "GS"))
+    regime = tiling.regime_for(M, K, nbits, gs)
+    if regime == "mgemv":
+        t = tiling.mgemv_tiling(M, N, K, nbits, gs)
+        chunk = 4 * (128 // nbits)
+        nchunk = K // chunk
+        assert t["WK"] * t["CH"] >= nchunk and (t["WK"] - 1) * t["CH"] < nchunk and t["WK"] <= 16
+        assert tiling.mgemv_lds_bytes(t["MT16"], t["WK"], t["CH"], nbits) <= 160 * 1024
+        assert tiling.mgemv_regs(t["MT16"], t["CH"], t["PF"], nbits) <= tiling.mgemv_reg_limit(t["WK"])
+    elif regime == "skinny":
+        t = tiling.skinny_tiling(M, N, K, nbits, gs)
+        assert t is not None and tiling.skinny_valid(t, N, K, nbits, gs)
+        nstep = K // (8 * (128 // nbits))
+        spw = -(-nstep // t["WK"])
+        assert t["MT16"] == 1 and (t["WK"] - 1) * spw < nstep <= t["WK"] * spw
+        assert math.lcm(spw, t["D"]) <= 32
+        assert tiling.skinny_lds_bytes(t, nbits) <= 160 * 1024
+    elif regime == "gemm":
+        t = tiling.gemm_tiling(M, N, K, nbits, gs)
+        assert tiling.gemm_valid(t, K, nbits, gs), t
+        assert tiling.gemm_lds_bytes(t, nbits) <= 160 * 1024
+        assert 64 * t["WN"] * t["WK"] <= 1024
+        assert t["PA"] >= (3 if t["BM"] <= 128 else 2)
+    elif regime == "gemv":
+        t = tiling.gemv_tiling(M, N, K, nbits, gs)
+        assert t["VB"] in (4, 8, 16) and 64 * t["WK"] * t["WN"] <= 1024
+    else:
+        assert regime == "mfma"
+
+
+def test_two_bit_k4096_mgemv_fits_lds():
+    # sixteen waves with 2-bit chunks (512 B of activations per row) would need 199 KB of LDS
+    for M in (3, 16, 32):
+        t = tiling.mgemv_tiling(M, 22016, 4096, 2, 128)
+        assert t is not None and tiling.mgemv_lds_bytes(t["MT16"], t["WK"], t["CH"], 2) <= 160 * 1024
+
+
+def test_skinny_is_not_chosen_where_it_measured_slower():
+    assert not tiling.skinny_preferred(16, 28672, 4, 128)        # activations per block twice the weight bytes
+    assert not tiling.skinny_preferred(17, 11008, 4, 128)        # two 16-row tiles spill
+    assert not tiling.skinny_preferred(2, 11008, 4, 128)         # dot2 GEMV territory
+    assert tiling.skinny_tiling(16, 4096, 11008, 2, 128) is None  # 11008 is not a multiple of a 2-bit step
+
+
+def test_wide_layers_get_256_row_tiles_only_when_they_fill_the_machine():
+    assert tiling.gemm_tiling(256, 57344, 8192, 4, 128)["BM"] == 256
+    assert tiling.gemm_tiling(256, 8192, 8192, 4, 128)["BM"] < 256
+    assert tiling.gemm_tiling(64, 57344, 8192, 4, 128)["BM"] <= 64
+
+
+@pytest.mark.parametrize("regime,M,N,K,nbits", [("gemv", 1, 512, 1024, 4), ("mgemv", 16, 384, 1024, 4),
+                                                ("skinny", 9, 64, 8192, 8), ("gemm", 64, 384, 1024, 4)])
+def test_emit_names_the_kernel_of_the_regime(regime, M, N, K, nbits):
+    import torch
+    from qfactory.core.qfunc import QMatmulQFunc
+    from qfactory.core.qtile import QTile, AsymQTile
+    q = QMatmulQFunc(QTile((M, K), torch.float16, 16), AsymQTile((N, K), torch.int8, nbits, (1, 128)), "nt")
+    assert q.regime == regime
+    code = q.emit()
+    header = {"gemv": "qf_gemv.hip.h", "mgemv": "qf_mgemv.hip.h", "skinny": "qf_skinny.hip.h", "gemm": "qf_gemm.hip.h"}[regime]
+    assert f'#include "{header}"' in code and f"regime={regime}" in code
+    assert 'extern "C"' in code and "launch_m" in code
