@@ -456,8 +456,7 @@ GEMM_BK = 64
 def gemm_lds_bytes(cfg, nbits=4):
     bm, nt32, wn, wk = cfg["BM"], cfg["NT32"], cfg["WN"], cfg["WK"]
     bn = 32 * nt32 * wn
-    nbuf = cfg["PA"] + (0 if bm // 32 <= 4 else 1)     # tiles in flight (+ the one being read when fragments are not prefetched)
-    lds_a = wk * nbuf * bm * GEMM_BK * 2
+    lds_a = wk * cfg["PA"] * bm * GEMM_BK * 2
     lds_red = (wk - 1) * bm * bn * 4
     return max(lds_a, lds_red) + wk * wn * 32 * nt32 * (144 + (80 if nbits == 3 else 0))
 
@@ -491,7 +490,7 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     if (K // group_size) % (8 // zfb):
         return False
-    if (bm * 8) % (64 * wn) or not (3 if bm // 32 <= 4 else 2) <= pa <= 12:
+    if (bm * 8) % (64 * wn) or not 3 <= pa <= 12:
         return False
     if (bm // 32) * nt32 * 16 > 256:
         return False
@@ -535,7 +534,7 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
         wk = 1
     nsup = K // (1024 // plane_bits(nbits))
     wk = max(1, min(wk, nsup))
-    pa = 4 if bm <= 128 else 2                        # tall tiles: LDS holds PA + 1 of them
+    pa = 4
     while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
         if pa == 4:
             pa = 3                                    # one activation tile less in LDS
@@ -564,7 +563,7 @@ def gemm_candidates(M, N, K, nbits, group_size):
         for nt32 in (1, 2):
             for wn in (1, 2, 4, 8):
                 for wk in (1, 2, 4, 8):
-                    for pa in (2, 3, 4, 6):
+                    for pa in (3, 4, 6):
                         add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})
     return out
 

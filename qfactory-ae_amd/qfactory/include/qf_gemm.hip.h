@@ -22,7 +22,7 @@
 //     (no block barrier on that path); a lane then picks its 4*NBITS bytes per K-iteration with
 //     one LDS read.  The scales and zero-points of a super are loaded with it and stay in registers.
 //   * Activations go from global memory straight into LDS (global_load_lds_dwordx4: no register
-//     in between, no ds_write), PA tiles of BM x 64 ahead per group.  The only wait is an explicit
+//     in between, no ds_write), PA tiles of BM x 64 in LDS per group.  The only wait is an explicit
 //     s_waitcnt vmcnt(n) in front of the one block barrier per K-iteration, n being the number of
 //     younger loads of the wave, which stay in flight (measured 6-12 % faster at M = 128 .. 256
 //     than a register ring with ds_write, whose waits the compiler places itself).  Tiles are read
@@ -91,9 +91,11 @@ struct GemmCfg {
     // PREFETCH_A: fetch the activation fragments of tile it+1 during iteration it (a second register
     // set of 16 * MT32 registers); tall tiles read each fragment just before its MFMAs instead
     static constexpr bool PREFETCH_A = BM / 32 <= 4;
-    // activation tiles in LDS per group: the PA tiles in flight, plus the one being read when
-    // fragments are not prefetched
-    static constexpr int NBUF = PA + (PREFETCH_A ? 0 : 1);
+    // activation tiles in LDS per group: tile t lives in buffer t % PA.  With fragment prefetch a
+    // tile is requested at the end of an iteration, PA tiles ahead, into the buffer whose tile went
+    // to registers an iteration ago; without, at the start of an iteration, PA - 1 tiles ahead, into
+    // the buffer every wave finished reading before the barrier that has just been passed.
+    static constexpr int NBUF = PA;
     static constexpr int ROWB = BK * 2;                        // bytes of one activation tile row in LDS
     static constexpr size_t LDS_A = (size_t)WK * NBUF * BM * ROWB;
     // vector-memory loads of one super per wave (packed words, 1-bit plane, scales, zero-points)
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 
     // ---- one super of this wave's TN weight rows: packed fields, scales, zero-points ----
     struct Quant { uint32_t s[NT32][SREGS]; uint32_t z[NT32]; };
-    struct WStage { u32x4 w[UPS]; u32x4 h[C::HI ? C::UPH : 1]; Quant q; };
+    struct WStage { u32x4 w[UPS]; u32x4 h[C::HI ? C::UPH : 1]; };
     uint32_t w_off[UPS], h_off[C::HI ? C::UPH : 1], s_off[NT32], z_off[NT32];   // per-lane byte offsets from the wave's first row
     const int n_base = min(n_wave, C::N - 1);                  // a wave wholly past the last row re-reads it
 #pragma unroll
@@ -262,6 +264,10 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 st.h[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
             }
         }
+    };
+    auto load_quant = [&](Quant& qu, int sup_local) {
+        if (QF_GEMM_EXPERIMENT & 32) return;
+        const int sup = min(sup_local * WK + grp, C::NSUP - 1);
         const int g0 = sup * C::SUPK / C::GS;                  // first group of the super
         const uint8_t* sb = s_rows + (size_t)g0 * 2;
         const uint8_t* zb = z_rows + (g0 * C::ZFB) / 8;
@@ -269,23 +275,23 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         for (int j = 0; j < NT32; j++) {
             const uint8_t* sp = sb + s_off[j];
             if constexpr (NGS == 1) {
-                st.q.s[j][0] = *reinterpret_cast<const uint16_t*>(sp);
+                qu.s[j][0] = *reinterpret_cast<const uint16_t*>(sp);
             } else if constexpr (NGS == 2) {
-                st.q.s[j][0] = *reinterpret_cast<const uint32_t*>(sp);
+                qu.s[j][0] = *reinterpret_cast<const uint32_t*>(sp);
             } else if constexpr (NGS == 4) {
                 const u32x2 v = *reinterpret_cast<const u32x2*>(sp);
-                st.q.s[j][0] = v.x; st.q.s[j][1] = v.y;
+                qu.s[j][0] = v.x; qu.s[j][1] = v.y;
             } else {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(sp);
-                st.q.s[j][0] = v.x; st.q.s[j][1] = v.y; st.q.s[j][2] = v.z; st.q.s[j][3] = v.w;
+                qu.s[j][0] = v.x; qu.s[j][1] = v.y; qu.s[j][2] = v.z; qu.s[j][3] = v.w;
             }
-            st.q.z[j] = 0;
+            qu.z[j] = 0;
             if constexpr (!C::SYM) {
                 const uint8_t* zp = zb + z_off[j];
-                if constexpr (C::ZBITS >= 32) st.q.z[j] = *reinterpret_cast<const uint32_t*>(zp);
-                else if constexpr (C::ZBITS == 16) st.q.z[j] = *reinterpret_cast<const uint16_t*>(zp);
-                else if constexpr (C::ZBITS == 8) st.q.z[j] = *zp;
-                else st.q.z[j] = (uint32_t)*zp >> ((g0 * C::ZFB) % 8);         // fewer than 8 bits: inside one byte
+                if constexpr (C::ZBITS >= 32) qu.z[j] = *reinterpret_cast<const uint32_t*>(zp);
+                else if constexpr (C::ZBITS == 16) qu.z[j] = *reinterpret_cast<const uint16_t*>(zp);
+                else if constexpr (C::ZBITS == 8) qu.z[j] = *zp;
+                else qu.z[j] = (uint32_t)*zp >> ((g0 * C::ZFB) % 8);         // fewer than 8 bits: inside one byte
             }
         }
     };
@@ -367,13 +373,14 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             }
     };
 
-    WStage ringW[2];
+    WStage ringW[2];            // packed words of the two supers after the one in LDS
+    Quant ringQ[2];             // scales and zero-points: slot P % 2 serves super P for its whole duration
     Packed cur, nxt;
-    Quant qcur;
     AFrags fcur, fnxt;
 
     // One K-iteration; s = it % (2*SUP) is a compile-time constant at every call site; b0, b1 and
-    // b2 are the LDS buffers of tiles it, it+1 and it+PA (tile t lives in buffer t % NBUF).
+    // b2 are the LDS buffers of tiles it, it+1 and it+PA-1 (tile t lives in buffer t % PA; tile
+    // it+PA shares b0).
     //   * the fragments of tile it+1 (complete in LDS since the last barrier) are fetched now and
     //     used in the next iteration: no wave waits on LDS right after a barrier;
     //   * the MFMAs of tile it run on registers filled one iteration ago, interleaved with the
@@ -386,6 +393,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         const int q = s % SUP, pslot = (s / SUP) & 1;
         const int P = it / SUP;                                 // super index inside the group
         if constexpr (C::PREFETCH_A) read_frags(fnxt, b1);
+        else load_a(b2, min(it + C::PA - 1, C::ITERS - 1));
         // every read of the current super has been issued one iteration ago: the next super
         // (loaded two supers back) takes its place in LDS
         if (q == SUP - 1) store_super(ringW[pslot ^ 1]);
@@ -403,7 +411,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 }
 #pragma unroll
                 for (int j = 0; j < NT32; j++) {
-                    const QConst qc = qconst_of(qcur, j, q);
+                    const QConst qc = qconst_of(ringQ[pslot], j, q);
                     if constexpr ((QF_GEMM_EXPERIMENT & 1) != 0) {
                         wf[j] = __builtin_bit_cast(f16x8, u32x4{cur.w[j][0], cur.w[j][1], cur.w[j][2], cur.w[j][3] + (uint32_t)ks});
                     } else if constexpr (C::NBITS == 3) {
@@ -427,36 +435,38 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                         else acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], af[i], acc[j][i], 0, 0, 0);
             }
         }
-        load_a(b2, min(it + C::PA, C::ITERS - 1));
+        if constexpr (C::PREFETCH_A) load_a(b0, min(it + C::PA, C::ITERS - 1));
         cur = nxt;
         if constexpr (C::PREFETCH_A) fcur = fnxt;
         if (q == SUP - 1) {
-            // its register slot goes to the super two after it
-            qcur = ringW[pslot ^ 1].q;
+            // its register slot goes to the super two after it; the quantisation slot of the super
+            // that ends here goes to the one after next (no register is copied: a copy of a loaded
+            // value at the loop's back-edge would wait for every load in flight)
             load_super(ringW[pslot ^ 1], P + 3);
+            load_quant(ringQ[pslot], P + 2);
         }
-        // Publish the tile the next iteration reads (tile it+2 with fragment prefetch, else it+1):
-        // it was requested PA - W iterations ago, and every vector-memory load the wave has issued
-        // in the iterations since (activation tiles and whole supers) may stay in flight.  Loads
-        // return in order; the supers of the requesting iteration itself are not counted, wherever
-        // the compiler places them relative to the request.
-        constexpr int W = C::PREFETCH_A ? 2 : 1;
-        wait_loads_and_barrier<loads_since<C>(s, C::PA - W)>();
+        // Publish the tile the next iteration reads (tile it+2 with fragment prefetch, else it+1).
+        // Either way its request is PA - 2 whole iterations old, and every vector-memory load the
+        // wave has issued in those iterations (activation tiles and whole supers) may stay in
+        // flight.  Loads return in order; what the requesting iteration itself issued next to the
+        // request is not counted, wherever the compiler placed it.
+        wait_loads_and_barrier<loads_since<C>(s, C::PA - 2)>();
     };
 
     // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----
     load_super(ringW[0], 0);
+    load_quant(ringQ[0], 0);
     load_super(ringW[1], 1);
+    load_quant(ringQ[1], 1);
 #pragma unroll
-    for (int p = 0; p < C::PA; p++) load_a(p, min(p, C::ITERS - 1));
+    for (int p = 0; p < (C::PREFETCH_A ? C::PA : C::PA - 1); p++) load_a(p, min(p, C::ITERS - 1));
     store_super(ringW[0]);
-    qcur = ringW[0].q;
     load_super(ringW[0], 2);
     read_packed(cur, 0);
     wait_loads_and_barrier<0>();
     if constexpr (C::PREFETCH_A) read_frags(fcur, 0);
 
-    int b0 = 0, b1 = 1, b2 = C::PA % C::NBUF;
+    int b0 = 0, b1 = 1, b2 = C::PA - 1;
 #pragma unroll 1
     for (int it0 = 0; it0 < C::ITERS; it0 += 2 * SUP) {
         static_for<0, 2 * SUP>([&](auto s_tag) {
@@ -541,7 +551,7 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::NGS > 8 || C::ZBITS > 32) why = "too many groups per 128 packed bytes";
     else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if ((C::BM * (C::BK / 8)) % C::TG != 0) why = "the activation tile must split evenly over a group's threads";
-    else if (C::PA < (C::PREFETCH_A ? 3 : 2) || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12 (2 .. 12 for tiles taller than 128 rows)";
+    else if (C::PA < 3 || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12";
     else if (C::LDS_BYTES > 160 * 1024) why = "tiles exceed the 160 KB of LDS";
     else if (C::ACC_PER_THREAD > 256) why = "accumulator tile exceeds the register file";
     if (why) {
