@@ -141,3 +141,26 @@ def test_reference_launch_symbol_through_plain_ctypes(qf, oracle, M):
     assert rc.value == 0
     ref = reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS)
     assert_close(oracle, out.cpu().numpy(), ref, f"launch M={M}")
+
+
+@pytest.mark.parametrize("M,N,K,nbits", [(256, 8192, 8192, 4), (256, 57344, 8192, 4), (128, 10240, 8192, 4),
+                                         (16, 4096, 11008, 4), (16, 8192, 8192, 8)])
+def test_repeated_launches_give_identical_bits(qf, M, N, K, nbits):
+    """The GEMM kernel publishes activation tiles with explicit load-count waits and bare barriers, the
+    skinny kernel reduces through alternating LDS slots behind a bare barrier: a missed wait would show
+    as a launch-to-launch difference.  Every reduction order is fixed, so 30 launches over cold and warm
+    caches must agree bit for bit."""
+    print(f"[case] repeat M{M}-N{N}-K{K}-b{nbits}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(7 + N + K + M)
+    layer = qf.empty(M, K, N, nbits, 128, sym=False, compile_flags=NO_SEARCH)
+    layer.w.copy_(torch.randint(-128, 128, layer.w.shape, dtype=torch.int8, device="cuda", generator=g))
+    layer.s.copy_((torch.rand(layer.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
+    layer.z.copy_(torch.randint(-128, 128, layer.z.shape, dtype=torch.int8, device="cuda", generator=g))
+    A = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
+    first = layer(A).clone()
+    scrub = torch.empty(64 << 20, dtype=torch.int8, device="cuda")
+    for i in range(30):
+        if i % 3 == 0:
+            scrub.fill_(i)                        # push the operands out of L2 now and then
+        out = layer(A)
+        assert torch.equal(out, first), f"launch {i} differs"
