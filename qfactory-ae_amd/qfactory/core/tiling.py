@@ -532,6 +532,12 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     wk = max(1, 8 // wn) if blocks <= NUM_CUS else 1
     if bm == 256:
         wk = 1
+    if M >= 256 and (bm, wn, nt32) == (64, 4, 1) and wk == 2:
+        # one round of 64 x 128 tiles with two groups: a 64 x 64 wave tile (two 32-row weight tiles
+        # per wave) reuses every activation fragment twice; measured 59.7 against 62.6 us on
+        # 8192 x 8192 and 172 against 183 us on 8192 x 28672 at M = 256 (slower than four 64 x 32
+        # waves when blocks come in several rounds and there is only one group)
+        wn, nt32 = 2, 2
     nsup = K // (1024 // plane_bits(nbits))
     wk = max(1, min(wk, nsup))
     pa = 4
