@@ -66,7 +66,8 @@ def large_parity_cases():
     """W4A16 g128 GEMM at M in {32..256} on Llama-3-70B-style shapes.  The weights are too large to
     build from int32 tensors in a test; the tests fill packed tensors directly (every byte pattern
     is a valid packed weight) and check a seeded subset of output columns."""
-    return [_case(M, N, K) for N, K in LLAMA3_70B for M in (32, 64, 128, 256)]
+    return ([_case(M, N, K) for N, K in LLAMA3_70B for M in (32, 64, 128, 256)]
+            + [_case(512, 10240, 8192), _case(1024, 12288, 4096), _case(700, 22016, 4096)])
 
 
 def bench_cases():
@@ -91,7 +92,7 @@ TINY_LLAMA = [(768, 256), (256, 256), (1024, 256), (256, 512)]      # the decode
 def decode_cases():
     """decode_llama.py: Llama-2-7B shapes at batch 1 / 16 / 64 (decode) and at prefill row counts,
     plus the tiny model tests/test_decode_gpu.py runs."""
-    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256)]
+    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 1024)]
     cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
     return cases
 

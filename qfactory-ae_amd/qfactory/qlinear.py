@@ -25,7 +25,7 @@ def _m_bucket(m):
     if m <= 16:
         return 16
     bucket = 32
-    while bucket < m and bucket < 256:
+    while bucket < m and bucket < 1024:        # 512 and 1024: prefill-sized tiles (256 x 256 blocks on wide layers)
         bucket *= 2
     return bucket
 
