@@ -95,3 +95,16 @@ def test_emit_names_the_kernel_of_the_regime(regime, M, N, K, nbits):
     header = {"gemv": "qf_gemv.hip.h", "mgemv": "qf_mgemv.hip.h", "skinny": "qf_skinny.hip.h", "gemm": "qf_gemm.hip.h"}[regime]
     assert f'#include "{header}"' in code and f"regime={regime}" in code
     assert 'extern "C"' in code and "launch_m" in code
+
+
+def test_row_count_buckets():
+    from qfactory.qlinear import _m_bucket
+    assert [_m_bucket(m) for m in (1, 2, 3, 16, 17, 32, 33, 100, 256, 257, 512, 700, 1024, 5000)] == \
+        [1, 2, 16, 16, 32, 32, 64, 128, 256, 512, 512, 1024, 1024, 1024]
+
+
+def test_prefill_sizes_use_the_many_rows_model_only_for_several_rounds():
+    assert tiling.gemm_tiling(1024, 57344, 8192, 4, 128)["BM"] == 256
+    assert tiling.gemm_tiling(512, 10240, 8192, 4, 128) == {"BM": 128, "NT32": 2, "WN": 4, "WK": 1, "PA": 4}
+    # one round of 64 x 128 tiles: the K axis is still split over wave groups
+    assert tiling.gemm_tiling(512, 4096, 4096, 4, 128)["WK"] == 2
