@@ -1,4 +1,6 @@
-// Dequant-fused low-bit "skinny GEMM" on the gfx950 matrix cores for 3 <= M <= 32, HBM-bound.
+// Dequant-fused low-bit "skinny GEMM" on the gfx950 matrix cores for 3 <= M <= 16, HBM-bound
+// (two 16-row tiles per block, M <= 32, are accepted but need more registers than two waves per
+// SIMD have: measured 2 - 4 times slower than the GEMM kernel, which serves those row counts).
 //
 //   C[m][n] = fp16( sum_g s[n][g] * sum_{k in g} A[m][k] * (q[n][k] - Z[n][g]) )
 //
