@@ -436,12 +436,11 @@ def skinny_candidates(M, N, K, nbits, group_size):
             out.append(cfg)
 
     add(base)
-    for wk in (16, 14, 12, 11, 8, 7, 6, 4):
-        for sb in (1, 2, 4):
+    for wk in (base["WK"], 8, 7, 6, 4):
+        for sb in (1, 2):
             for d in (1, 2, 3):
                 for ast in (0, 1):
-                    for pb in (NUM_CUS, 2 * NUM_CUS):
-                        add({"MT16": base["MT16"], "WK": wk, "SB": sb, "D": d, "AST": ast, "PB": pb})
+                    add({"MT16": base["MT16"], "WK": wk, "SB": sb, "D": d, "AST": ast, "PB": NUM_CUS})
     return out
 
 
