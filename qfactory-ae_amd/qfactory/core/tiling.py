@@ -274,13 +274,15 @@ def mgemv_tiling(M, N, K, nbits, group_size, max_waves=16, **pins):
         wk = -(-nchunk // ch)
         if wk > max_waves or (wk - 1) * ch >= nchunk:
             continue
-        for pf in (2, 4, 1):
+        for pf in (1, 2, 4):
             if mgemv_regs(mt16, ch, pf, nbits) > mgemv_reg_limit(wk):
                 continue
             if mgemv_lds_bytes(mt16, wk, ch, nbits) > 160 * 1024:
                 continue
             waste = wk * ch - nchunk
-            key = (waste > ch // 2, -wk, pf != 2, waste)      # more, thinner waves measured best on MI355X
+            # more, thinner waves measured best on MI355X; with 8 - 16 waves per CU one tile ahead per
+            # wave is enough (two ahead measured 3 - 8 % slower, four 5 - 150 % slower)
+            key = (waste > ch // 2, -wk, pf != 1, waste)
             if best is None or key < best[0]:
                 best = (key, wk, ch, pf)
     if best is None:

@@ -37,6 +37,17 @@
 
 namespace qf {
 
+template <int V> struct MgTag { static constexpr int value = V; };
+template <class T> struct mg_is_tag { static constexpr bool value = false; };
+template <int V> struct mg_is_tag<MgTag<V>> { static constexpr bool value = true; };
+template <int I, int N, class F>
+__device__ __forceinline__ void mg_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(MgTag<I>{});
+        mg_static_for<I + 1, N>(f);
+    }
+}
+
 template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_>
 struct MGemvCfg {
     static constexpr int NBITS = NBITS_, GS = GS_, N = N_, K = K_;
@@ -193,24 +204,39 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     const float* redf = reinterpret_cast<const float*>(smem);
     static_assert(SB % PF == 0, "ring index must be static inside a batch");
     constexpr int PITCH_W = CH * 64 + 16;
-#pragma unroll 1
-    for (int batch = 0; batch < C::NBATCH; batch++) {
-#pragma unroll
-        for (int sb = 0; sb < SB; sb++) {
+    // One batch of SB tiles.  With few batches (the usual case) the batch index is a compile-time
+    // constant, so "is there a tile PF ahead to load" is decided at compile time: a load inside a
+    // run-time branch reaches its users through a copy at the join, and that copy waits for every
+    // load in flight -- measured as a full drain (vmcnt(0)) at the end of every tile, i.e. weight
+    // loads and compute did not overlap at all.
+    auto do_batch = [&](auto batch_v) {
+        using BT = decltype(batch_v);
+        constexpr bool STATIC_BATCH = mg_is_tag<BT>::value;
+        int batch;
+        if constexpr (STATIC_BATCH) batch = BT::value; else batch = batch_v;
+        mg_static_for<0, SB>([&](auto sb_tag) {
+            constexpr int sb = decltype(sb_tag)::value;
             const int slot = batch * SB + sb;
             const int tile = team_id + slot * TEAM_STRIDE;
             WStage& cur = ring[sb % PF];
             f32x4 acc[MT16];
 #pragma unroll
             for (int mt = 0; mt < MT16; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (slot < SLOTS && tile < C::NT && !(QF_MGEMV_EXPERIMENT & 2)) {               // wave-uniform
+            // Hand-off and refill of a slot the block really has run outside the run-time test for a
+            // ragged last tile (its stage holds the clamped last tile: valid memory, results unused),
+            // so that with a static batch index no load sits inside a run-time branch.
+            bool have_slot = true;
+            if constexpr (STATIC_BATCH) { if constexpr (BT::value * SB + sb >= SLOTS) have_slot = false; }
+            else have_slot = slot < SLOTS;
+            u32x4 wfrag[CH];
+            uint32_t qs[NSI], qz[NZI];
+            if (have_slot && !(QF_MGEMV_EXPERIMENT & 2)) {
                 // coalesced registers -> LDS -> fragment registers: lane (r, kb) takes the 16 bytes
                 // of row r at chunk c, k-block kb
 #pragma unroll
                 for (int i = 0; i < CH; i++)
                     *reinterpret_cast<u32x4*>(wbuf + (i * RPI + lane / LPR) * PITCH_W + (lane % LPR) * 16) = cur.w[i];
                 __builtin_amdgcn_wave_barrier();
-                u32x4 wfrag[CH];
 #pragma unroll
                 for (int c = 0; c < CH; c++)
                     wfrag[c] = *reinterpret_cast<const u32x4*>(wbuf + r * PITCH_W + c * 64 + kb * 16);
@@ -218,12 +244,17 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                 // the stage's packed words are in LDS and its scales / zero-points in `qs` / `qz`:
                 // it takes the loads of the tile PF ahead right away, one whole tile of
                 // dequantisation and MFMAs before they are needed
-                uint32_t qs[NSI], qz[NZI];
 #pragma unroll
                 for (int j = 0; j < NSI; j++) qs[j] = cur.s[j];
 #pragma unroll
                 for (int j = 0; j < NZI; j++) qz[j] = C::SYM ? 0u : cur.z[j];
-                if (slot + PF < SLOTS) load_tile(cur, min(tile + PF * TEAM_STRIDE, C::NT - 1));
+                if constexpr (STATIC_BATCH) {
+                    if constexpr (BT::value * SB + sb + PF < SLOTS) load_tile(cur, min(tile + PF * TEAM_STRIDE, C::NT - 1));
+                } else {
+                    if (slot + PF < SLOTS) load_tile(cur, min(tile + PF * TEAM_STRIDE, C::NT - 1));
+                }
+            }
+            if (have_slot && tile < C::NT && !(QF_MGEMV_EXPERIMENT & 2)) {               // wave-uniform
 #pragma unroll
                 for (int c = 0; c < CH; c++) {
                     const int g = ((lo + c) * CHUNK + kb * EPL) / C::GS;     // group of this lane's fields
@@ -283,7 +314,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT16; mt++)
                 red[(((size_t)wk * SB + sb) * MT16 + mt) * 64 + lane] = acc[mt];
-        }
+        });
 
         __syncthreads();
 
@@ -320,6 +351,12 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             }
         }
         if (batch + 1 < C::NBATCH) __syncthreads();           // LDS slots are reused by the next batch
+    };
+    if constexpr (C::NBATCH <= 8) {
+        mg_static_for<0, C::NBATCH>(do_batch);
+    } else {
+#pragma unroll 1
+        for (int batch = 0; batch < C::NBATCH; batch++) do_batch(batch);
     }
 }
 
