@@ -322,8 +322,9 @@ __global__ __launch_bounds__(C::THREADS) void skinny_kernel(
     };
 
     // ---- end of a batch: the WK partial tiles meet in LDS and every output is stored once.  A
-    //      partial tile sits in LDS as [lane = n + 16*(m/4)][e = m%4]; the storing lane takes
-    //      (m = lane/4, n = 4*(lane%4) .. +3): one 8-byte store per lane.  The two sets of slots
+    //      partial tile sits in LDS as [lane = n + 16*(m/4)][e = m%4]; every thread of the block takes
+    //      single outputs (m = o/16, n = o%16 inside a tile), so sixteen neighbouring lanes read sixteen
+    //      banks and store 32 contiguous bytes and the WK-deep sums are spread over all waves.  The two sets of slots
     //      alternate, so a fast wave parking batch b+1 never touches what a slow one still reads. ----
     auto finish_batch = [&](int batch) {
         f32x4* red = reinterpret_cast<f32x4*>(smem) + (size_t)(batch & 1) * (WK * SB * MT16 * 64);   // [WK][SB][MT16][64]
@@ -336,34 +337,20 @@ __global__ __launch_bounds__(C::THREADS) void skinny_kernel(
             }
         skinny_lds_barrier();
         const float* redf = reinterpret_cast<const float*>(red);
-        for (int p = wk; p < SB * MT16 && !(QF_SKINNY_EXPERIMENT & 4); p += WK) {
+        constexpr int OUTPUTS = SB * MT16 * 256;
+        for (int o = (int)threadIdx.x; o < OUTPUTS && !(QF_SKINNY_EXPERIMENT & 4); o += 64 * WK) {
+            const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
             const int sb = p / MT16, mt = p % MT16;
             const int slot = batch * SB + sb;
             const int tile = team + slot * C::GRID_X;
             if (slot >= C::SLOTS || tile >= C::NT) continue;
-            const int ml = lane >> 2, nq = (lane & 3) * 4;
-            float total[4] = {0.f, 0.f, 0.f, 0.f};
+            const float* base = redf + (((size_t)sb * MT16 + mt) * 64 + nl + 16 * (ml >> 2)) * 4 + (ml & 3);
+            float total = 0.f;
 #pragma unroll
-            for (int k2 = 0; k2 < WK; k2++) {
-                const float* base = redf + ((((size_t)k2 * SB + sb) * MT16 + mt) * 64) * 4;
-#pragma unroll
-                for (int j = 0; j < 4; j++) total[j] += base[((nq + j) + 16 * (ml >> 2)) * 4 + (ml & 3)];
-            }
+            for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
             const int m = m0 + 16 * mt + ml;
-            const int n = tile * 16 + nq;
-            if (m < m_total) {
-                uint16_t h[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) h[e] = f32_to_f16_bits(total[e]);
-                uint16_t* dst = Cout + (size_t)m * C::N + n;
-                if constexpr (C::N % 4 == 0) {
-                    if (n < C::N) *reinterpret_cast<u32x2*>(dst) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < C::N) dst[e] = h[e];
-                }
-            }
+            const int n = tile * 16 + nl;
+            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_f16_bits(total);
         }
     };
 
