@@ -59,6 +59,10 @@ def parity_cases():
     cases += [_case(2, 22016, 4096)]
     # 2-bit at K = 4096: the A-stationary kernel's 16-wave tiling does not fit LDS, 8 waves do
     cases += [_case(16, 100, 4096, 2, 128), _case(32, 48, 4096, 2, 64, True)]
+    # 3-bit (two planes per row) in the A-stationary kernel: ragged M and N, a last wave that owns fewer
+    # chunks, group per lane / per chunk / over two chunks
+    cases += [_case(3, 77, 4096, 3, 128), _case(12, 100, 2048, 3, 64), _case(16, 48, 8192, 3, 256, True),
+              _case(9, 100, 1024, 3, 512), _case(16, 272, 4864, 3, 128), _case(32, 40, 1024, 3, 128)]
     return cases
 
 

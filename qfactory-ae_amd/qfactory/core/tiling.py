@@ -35,7 +35,9 @@ def regime_for(M, K=None, nbits=None, group_size=None):
     if M < MGEMV_MIN_M or not MFMA_AVAILABLE:
         return "gemv"
     if K is not None and nbits == 3:
-        # 3-bit has two kernels: the dot2 GEMV (any M, tiled over grid.y) and the GEMM
+        # 3-bit has three kernels: the dot2 GEMV (any M, tiled over grid.y), the A-stationary kernel and the GEMM
+        if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
+            return "mgemv"
         return "gemm" if gemm_supported(K, nbits, group_size) else "gemv"
     if K is None or not mfma_supported(K, nbits, group_size):
         return "gemv"
@@ -238,17 +240,26 @@ def mfma_cfg_string(problem, t, decode_strategy, nt_b):
 # A-stationary MFMA regime (2 <= M <= 64)
 # --------------------------------------------------------------------------------------------
 
+def mgemv_supported(K, nbits, group_size):
+    """Whole chunks of 16 bytes of the main plane per lane, and a lane's fields inside one group."""
+    if nbits not in (2, 3, 4, 8) or not group_size or group_size <= 0:
+        return False
+    epl = 128 // plane_bits(nbits)
+    return K % (4 * epl) == 0 and group_size % epl == 0
+
+
 def mgemv_regs(mt16, ch, pf, nbits):
     """Rough VGPR need of qf::mgemv_kernel: resident activations, the ring of weight stages and
-    the fragment copy of the tile being consumed."""
-    ksteps = (128 // nbits) // 8
-    return mt16 * ch * ksteps * 4 + pf * (ch * 4 + 4) + ch * 4 + 48
+    the fragment copy of the tile being consumed (3-bit: plus the 1-bit plane of both)."""
+    ksteps = (128 // plane_bits(nbits)) // 8
+    hi = (pf * 4 * -(-ch // 2) + 2 * ch) if nbits == 3 else 0
+    return mt16 * ch * ksteps * 4 + pf * (ch * 4 + 4) + ch * 4 + 48 + hi
 
 
 def mgemv_lds_bytes(mt16, wk, ch, nbits, sb=4):
     """LDS of qf::mgemv_kernel: SB partial tiles per wave plus the wave's transposition buffer."""
-    chunk = 4 * (128 // nbits)
-    wbuf = max(16 * (ch * 64 + 16), 16 * (chunk * 2 + 16))
+    chunk = 4 * (128 // plane_bits(nbits))
+    wbuf = max(16 * (ch * 64 + 16) + (16 * (ch * 32 + 16) if nbits == 3 else 0), 16 * (chunk * 2 + 16))
     return wk * sb * mt16 * 1024 + wk * wbuf
 
 
@@ -260,9 +271,9 @@ def mgemv_reg_limit(wk):
 def mgemv_tiling(M, N, K, nbits, group_size, max_waves=16, **pins):
     """MT16 activation tiles resident per wave, WK waves x CH chunks covering K, PF weight tiles in
     flight; None if the activations do not fit the register file of one block."""
-    if not mfma_supported(K, nbits, group_size):
+    if not mgemv_supported(K, nbits, group_size):
         return None
-    chunk = 4 * (128 // nbits)
+    chunk = 4 * (128 // plane_bits(nbits))
     if group_size % chunk and chunk % group_size:
         return None
     mt16 = -(-M // 16)
@@ -298,7 +309,7 @@ def mgemv_candidates(M, N, K, nbits, group_size):
     if base is None:
         return []
     seen, out = set(), []
-    nchunk = K // (4 * (128 // nbits))
+    nchunk = K // (4 * (128 // plane_bits(nbits)))
 
     def add(cfg):
         key = tuple(sorted(cfg.items()))

@@ -56,7 +56,10 @@ struct MGemvCfg {
     static constexpr int WK = WK_;                 // waves along K per team
     static constexpr int CH = CH_;                 // chunks per wave
     static constexpr int PB = PB_;                 // upper bound on blocks along N
-    static constexpr int EPL = 128 / NBITS;        // fields per lane and 16-byte load
+    static constexpr int PBITS = plane_bits(NBITS);   // 3-bit rows: a 2-bit main plane followed by a 1-bit plane
+    static constexpr int ZFB = zero_field_bits(NBITS); // stored width of one zero-point
+    static constexpr bool HI = NBITS == 3;
+    static constexpr int EPL = 128 / PBITS;        // fields per lane and 16-byte load of the main plane
     static constexpr int KSTEPS = EPL / 8;         // MFMA k-steps per chunk
     static constexpr int CHUNK = 4 * EPL;          // elements of K per chunk
     static constexpr int NCHUNK = K / CHUNK;
@@ -70,15 +73,22 @@ struct MGemvCfg {
     static constexpr int NBATCH = (SLOTS + SB - 1) / SB;
     static constexpr int RB = K * NBITS / 8;
     static constexpr int G = K / GS;
-    static constexpr int ZRB = G * NBITS / 8;
+    static constexpr int ZRB = G * ZFB / 8;
+    static constexpr int HI_OFF = K / 4;           // byte offset of the 1-bit plane in a 3-bit row
     static constexpr bool DEFERRED = (GS % CHUNK == 0);      // a chunk lies inside one group
     static constexpr int LPR = CH * 4;             // lanes covering one row's K-slice (CH*64 bytes)
     static constexpr int RPI = 64 / LPR;           // rows per coalesced weight load
     // groups and zero-point bytes of one row inside a wave's K-slice
     // (upper bounds when a slice may start inside a group / inside a byte; indices are clamped to the row)
     static constexpr int GWN = (GS <= CHUNK) ? CH * CHUNK / GS : (CH * CHUNK) / GS + 2;
-    static constexpr int ZB = (GWN * NBITS + 7) / 8 + 1;
-    static constexpr int WBUF_W = 16 * (CH * 64 + 16);
+    static constexpr int ZB = (GWN * ZFB + 7) / 8 + 1;
+    // 1-bit plane of a tile: CH*32 bytes per row, loaded 16 bytes per lane
+    static constexpr int LPRH = CH * 2;            // lanes per row
+    static constexpr int RPIH = 64 / LPRH;         // rows per load (may exceed 16: the extra lanes idle)
+    static constexpr int NHI = HI ? (16 + RPIH - 1) / RPIH : 0;
+    static constexpr int PITCH_W = CH * 64 + 16;
+    static constexpr int PITCH_H = CH * 32 + 16;
+    static constexpr int WBUF_W = 16 * PITCH_W + (HI ? 16 * PITCH_H : 0);
     static constexpr int WBUF_A = 16 * (CHUNK * 2 + 16);
     static constexpr int WBUF = WBUF_W > WBUF_A ? WBUF_W : WBUF_A;    // per-wave transposition buffer
     static constexpr size_t LDS_BYTES = (size_t)WK * SB * MT16 * 1024 + (size_t)WK * WBUF;
@@ -90,8 +100,9 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
     constexpr int MT16 = C::MT16, WK = C::WK, CH = C::CH, SLOTS = C::SLOTS, PF = C::PF, SB = C::SB;
     constexpr int EPL = C::EPL, KSTEPS = C::KSTEPS, CHUNK = C::CHUNK;
-    constexpr int P8 = 8 / C::NBITS;
-    constexpr uint32_t ZMASK = (1u << C::NBITS) - 1u;
+    constexpr int P8 = 8 / C::ZFB;                      // zero-point fields per byte
+    constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
+    constexpr int NHI = C::NHI;
     constexpr bool DEFERRED = C::DEFERRED;
     constexpr int LPR = C::LPR, RPI = C::RPI;            // lanes per row and rows per coalesced weight load
     constexpr int GWN = C::GWN, ZB = C::ZB;              // scales / zero bytes per row in a wave's K-slice
@@ -119,6 +130,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     // ---- coalesced loads: LPR consecutive lanes cover one row's K-slice (CH*64 bytes) ----
     struct WStage {
         u32x4 w[CH];                 // load i: row i*RPI + lane/LPR, bytes (lane%LPR)*16 of the slice
+        u32x4 h[NHI ? NHI : 1];      // 1-bit plane, load i: row i*RPIH + lane/LPRH, bytes (lane%LPRH)*16
         uint32_t s[NSI];             // lane -> (row, group) = (idx / GWN, idx % GWN), idx = lane + 64*j
         uint32_t z[NZI];             // lane -> (row, byte)  = (idx / ZB,  idx % ZB)
     };
@@ -132,6 +144,12 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             st.w[i] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)wp) : *(const u32x4*)wp;
         }
 #pragma unroll
+        for (int i = 0; i < NHI; i++) {
+            const int n = min(n_base + min(i * C::RPIH + lane / C::LPRH, 15), C::N - 1);
+            const uint8_t* hp = W + (size_t)n * C::RB + C::HI_OFF + (size_t)lo * 32 + (lane % C::LPRH) * 16;
+            st.h[i] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)hp) : *(const u32x4*)hp;
+        }
+#pragma unroll
         for (int j = 0; j < NSI; j++) {
             const int idx = lane + 64 * j;
             const int n = min(n_base + min(idx / GWN, 15), C::N - 1);
@@ -142,7 +160,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             for (int j = 0; j < NZI; j++) {
                 const int idx = lane + 64 * j;
                 const int n = min(n_base + min(idx / ZB, 15), C::N - 1);
-                st.z[j] = Zp[(size_t)n * C::ZRB + min((gw_lo * C::NBITS) / 8 + idx % ZB, C::ZRB - 1)];
+                st.z[j] = Zp[(size_t)n * C::ZRB + min((gw_lo * C::ZFB) / 8 + idx % ZB, C::ZRB - 1)];
             }
         }
     };
@@ -203,7 +221,8 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 
     const float* redf = reinterpret_cast<const float*>(smem);
     static_assert(SB % PF == 0, "ring index must be static inside a batch");
-    constexpr int PITCH_W = CH * 64 + 16;
+    constexpr int PITCH_W = C::PITCH_W, PITCH_H = C::PITCH_H;
+    uint8_t* hbuf = wbuf + 16 * PITCH_W;                 // 1-bit plane of the tile being handed over
     // One batch of SB tiles.  With few batches (the usual case) the batch index is a compile-time
     // constant, so "is there a tile PF ahead to load" is decided at compile time: a load inside a
     // run-time branch reaches its users through a copy at the join, and that copy waits for every
@@ -229,6 +248,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             if constexpr (STATIC_BATCH) { if constexpr (BT::value * SB + sb >= SLOTS) have_slot = false; }
             else have_slot = slot < SLOTS;
             u32x4 wfrag[CH];
+            u32x2 hfrag[C::HI ? CH : 1];
             uint32_t qs[NSI], qz[NZI];
             if (have_slot && !(QF_MGEMV_EXPERIMENT & 2)) {
                 // coalesced registers -> LDS -> fragment registers: lane (r, kb) takes the 16 bytes
@@ -236,10 +256,17 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 #pragma unroll
                 for (int i = 0; i < CH; i++)
                     *reinterpret_cast<u32x4*>(wbuf + (i * RPI + lane / LPR) * PITCH_W + (lane % LPR) * 16) = cur.w[i];
+#pragma unroll
+                for (int i = 0; i < NHI; i++) {
+                    const int row = i * C::RPIH + lane / C::LPRH;
+                    if (row < 16) *reinterpret_cast<u32x4*>(hbuf + row * PITCH_H + (lane % C::LPRH) * 16) = cur.h[i];
+                }
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int c = 0; c < CH; c++)
+                for (int c = 0; c < CH; c++) {
                     wfrag[c] = *reinterpret_cast<const u32x4*>(wbuf + r * PITCH_W + c * 64 + kb * 16);
+                    if constexpr (C::HI) hfrag[c] = *reinterpret_cast<const u32x2*>(hbuf + r * PITCH_H + c * 32 + kb * 8);
+                }
                 __builtin_amdgcn_wave_barrier();
                 // the stage's packed words are in LDS and its scales / zero-points in `qs` / `qz`:
                 // it takes the loads of the tile PF ahead right away, one whole tile of
@@ -268,7 +295,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     }
                     uint32_t zero = 1u << (C::NBITS - 1);
                     if constexpr (!C::SYM) {
-                        const int zbyte = (g * C::NBITS) / 8 - (gw_lo * C::NBITS) / 8;
+                        const int zbyte = (g * C::ZFB) / 8 - (gw_lo * C::ZFB) / 8;
                         const int zidx = r * ZB + zbyte;
                         uint32_t zraw = 0;
 #pragma unroll
@@ -276,21 +303,32 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                             const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((zidx & 63) << 2, (int)qz[j]);
                             zraw = (NZI == 1 || (zidx >> 6) == j) ? v : zraw;
                         }
-                        zero = (zraw >> ((g % P8) * C::NBITS)) & ZMASK;
+                        zero = (zraw >> ((g % P8) * C::ZFB)) & ZMASK;
                     }
                     const ZConst zc = make_zconst<C::NBITS>(zero);
                     const uint32_t w4[4] = {wfrag[c].x, wfrag[c].y, wfrag[c].z, wfrag[c].w};
+                    // fields 8t .. 8t+7 of the lane's EPL as exact integers q - Z (fp16)
+                    auto fields = [&](auto t_tag) {
+                        constexpr int t = decltype(t_tag)::value;
+                        if constexpr (C::HI) {
+                            // 32 fields = two words of the 2-bit plane + one word of the 1-bit plane
+                            const uint32_t w2[4] = {w4[2 * (t / 4)], w4[2 * (t / 4) + 1], 0u, 0u};
+                            return IntStep3::run<t % 4>(w2, t < 4 ? hfrag[c].x : hfrag[c].y, zc);
+                        } else {
+                            return IntStep<C::NBITS>::run(w4, t, zc);
+                        }
+                    };
                     if constexpr (DEFERRED) {
                         // the whole chunk lies in one group: integer sum on the matrix core, one fp32 scale
                         f32x4 gsum[MT16];
-#pragma unroll
-                        for (int t = 0; t < KSTEPS; t++) {
-                            const f16x8 wf = IntStep<C::NBITS>::run(w4, t, zc);
+                        mg_static_for<0, KSTEPS>([&](auto t_tag) {
+                            constexpr int t = decltype(t_tag)::value;
+                            const f16x8 wf = fields(t_tag);
 #pragma unroll
                             for (int mt = 0; mt < MT16; mt++)
                                 gsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                                     af[mt][c][t], wf, t == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : gsum[mt], 0, 0, 0);
-                        }
+                        });
                         const float sc = f16_bits_to_f32((uint16_t)sraw);
 #pragma unroll
                         for (int mt = 0; mt < MT16; mt++)
@@ -301,13 +339,13 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                         // ones): scale every element before the contraction
                         const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)sraw);
                         const f16x8 s8 = f16x8{sh, sh, sh, sh, sh, sh, sh, sh};
-#pragma unroll
-                        for (int t = 0; t < KSTEPS; t++) {
-                            const f16x8 wf = IntStep<C::NBITS>::run(w4, t, zc) * s8;
+                        mg_static_for<0, KSTEPS>([&](auto t_tag) {
+                            constexpr int t = decltype(t_tag)::value;
+                            const f16x8 wf = fields(t_tag) * s8;
 #pragma unroll
                             for (int mt = 0; mt < MT16; mt++)
                                 acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][c][t], wf, acc[mt], 0, 0, 0);
-                        }
+                        });
                     }
                 }
             }
@@ -351,11 +389,11 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 template <class C>
 int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m, hipStream_t stream) {
     const char* why = nullptr;
-    if (C::NBITS != 2 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 4 or 8 for this kernel";
-    else if (C::K % C::CHUNK != 0) why = "K must be a multiple of 4*128/NBITS";
+    if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8 for this kernel";
+    else if (C::K % C::CHUNK != 0) why = "K must be a multiple of 4*128 / (bits of the main plane)";
     else if (C::GS <= 0 || C::K % C::GS != 0) why = "GS must divide K";
     else if (C::GS % C::EPL != 0) why = "a lane's 16 bytes of fields must lie inside one group";
-    else if (!C::SYM && (C::G % (8 / C::NBITS)) != 0) why = "K/GS must fill whole zero-point bytes";
+    else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if (C::CH > C::NCHUNK) why = "more chunks per wave than the row has";
     else if (C::WK * C::CH < C::NCHUNK) why = "WK*CH must cover K";
     else if ((C::WK - 1) * C::CH >= C::NCHUNK) why = "a wave would own no chunk";

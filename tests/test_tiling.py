@@ -24,7 +24,8 @@ def _id(c):
     (16, 8192, 8, 128, "skinny"), (16, 11008, 8, 128, "skinny"),
     (17, 11008, 4, 128, "gemm"), (16, 28672, 4, 128, "gemm"), (32, 8192, 4, 128, "gemm"),
     (64, 4096, 4, 128, "gemm"), (256, 8192, 4, 128, "gemm"),
-    (1, 8192, 3, 128, "gemv"), (2, 8192, 3, 128, "gemv"), (16, 8192, 3, 128, "gemm"),
+    (1, 8192, 3, 128, "gemv"), (2, 8192, 3, 128, "gemv"), (16, 8192, 3, 128, "mgemv"), (32, 8192, 3, 128, "gemm"),
+    (16, 4096, 3, 128, "mgemv"), (16, 4096, 3, 32, "gemv"),
     (33, 2048, 3, 128, "gemm"),
 ])
 def test_regime_routing(M, K, nbits, gs, expected):
@@ -37,7 +38,7 @@ def test_default_tiling_respects_the_kernel_limits(case):
     regime = tiling.regime_for(M, K, nbits, gs)
     if regime == "mgemv":
         t = tiling.mgemv_tiling(M, N, K, nbits, gs)
-        chunk = 4 * (128 // nbits)
+        chunk = 4 * (128 // tiling.plane_bits(nbits))
         nchunk = K // chunk
         assert t["WK"] * t["CH"] >= nchunk and (t["WK"] - 1) * t["CH"] < nchunk and t["WK"] <= 16
         assert tiling.mgemv_lds_bytes(t["MT16"], t["WK"], t["CH"], nbits) <= 160 * 1024
