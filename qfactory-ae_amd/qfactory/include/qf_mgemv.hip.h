@@ -69,7 +69,8 @@ struct MGemvCfg {
     static constexpr int GRID_X = NT < PB ? NT : PB;
     static constexpr int SLOTS = (NT + GRID_X - 1) / GRID_X;               // tiles per block
     static constexpr int PF = PF_;                 // weight tiles in flight per wave (ring of stages): 2 or 4
-    static constexpr int SB = QF_MGEMV_SB;         // tiles per batch: partials are reduced and stored per batch
+    // tiles per batch (partials are reduced and stored per batch): no more than the block has
+    static constexpr int SB = SLOTS < QF_MGEMV_SB ? (SLOTS + PF - 1) / PF * PF : QF_MGEMV_SB;
     static constexpr int NBATCH = (SLOTS + SB - 1) / SB;
     static constexpr int RB = K * NBITS / 8;
     static constexpr int G = K / GS;
