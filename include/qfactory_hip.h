@@ -52,6 +52,34 @@ int qf_transpose_scale(const uint16_t* scale, uint16_t* out, int64_t G, int64_t 
 int qf_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
 int qf_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
 
+/*
+ * Steps of one decode token between the quantized linears of a Llama-style layer, one launch each.
+ * The reference has no kernels of its own for them: its end-to-end runs (reproduce/fig11/
+ * run_all_qfactory.sh:22-40, through third_party/vllm-qfactory.patch) leave them to vLLM's RMSNorm,
+ * rotary-embedding, paged-attention and SiluAndMul ops; the decode loop that stands in for those runs
+ * here (decode_llama.py) calls these instead of ~45 small framework kernels per layer.
+ * fp16 tensors are passed as uint16_t*; arithmetic inside is fp32.
+ *
+ * qf_add_rmsnorm: x (rows, hidden) += delta (same shape; NULL: no add), in place, fp16 addition;
+ *   out = fp16(fp16(x * rsqrt(mean(x^2) + eps)) * weight).  hidden a multiple of 8, at most 16384.
+ * qf_rope_kv_store: qkv (batch, 3, heads, head_dim) of the new position *pos (device int64):
+ *   q_out (batch, heads, head_dim) = rotate(q), k_cache[b][h][*pos] = rotate(k), v_cache[b][h][*pos] = v;
+ *   caches are (batch, heads, max_len, head_dim); rotation of pairs (2i, 2i+1) by the angles in row
+ *   *pos of cos_table / sin_table (max_len, head_dim/2) fp32.  Writes nothing if *pos is outside
+ *   [0, max_len).
+ * qf_decode_attention: out (batch, heads*head_dim) = softmax(q k^T / sqrt(head_dim)) v over cache
+ *   positions 0 .. *pos.  head_dim in {32, 64, 128, 256}.
+ * qf_silu_mul: out (rows, mlp) = fp16(silu(gate_up[:, :mlp])) * gate_up[:, mlp:]; mlp a multiple of 8.
+ */
+int qf_add_rmsnorm(uint16_t* x, const uint16_t* delta, const uint16_t* weight, uint16_t* out, int64_t rows,
+                   int64_t hidden, float eps, void* stream);
+int qf_rope_kv_store(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
+                     uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int64_t batch, int64_t heads,
+                     int64_t head_dim, int64_t max_len, void* stream);
+int qf_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int64_t* pos,
+                        uint16_t* out, int64_t batch, int64_t heads, int64_t head_dim, int64_t max_len, void* stream);
+int qf_silu_mul(const uint16_t* gate_up, uint16_t* out, int64_t rows, int64_t mlp, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,286 @@
+// libqfactory_hip.so, second translation unit: the steps of one decode token (one new position per
+// sequence) that sit between the quantized linears of a Llama-style layer -- residual add + RMSNorm,
+// rotary embedding + KV-cache append, attention of the new position over the cache, SiLU(gate) * up.
+// Each is one launch; entry points and contracts are declared in include/qfactory_hip.h.
+//
+// All four are HBM/latency-bound fp16 kernels with fp32 arithmetic inside: 16-byte accesses, one block
+// per row / per (sequence, head), reductions through wave shuffles and LDS.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <stdint.h>
+
+#include "qfactory_hip.h"
+
+namespace {
+
+typedef _Float16 f16;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+int fail(const char* fn, const char* why) {
+    fprintf(stderr, "%s: %s\n", fn, why);
+    return 1;
+}
+
+int launched(const char* fn) {
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        fprintf(stderr, "%s: launch failed: %s\n", fn, hipGetErrorString(err));
+        return 2;
+    }
+    return 0;
+}
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Sum (MAX = false) or maximum (MAX = true) over the block; `slots` holds kWaves floats and may be
+// reused right after the call returns.
+template <bool MAX>
+__device__ __forceinline__ float block_reduce(float v, float* slots) {
+    v = MAX ? wave_max(v) : wave_sum(v);
+    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = slots[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) r = MAX ? fmaxf(r, slots[w]) : r + slots[w];
+    __syncthreads();
+    return r;
+}
+
+// ---------------------------------------------------------------------------------------------
+// x += delta (optional);  out = fp16( fp16(x * rsqrt(mean(x^2) + eps)) * weight ).  One block per row;
+// a thread keeps its (at most kNormVec) 8-element vectors in registers between the two passes.
+// ---------------------------------------------------------------------------------------------
+constexpr int kNormVec = 8;
+
+__global__ __launch_bounds__(kThreads) void add_rmsnorm_kernel(f16* __restrict__ x, const f16* __restrict__ delta,
+                                                               const f16* __restrict__ weight, f16* __restrict__ out,
+                                                               int hidden, float eps) {
+    __shared__ float slots[kWaves];
+    const size_t row = (size_t)blockIdx.x * hidden;
+    f16x8 v[kNormVec];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNormVec; i++) {
+        const int c = (threadIdx.x + i * kThreads) * 8;
+        if (c < hidden) {
+            v[i] = *reinterpret_cast<const f16x8*>(x + row + c);
+            if (delta) {
+                v[i] = v[i] + *reinterpret_cast<const f16x8*>(delta + row + c);      // fp16 add, as the residual stream is fp16
+                *reinterpret_cast<f16x8*>(x + row + c) = v[i];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) ss += (float)v[i][e] * (float)v[i][e];
+        }
+    }
+    const float r = rsqrtf(block_reduce<false>(ss, slots) / (float)hidden + eps);
+#pragma unroll
+    for (int i = 0; i < kNormVec; i++) {
+        const int c = (threadIdx.x + i * kThreads) * 8;
+        if (c < hidden) {
+            const f16x8 w = *reinterpret_cast<const f16x8*>(weight + c);
+            f16x8 o;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = (f16)((float)v[i][e] * r) * w[e];
+            *reinterpret_cast<f16x8*>(out + row + c) = o;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rotary embedding of q and k of the new position (pairs (2i, 2i+1), angle table row pos) and append
+// of k, v to the cache.  qkv row b is [3][H][hd]; caches are (B, H, max_len, hd).  One thread per pair.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void rope_kv_store_kernel(const f16* __restrict__ qkv, const int64_t* __restrict__ pos_ptr,
+                                                                 const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                 f16* __restrict__ q_out, f16* __restrict__ k_cache,
+                                                                 f16* __restrict__ v_cache, int batch, int heads, int hd, int max_len) {
+    const int64_t pos = pos_ptr[0];
+    if (pos < 0 || pos >= max_len) return;                    // nothing is written for a position outside the cache
+    const int half = hd / 2;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= (int64_t)batch * heads * half) return;
+    const int i = (int)(idx % half);
+    const int h = (int)((idx / half) % heads);
+    const int b = (int)(idx / ((int64_t)half * heads));
+    const float c = cos_t[pos * half + i], s = sin_t[pos * half + i];
+    const f16* row = qkv + (size_t)b * 3 * heads * hd;
+    const size_t in_off = (size_t)h * hd + 2 * i;
+    const size_t cache_off = (((size_t)b * heads + h) * max_len + (size_t)pos) * hd + 2 * i;
+    const float q0 = (float)row[in_off], q1 = (float)row[in_off + 1];
+    const float k0 = (float)row[(size_t)heads * hd + in_off], k1 = (float)row[(size_t)heads * hd + in_off + 1];
+    f16* qo = q_out + ((size_t)b * heads + h) * hd + 2 * i;
+    qo[0] = (f16)(q0 * c - q1 * s);
+    qo[1] = (f16)(q0 * s + q1 * c);
+    k_cache[cache_off] = (f16)(k0 * c - k1 * s);
+    k_cache[cache_off + 1] = (f16)(k0 * s + k1 * c);
+    v_cache[cache_off] = row[(size_t)2 * heads * hd + in_off];
+    v_cache[cache_off + 1] = row[(size_t)2 * heads * hd + in_off + 1];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Attention of one query per (sequence, head) over cache positions 0 .. pos.  LPK = hd/8 lanes share
+// a key or value row (16 bytes each).  Scores -> LDS, block max and sum, then every group of LPK lanes
+// walks its share of the value rows and the groups' partial outputs meet in LDS.
+// ---------------------------------------------------------------------------------------------
+template <int LPK>
+__global__ __launch_bounds__(kThreads) void decode_attention_kernel(const f16* __restrict__ q, const f16* __restrict__ k_cache,
+                                                                    const f16* __restrict__ v_cache, const int64_t* __restrict__ pos_ptr,
+                                                                    f16* __restrict__ out, int heads, int max_len, float scale) {
+    constexpr int HD = LPK * 8;
+    constexpr int GROUPS = kThreads / LPK;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* sc = smem;                                          // [max_len]
+    float* part = smem + max_len;                              // [GROUPS][HD]
+    __shared__ float slots[kWaves];
+    const int h = blockIdx.x, b = blockIdx.y;
+    int64_t pos = pos_ptr[0];
+    if (pos < 0) return;
+    const int n = (int)(pos < max_len ? pos + 1 : max_len);    // keys 0 .. n-1
+    const int g = threadIdx.x / LPK, j = threadIdx.x % LPK;
+    const size_t head = ((size_t)b * heads + h);
+    const f16* kc = k_cache + head * max_len * HD;
+    const f16* vc = v_cache + head * max_len * HD;
+
+    const f16x8 qv = *reinterpret_cast<const f16x8*>(q + head * HD + j * 8);
+    float qf[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) qf[e] = (float)qv[e] * scale;
+
+    float local_max = -INFINITY;
+    for (int p0 = 0; p0 < n; p0 += GROUPS) {
+        const int p = p0 + g;
+        float d = 0.f;
+        if (p < n) {
+            const f16x8 kv = *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
+#pragma unroll
+            for (int e = 0; e < 8; e++) d += qf[e] * (float)kv[e];
+        }
+#pragma unroll
+        for (int o = LPK / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
+        if (p < n) {
+            if (j == 0) sc[p] = d;
+            local_max = fmaxf(local_max, d);
+        }
+    }
+    const float mx = block_reduce<true>(local_max, slots);     // also publishes sc[] to the block
+    float local_sum = 0.f;
+    for (int p = threadIdx.x; p < n; p += kThreads) {
+        const float e = __expf(sc[p] - mx);
+        sc[p] = e;
+        local_sum += e;
+    }
+    const float total = block_reduce<false>(local_sum, slots);
+
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int p = g; p < n; p += GROUPS) {
+        const float w = sc[p];
+        const f16x8 vv = *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += w * (float)vv[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[g * HD + j * 8 + e] = acc[e];
+    __syncthreads();
+    for (int d = threadIdx.x; d < HD; d += kThreads) {
+        float s = 0.f;
+        for (int gg = 0; gg < GROUPS; gg++) s += part[gg * HD + d];
+        out[head * HD + d] = (f16)(s / total);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[m][i] = fp16(silu(gate[m][i])) * up[m][i], gate = gate_up[:, :mlp], up = gate_up[:, mlp:].
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void silu_mul_kernel(const f16* __restrict__ gate_up, f16* __restrict__ out,
+                                                            int64_t rows, int mlp) {
+    const int per_row = mlp / 8;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= rows * per_row) return;
+    const int64_t m = idx / per_row;
+    const int c = (int)(idx % per_row) * 8;
+    const f16x8 gv = *reinterpret_cast<const f16x8*>(gate_up + m * 2 * mlp + c);
+    const f16x8 uv = *reinterpret_cast<const f16x8*>(gate_up + m * 2 * mlp + mlp + c);
+    f16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float x = (float)gv[e];
+        o[e] = (f16)(x / (1.f + expf(-x))) * uv[e];
+    }
+    *reinterpret_cast<f16x8*>(out + m * mlp + c) = o;
+}
+
+template <int LPK>
+int launch_attention(const f16* q, const f16* k, const f16* v, const int64_t* pos, f16* out, int batch, int heads,
+                     int max_len, hipStream_t stream) {
+    constexpr int HD = LPK * 8;
+    const size_t lds = ((size_t)max_len + (size_t)(kThreads / LPK) * HD) * sizeof(float);
+    if (lds > 64 * 1024) return fail("qf_decode_attention", "max_len too large for the score buffer in LDS");
+    hipLaunchKernelGGL(decode_attention_kernel<LPK>, dim3(heads, batch), dim3(kThreads), lds, stream, q, k, v, pos, out,
+                       heads, max_len, 1.0f / sqrtf((float)HD));
+    return launched("qf_decode_attention");
+}
+
+}  // namespace
+
+extern "C" int qf_add_rmsnorm(uint16_t* x, const uint16_t* delta, const uint16_t* weight, uint16_t* out, int64_t rows,
+                              int64_t hidden, float eps, void* stream) {
+    if (!x || !weight || !out) return fail("qf_add_rmsnorm", "null pointer");
+    if (rows <= 0 || hidden <= 0 || hidden % 8 != 0) return fail("qf_add_rmsnorm", "rows positive, hidden a positive multiple of 8");
+    if (hidden > kThreads * 8 * kNormVec) return fail("qf_add_rmsnorm", "hidden above 16384");
+    if (rows > 0x7fffffff) return fail("qf_add_rmsnorm", "too many rows");
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)rows), dim3(kThreads), 0, (hipStream_t)stream, (f16*)x, (const f16*)delta,
+                       (const f16*)weight, (f16*)out, (int)hidden, eps);
+    return launched("qf_add_rmsnorm");
+}
+
+extern "C" int qf_rope_kv_store(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
+                                uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int64_t batch, int64_t heads,
+                                int64_t head_dim, int64_t max_len, void* stream) {
+    if (!qkv || !pos || !cos_table || !sin_table || !q_out || !k_cache || !v_cache) return fail("qf_rope_kv_store", "null pointer");
+    if (batch <= 0 || heads <= 0 || head_dim <= 0 || head_dim % 2 != 0 || max_len <= 0)
+        return fail("qf_rope_kv_store", "batch, heads, max_len positive and head_dim even");
+    const int64_t pairs = batch * heads * (head_dim / 2);
+    if (pairs > (int64_t)0x7fffffff * kThreads || batch * heads * max_len * head_dim < 0) return fail("qf_rope_kv_store", "problem too large");
+    hipLaunchKernelGGL(rope_kv_store_kernel, dim3((unsigned)((pairs + kThreads - 1) / kThreads)), dim3(kThreads), 0, (hipStream_t)stream,
+                       (const f16*)qkv, pos, cos_table, sin_table, (f16*)q_out, (f16*)k_cache, (f16*)v_cache, (int)batch,
+                       (int)heads, (int)head_dim, (int)max_len);
+    return launched("qf_rope_kv_store");
+}
+
+extern "C" int qf_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int64_t* pos,
+                                   uint16_t* out, int64_t batch, int64_t heads, int64_t head_dim, int64_t max_len, void* stream) {
+    if (!q || !k_cache || !v_cache || !pos || !out) return fail("qf_decode_attention", "null pointer");
+    if (batch <= 0 || heads <= 0 || max_len <= 0 || batch > 65535) return fail("qf_decode_attention", "batch in 1..65535, heads and max_len positive");
+    const f16 *qp = (const f16*)q, *kp = (const f16*)k_cache, *vp = (const f16*)v_cache;
+    hipStream_t s = (hipStream_t)stream;
+    switch (head_dim) {
+        case 32: return launch_attention<4>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
+        case 64: return launch_attention<8>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
+        case 128: return launch_attention<16>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
+        case 256: return launch_attention<32>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
+        default: return fail("qf_decode_attention", "head_dim must be 32, 64, 128 or 256");
+    }
+}
+
+extern "C" int qf_silu_mul(const uint16_t* gate_up, uint16_t* out, int64_t rows, int64_t mlp, void* stream) {
+    if (!gate_up || !out) return fail("qf_silu_mul", "null pointer");
+    if (rows <= 0 || mlp <= 0 || mlp % 8 != 0) return fail("qf_silu_mul", "rows positive, mlp a positive multiple of 8");
+    const int64_t work = rows * (mlp / 8);
+    if (mlp > 0x7fffffff || work > (int64_t)0x7fffffff * kThreads) return fail("qf_silu_mul", "problem too large");
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((work + kThreads - 1) / kThreads)), dim3(kThreads), 0, (hipStream_t)stream,
+                       (const f16*)gate_up, (f16*)out, rows, (int)mlp);
+    return launched("qf_silu_mul");
+}

@@ -8,8 +8,11 @@ third_party/vllm-qfactory.patch), which need vLLM and model downloads.
 
 The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear modules; prefill
 (M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
-regimes through the layers' own row-count dispatch.  Everything else (embedding, RMSNorm, RoPE,
-attention over a static KV cache, SiLU, the fp16 lm_head) is plain PyTorch.  One decode step --
+regimes through the layers' own row-count dispatch.  Prefill runs everything else (embedding,
+RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch.  A decode
+step runs the steps between the linears as one HIP launch each (residual add + RMSNorm, RoPE + cache
+append, attention of the new position, SiLU * up: libqfactory_hip.so) -- nine launches per layer
+instead of about fifty; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
 Prints one JSON line per batch size: tokens/s over the decode phase, prefill time, and the share of
@@ -84,6 +87,10 @@ class QuantLlama:
         ang = torch.arange(shape.max_len, device="cuda", dtype=torch.float32)[:, None] * inv[None, :]
         self.cos, self.sin = ang.cos(), ang.sin()                                   # (max_len, hd/2) fp32
         self.linear = lambda lin, x: lin(x)                 # hook: tests swap in a dense fp32 evaluation
+        # buffers of the fused decode step (one new position per sequence)
+        f16 = dict(dtype=torch.float16, device="cuda")
+        self._hdn, self._q, self._att = (torch.empty(batch, h, **f16) for _ in range(3))
+        self._act = torch.empty(batch, shape.mlp, **f16)
 
     def _norm(self, x, w):
         xf = x.float()
@@ -122,6 +129,26 @@ class QuantLlama:
         last = self._norm(x[:, -1], self.final_norm)
         return last @ self.lm_head.T
 
+    def decode_step(self, tok, pos):
+        """tok (B, 1) int64, pos one-element int64 device tensor: logits (B, vocab) of the next token, like
+        ``forward`` at T = 1, with every step between the linears a single launch of libqfactory_hip.so."""
+        from qfactory import native
+        shape = self.shape
+        x = self.embed[tok[:, 0]]                                # (B, h): the residual stream, updated in place
+        delta = None
+        for li, layer in enumerate(self.layers):
+            native.add_rmsnorm(x, delta, layer["norm1"], self._hdn, shape.eps)
+            qkv = self.linear(layer["qkv"], self._hdn)
+            native.rope_kv_store(qkv, pos, self.cos, self.sin, self._q, self.k_cache[li], self.v_cache[li])
+            native.decode_attention(self._q, self.k_cache[li], self.v_cache[li], pos, self._att)
+            delta = self.linear(layer["o"], self._att)
+            native.add_rmsnorm(x, delta, layer["norm2"], self._hdn, shape.eps)
+            gate_up = self.linear(layer["gate_up"], self._hdn)
+            native.silu_mul(gate_up, self._act)
+            delta = self.linear(layer["down"], self._act)
+        native.add_rmsnorm(x, delta, self.final_norm, self._hdn, shape.eps)
+        return self._hdn @ self.lm_head.T
+
 
 def linears_time_us(model, M, reps=8):
     """Time of the quantized linears of one decode step at M rows: every layer's four kernels once,
@@ -152,7 +179,7 @@ def linears_time_us(model, M, reps=8):
     return t0.elapsed_time(t1) * 1e3 / reps
 
 
-def run(shape, batch, prompt_len, new_tokens, seed=0):
+def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
     assert prompt_len + new_tokens <= shape.max_len
     model = QuantLlama(shape, batch, seed)
     gen = torch.Generator(device="cuda").manual_seed(seed + 1)
@@ -172,7 +199,7 @@ def run(shape, batch, prompt_len, new_tokens, seed=0):
     tok0, pos0 = tok.clone(), pos.clone()
 
     def step():
-        lg = model.forward(tok, pos)
+        lg = model.forward(tok, pos) if torch_glue else model.decode_step(tok, pos)
         tok.copy_(lg.argmax(-1, keepdim=True))
         pos.add_(1)
 
@@ -203,7 +230,8 @@ def run(shape, batch, prompt_len, new_tokens, seed=0):
             "new_tokens": new_tokens, "decode_step_us": round(step_us, 1), "prefill_ms": round(prefill_s * 1e3, 2),
             "prefill_tokens_per_s": round(batch * prompt_len / prefill_s, 1),
             "quantized_linears_us_per_step": round(lin_us, 1), "quantized_linear_share": round(lin_us / step_us, 3),
-            "layers": shape.layers, "hidden": shape.hidden, "data": "random weights, random prompt ids"}
+            "layers": shape.layers, "hidden": shape.hidden, "data": "random weights, random prompt ids",
+            "between_linears": "torch ops" if torch_glue else "one HIP launch per step (libqfactory_hip.so)"}
 
 
 def main():
@@ -212,11 +240,12 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=128)
     ap.add_argument("--new-tokens", type=int, default=128)
     ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--torch-glue", action="store_true", help="PyTorch ops between the linears of a decode step")
     args = ap.parse_args()
     assert torch.cuda.is_available(), "decode_llama.py needs the MI355X"
     shape = LlamaShape(layers=args.layers, max_len=args.prompt_len + args.new_tokens)
     for batch in args.batches:
-        print(json.dumps(run(shape, batch, args.prompt_len, args.new_tokens)), flush=True)
+        print(json.dumps(run(shape, batch, args.prompt_len, args.new_tokens, torch_glue=args.torch_glue)), flush=True)
         torch.cuda.empty_cache()
 
 

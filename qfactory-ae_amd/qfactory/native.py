@@ -1,5 +1,5 @@
-"""ctypes binding of libqfactory_hip.so, the ahead-of-time HIP library (device-side repacking and
-the stream read / copy calibration kernels).  Its C ABI is declared in include/qfactory_hip.h.
+"""ctypes binding of libqfactory_hip.so, the ahead-of-time HIP library (device-side repacking, the
+stream read / copy calibration kernels and the per-token steps between the linears of a decoder layer).  Its C ABI is declared in include/qfactory_hip.h.
 
 The library is built in-tree with hipcc (``build()``; no GPU needed) and loaded lazily.  There is
 no substitute path: calling an entry point without the built library raises.
@@ -12,14 +12,14 @@ import threading
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(os.path.dirname(PKG_DIR), "csrc")
 REPO_INCLUDE = os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include")
-SOURCE = os.path.join(CSRC_DIR, "qfactory_hip.hip")
+SOURCES = [os.path.join(CSRC_DIR, "qfactory_hip.hip"), os.path.join(CSRC_DIR, "qfactory_decode.hip")]
 LIBRARY = os.path.join(CSRC_DIR, "libqfactory_hip.so")
 
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-std=c++20", "-shared", "-fPIC", "-O3",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 # name -> (restype, argtypes); mirrors include/qfactory_hip.h
-_P, _I64, _INT, _SZ = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+_P, _I64, _INT, _SZ, _F = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
 SIGNATURES = {
     "qf_version": (_INT, []),
     "qf_pack_weight": (_INT, [_P, _P, _I64, _I64, _INT, _P]),
@@ -27,6 +27,10 @@ SIGNATURES = {
     "qf_transpose_scale": (_INT, [_P, _P, _I64, _I64, _P]),
     "qf_stream_read": (_INT, [_P, _SZ, _P, _P]),
     "qf_stream_copy": (_INT, [_P, _P, _SZ, _P]),
+    "qf_add_rmsnorm": (_INT, [_P, _P, _P, _P, _I64, _I64, _F, _P]),
+    "qf_rope_kv_store": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    "qf_decode_attention": (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    "qf_silu_mul": (_INT, [_P, _P, _I64, _I64, _P]),
 }
 
 _lock = threading.Lock()
@@ -34,15 +38,15 @@ _lib = None
 
 
 def build(force=False):
-    """Compile csrc/qfactory_hip.hip for gfx950 into csrc/libqfactory_hip.so."""
+    """Compile csrc/*.hip for gfx950 into csrc/libqfactory_hip.so."""
     hipcc = os.environ.get("QFACTORY_HIPCC", "/opt/rocm/bin/hipcc")
-    if not force and os.path.exists(LIBRARY) and os.path.getmtime(LIBRARY) >= os.path.getmtime(SOURCE):
+    if not force and os.path.exists(LIBRARY) and os.path.getmtime(LIBRARY) >= max(os.path.getmtime(p) for p in SOURCES):
         return LIBRARY
     tmp = f"{LIBRARY}.tmp.{os.getpid()}"
-    cmd = [hipcc, "-x", "hip", SOURCE, "-o", tmp, *HIPCC_FLAGS, f"-I{REPO_INCLUDE}"]
+    cmd = [hipcc, "-x", "hip", *SOURCES, "-o", tmp, *HIPCC_FLAGS, f"-I{REPO_INCLUDE}"]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed on {SOURCE}:\n{proc.stderr}")
+        raise RuntimeError(f"hipcc failed on {SOURCES}:\n{proc.stderr}")
     os.replace(tmp, LIBRARY)
     return LIBRARY
 
@@ -111,3 +115,51 @@ def stream_read(src, sink):
 def stream_copy(dst, src):
     assert dst.numel() * dst.element_size() == src.numel() * src.element_size()
     _check(load().qf_stream_copy(dst.data_ptr(), src.data_ptr(), src.numel() * src.element_size(), _stream()), "qf_stream_copy")
+
+
+def _f16(t):
+    import torch
+    assert t.is_cuda and t.dtype == torch.float16 and t.is_contiguous()
+    return t.data_ptr()
+
+
+def add_rmsnorm(x, delta, weight, out, eps):
+    """x (rows, hidden) fp16 += delta (or None) in place; out = RMSNorm(x) * weight."""
+    rows, hidden = x.shape
+    assert out.shape == x.shape and weight.shape == (hidden,) and (delta is None or delta.shape == x.shape)
+    _check(load().qf_add_rmsnorm(_f16(x), None if delta is None else _f16(delta), _f16(weight), _f16(out), rows, hidden,
+                                 float(eps), _stream()), "qf_add_rmsnorm")
+    return out
+
+
+def rope_kv_store(qkv, pos, cos, sin, q_out, k_cache, v_cache):
+    """qkv (B, 3*H*hd) of the position pos (one-element int64 device tensor): rotated q to q_out (B, H*hd),
+    rotated k and v appended to the caches (B, H, max_len, hd)."""
+    import torch
+    B, H, max_len, hd = k_cache.shape
+    assert qkv.shape == (B, 3 * H * hd) and q_out.shape == (B, H * hd) and v_cache.shape == k_cache.shape
+    assert pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1
+    assert cos.dtype == torch.float32 and cos.is_contiguous() and cos.shape == (max_len, hd // 2) and sin.shape == cos.shape
+    assert sin.dtype == torch.float32 and sin.is_contiguous()
+    _check(load().qf_rope_kv_store(_f16(qkv), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), _f16(q_out), _f16(k_cache),
+                                   _f16(v_cache), B, H, hd, max_len, _stream()), "qf_rope_kv_store")
+    return q_out
+
+
+def decode_attention(q, k_cache, v_cache, pos, out):
+    """q (B, H*hd), caches (B, H, max_len, hd), pos one-element int64 device tensor -> out (B, H*hd)."""
+    import torch
+    B, H, max_len, hd = k_cache.shape
+    assert q.shape == (B, H * hd) and out.shape == q.shape and v_cache.shape == k_cache.shape
+    assert pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1
+    _check(load().qf_decode_attention(_f16(q), _f16(k_cache), _f16(v_cache), pos.data_ptr(), _f16(out), B, H, hd, max_len,
+                                      _stream()), "qf_decode_attention")
+    return out
+
+
+def silu_mul(gate_up, out):
+    """gate_up (rows, 2*mlp) -> out (rows, mlp) = silu(gate) * up."""
+    rows, two_mlp = gate_up.shape
+    assert out.shape == (rows, two_mlp // 2)
+    _check(load().qf_silu_mul(_f16(gate_up), _f16(out), rows, two_mlp // 2, _stream()), "qf_silu_mul")
+    return out

@@ -1,5 +1,6 @@
 """The Llama-shaped decode loop on a tiny model: logits with QLinear layers against the same model
-evaluated with dense fp32 matmuls on the dequantised weights (prefill and three decode steps)."""
+evaluated with dense fp32 matmuls on the dequantised weights (prefill and three decode steps), and
+the single-launch steps between the linears of a decode token against the PyTorch ops they replace."""
 import pytest
 import torch
 
@@ -47,3 +48,117 @@ def test_graph_decode_runs_and_reports():
     shape = decode_llama.LlamaShape(layers=2, hidden=256, heads=4, mlp=512, vocab=1000, max_len=32, group_size=64)
     rec = decode_llama.run(shape, batch=2, prompt_len=8, new_tokens=6)
     assert rec["value"] > 0 and 0 < rec["quantized_linear_share"] <= 1.5
+
+
+# ---- the per-token steps between the linears (libqfactory_hip.so through its C ABI) ----
+
+def _gen(seed):
+    return torch.Generator(device="cuda").manual_seed(seed)
+
+
+@pytest.mark.parametrize("rows,hidden,with_delta", [(1, 4096, True), (16, 4096, False), (3, 256, True), (5, 11008, True),
+                                                    (2, 16384, True), (7, 8, False)])
+def test_add_rmsnorm_matches_torch(rows, hidden, with_delta):
+    from qfactory import native
+    g = _gen(rows * 31 + hidden)
+    x = torch.randn(rows, hidden, device="cuda", generator=g).to(torch.float16)
+    delta = (torch.randn(rows, hidden, device="cuda", generator=g) * 0.3).to(torch.float16) if with_delta else None
+    w = (torch.rand(hidden, device="cuda", generator=g) + 0.5).to(torch.float16)
+    want_x = x + delta if with_delta else x.clone()
+    xf = want_x.float()
+    want = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).to(torch.float16) * w
+    out = torch.empty_like(x)
+    native.add_rmsnorm(x, delta, w, out, 1e-5)
+    assert torch.equal(x, want_x)                                   # the fp16 residual add is exact
+    # the mean of squares is summed in another order: at most one fp16 ulp on a few elements
+    assert (out.float() - want.float()).abs().max() <= 2e-3 * want.float().abs().max()
+    assert ((out.float() - want.float()).norm() / want.float().norm()).item() <= 2e-4
+
+
+@pytest.mark.parametrize("B,H,hd,max_len,pos", [(1, 32, 128, 256, 0), (2, 4, 64, 32, 8), (16, 32, 128, 256, 200),
+                                                (3, 5, 32, 40, 39), (2, 2, 256, 300, 299)])
+def test_rope_cache_append_and_attention_match_torch(B, H, hd, max_len, pos):
+    import torch.nn.functional as F
+    from qfactory import native
+    g = _gen(B * 1000 + pos)
+    qkv = torch.randn(B, 3 * H * hd, device="cuda", generator=g).to(torch.float16)
+    k_cache = torch.randn(B, H, max_len, hd, device="cuda", generator=g).to(torch.float16)
+    v_cache = torch.randn(B, H, max_len, hd, device="cuda", generator=g).to(torch.float16)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, device="cuda", dtype=torch.float32) / hd))
+    ang = torch.arange(max_len, device="cuda", dtype=torch.float32)[:, None] * inv[None, :]
+    cos, sin = ang.cos(), ang.sin()
+    pos_t = torch.tensor([pos], device="cuda", dtype=torch.int64)
+
+    def rope(x):                                                    # (B, H, hd), pairs (2i, 2i+1)
+        xf = x.float()
+        x0, x1 = xf[..., 0::2], xf[..., 1::2]
+        return torch.stack((x0 * cos[pos] - x1 * sin[pos], x0 * sin[pos] + x1 * cos[pos]), dim=-1).flatten(-2).to(torch.float16)
+
+    q3 = qkv.reshape(B, 3, H, hd)
+    want_q, want_k = rope(q3[:, 0]), rope(q3[:, 1])
+    want_kc, want_vc = k_cache.clone(), v_cache.clone()
+    want_kc[:, :, pos], want_vc[:, :, pos] = want_k, q3[:, 2]
+    mask = (torch.arange(max_len, device="cuda") <= pos)[None, None, None]
+    want_att = F.scaled_dot_product_attention(want_q[:, :, None].float(), want_kc.float(), want_vc.float(), attn_mask=mask)
+    want_att = want_att[:, :, 0].reshape(B, H * hd)
+
+    q_out, att = torch.empty(B, H * hd, dtype=torch.float16, device="cuda"), torch.empty(B, H * hd, dtype=torch.float16, device="cuda")
+    native.rope_kv_store(qkv, pos_t, cos, sin, q_out, k_cache, v_cache)
+    native.decode_attention(q_out, k_cache, v_cache, pos_t, att)
+    # rotation: fp32 products of the same table entries, rounded once to fp16 (a fused multiply-add may differ by one ulp)
+    assert (q_out.float() - want_q.reshape(B, -1).float()).abs().max() <= 4e-3
+    assert (k_cache.float() - want_kc.float()).abs().max() <= 4e-3
+    assert torch.equal(v_cache, want_vc)
+    untouched = torch.arange(max_len, device="cuda") != pos
+    assert torch.equal(k_cache[:, :, untouched], want_kc[:, :, untouched])
+    assert ((att.float() - want_att).norm() / want_att.norm()).item() <= 2e-3
+    assert (att.float() - want_att).abs().max() <= 1e-2 * want_att.abs().max() + 2e-3
+
+
+def test_rope_writes_nothing_for_a_position_outside_the_cache():
+    from qfactory import native
+    B, H, hd, max_len = 2, 4, 64, 16
+    qkv = torch.randn(B, 3 * H * hd, device="cuda").to(torch.float16)
+    k_cache = torch.zeros(B, H, max_len, hd, dtype=torch.float16, device="cuda")
+    v_cache = torch.zeros_like(k_cache)
+    cos = torch.ones(max_len, hd // 2, device="cuda")
+    sin = torch.zeros_like(cos)
+    q_out = torch.zeros(B, H * hd, dtype=torch.float16, device="cuda")
+    native.rope_kv_store(qkv, torch.tensor([max_len], device="cuda"), cos, sin, q_out, k_cache, v_cache)
+    torch.cuda.synchronize()
+    assert not k_cache.any() and not v_cache.any() and not q_out.any()
+
+
+@pytest.mark.parametrize("rows,mlp", [(1, 11008), (16, 11008), (3, 512), (64, 8)])
+def test_silu_mul_matches_torch(rows, mlp):
+    import torch.nn.functional as F
+    from qfactory import native
+    gu = (torch.randn(rows, 2 * mlp, device="cuda", generator=_gen(rows + mlp)) * 3).to(torch.float16)
+    want = F.silu(gu[:, :mlp]) * gu[:, mlp:]
+    out = torch.empty(rows, mlp, dtype=torch.float16, device="cuda")
+    native.silu_mul(gu, out)
+    assert (out.float() - want.float()).abs().max() <= 2e-3 * want.float().abs().max()      # exp() of two libraries: one ulp
+    assert ((out.float() - want.float()).norm() / want.float().norm()).item() <= 2e-4
+
+
+def test_decode_step_matches_the_torch_evaluation_of_the_same_model():
+    import decode_llama
+    shape = decode_llama.LlamaShape(layers=2, hidden=256, heads=4, mlp=512, vocab=1000, max_len=32, group_size=64)
+    model = decode_llama.QuantLlama(shape, batch=2, seed=5)
+    prompt = torch.randint(0, shape.vocab, (2, 8), device="cuda", generator=_gen(6))
+
+    def run(step_fn):
+        model.k_cache.zero_(), model.v_cache.zero_()
+        logits = [model.forward(prompt, torch.arange(8, device="cuda"))]
+        for i in range(4):
+            tok = logits[-1].argmax(-1, keepdim=True)
+            logits.append(step_fn(tok, torch.tensor([8 + i], device="cuda")).clone())
+        return torch.stack(logits).float(), model.k_cache.clone(), model.v_cache.clone()
+
+    want, want_k, want_v = run(model.forward)
+    got, got_k, got_v = run(model.decode_step)
+    assert torch.isfinite(got).all()
+    assert ((got - want).norm() / want.norm()).item() <= 3e-3
+    assert torch.equal(got.argmax(-1), want.argmax(-1))
+    assert ((got_k.float() - want_k.float()).norm() / want_k.float().norm()).item() <= 3e-3
+    assert ((got_v.float() - want_v.float()).norm() / want_v.float().norm()).item() <= 3e-3
