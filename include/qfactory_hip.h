@@ -69,6 +69,9 @@ int qf_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
  *   [0, max_len).
  * qf_decode_attention: out (batch, heads*head_dim) = softmax(q k^T / sqrt(head_dim)) v over cache
  *   positions 0 .. *pos.  head_dim in {32, 64, 128, 256}.
+ * qf_rope_decode_attention: the two above in one launch, straight from the QKV projection: rotates q and k
+ *   of position *pos, appends k and v to the caches and writes the attention output; nothing is written
+ *   if *pos is outside [0, max_len).  Results equal qf_rope_kv_store followed by qf_decode_attention.
  * qf_silu_mul: out (rows, mlp) = fp16(silu(gate_up[:, :mlp])) * gate_up[:, mlp:]; mlp a multiple of 8.
  */
 int qf_add_rmsnorm(uint16_t* x, const uint16_t* delta, const uint16_t* weight, uint16_t* out, int64_t rows,
@@ -78,6 +81,9 @@ int qf_rope_kv_store(const uint16_t* qkv, const int64_t* pos, const float* cos_t
                      int64_t head_dim, int64_t max_len, void* stream);
 int qf_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int64_t* pos,
                         uint16_t* out, int64_t batch, int64_t heads, int64_t head_dim, int64_t max_len, void* stream);
+int qf_rope_decode_attention(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
+                             uint16_t* k_cache, uint16_t* v_cache, uint16_t* out, int64_t batch, int64_t heads,
+                             int64_t head_dim, int64_t max_len, void* stream);
 int qf_silu_mul(const uint16_t* gate_up, uint16_t* out, int64_t rows, int64_t mlp, void* stream);
 
 #ifdef __cplusplus

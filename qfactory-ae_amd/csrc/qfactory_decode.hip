@@ -45,16 +45,16 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// Sum (MAX = false) or maximum (MAX = true) over the block; `slots` holds kWaves floats and may be
-// reused right after the call returns.
-template <bool MAX>
+// Sum (MAX = false) or maximum (MAX = true) over a block of WAVES waves; `slots` holds WAVES floats and
+// may be reused right after the call returns.
+template <bool MAX, int WAVES>
 __device__ __forceinline__ float block_reduce(float v, float* slots) {
     v = MAX ? wave_max(v) : wave_sum(v);
     if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
     __syncthreads();
     float r = slots[0];
 #pragma unroll
-    for (int w = 1; w < kWaves; w++) r = MAX ? fmaxf(r, slots[w]) : r + slots[w];
+    for (int w = 1; w < WAVES; w++) r = MAX ? fmaxf(r, slots[w]) : r + slots[w];
     __syncthreads();
     return r;
 }
@@ -70,12 +70,13 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_kernel(f16* __restrict__
                                                                int hidden, float eps) {
     __shared__ float slots[kWaves];
     const size_t row = (size_t)blockIdx.x * hidden;
-    f16x8 v[kNormVec];
+    f16x8 v[kNormVec], w[kNormVec];
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < kNormVec; i++) {
         const int c = (threadIdx.x + i * kThreads) * 8;
         if (c < hidden) {
+            w[i] = *reinterpret_cast<const f16x8*>(weight + c);       // requested with x: not a second round trip after the reduction
             v[i] = *reinterpret_cast<const f16x8*>(x + row + c);
             if (delta) {
                 v[i] = v[i] + *reinterpret_cast<const f16x8*>(delta + row + c);      // fp16 add, as the residual stream is fp16
@@ -85,15 +86,14 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_kernel(f16* __restrict__
             for (int e = 0; e < 8; e++) ss += (float)v[i][e] * (float)v[i][e];
         }
     }
-    const float r = rsqrtf(block_reduce<false>(ss, slots) / (float)hidden + eps);
+    const float r = rsqrtf(block_reduce<false, kWaves>(ss, slots) / (float)hidden + eps);
 #pragma unroll
     for (int i = 0; i < kNormVec; i++) {
         const int c = (threadIdx.x + i * kThreads) * 8;
         if (c < hidden) {
-            const f16x8 w = *reinterpret_cast<const f16x8*>(weight + c);
             f16x8 o;
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = (f16)((float)v[i][e] * r) * w[e];
+            for (int e = 0; e < 8; e++) o[e] = (f16)((float)v[i][e] * r) * w[i][e];
             *reinterpret_cast<f16x8*>(out + row + c) = o;
         }
     }
@@ -107,6 +107,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_kernel(const f16* __re
                                                                  const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                  f16* __restrict__ q_out, f16* __restrict__ k_cache,
                                                                  f16* __restrict__ v_cache, int batch, int heads, int hd, int max_len) {
+#pragma clang fp contract(off)                                // two products and a sum, each rounded, like the ops this replaces
     const int64_t pos = pos_ptr[0];
     if (pos < 0 || pos >= max_len) return;                    // nothing is written for a position outside the cache
     const int half = hd / 2;
@@ -131,40 +132,89 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_kernel(const f16* __re
 }
 
 // ---------------------------------------------------------------------------------------------
-// Attention of one query per (sequence, head) over cache positions 0 .. pos.  LPK = hd/8 lanes share
-// a key or value row (16 bytes each).  Scores -> LDS, block max and sum, then every group of LPK lanes
-// walks its share of the value rows and the groups' partial outputs meet in LDS.
+// Attention of one query per (sequence, head) over cache positions 0 .. pos, one block of 16 or 4 waves per
+// (head, sequence).  LPK = hd/8 lanes share a key or value row (16 bytes each), so a block covers
+// 1024/LPK or 256/LPK positions per pass.  Scores -> LDS, block max and sum, then every group of LPK lanes walks its
+// share of the value rows; the groups of a wave are summed by lane shuffles, the waves through LDS.
+//
+// FUSED: q, k, v of the new position come straight from the QKV projection (row b = [3][H][hd]); q and k are
+// rotated here (pairs (2i, 2i+1), angles of table row pos, rounded to fp16 as a separate rotation kernel would
+// store them), k and v are appended to the cache, and the new position is served from LDS rather than
+// re-read from memory the block has just written.
 // ---------------------------------------------------------------------------------------------
-template <int LPK>
-__global__ __launch_bounds__(kThreads) void decode_attention_kernel(const f16* __restrict__ q, const f16* __restrict__ k_cache,
-                                                                    const f16* __restrict__ v_cache, const int64_t* __restrict__ pos_ptr,
-                                                                    f16* __restrict__ out, int heads, int max_len, float scale) {
+// Few (sequence, head) pairs: 16 waves per block shorten the walk over the cache; many: 4 waves per block
+// keep more blocks resident (measured with 32 heads: 16 waves are faster at batch 16, slower at batch 64).
+constexpr int kAttnThreadsFew = 1024, kAttnThreadsMany = 256;
+constexpr int kAttnManyBlocks = 1024;
+
+__device__ __forceinline__ f16x8 rotate8(const f16x8 x, const float* __restrict__ c, const float* __restrict__ s) {
+#pragma clang fp contract(off)                                // same roundings as rope_kv_store_kernel
+    f16x8 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float x0 = (float)x[2 * i], x1 = (float)x[2 * i + 1];
+        r[2 * i] = (f16)(x0 * c[i] - x1 * s[i]);
+        r[2 * i + 1] = (f16)(x0 * s[i] + x1 * c[i]);
+    }
+    return r;
+}
+
+template <int LPK, bool FUSED, int THREADS>
+__global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __restrict__ q_or_qkv, f16* __restrict__ k_cache,
+                                                                        f16* __restrict__ v_cache, const int64_t* __restrict__ pos_ptr,
+                                                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                        f16* __restrict__ out, int heads, int max_len, float scale) {
     constexpr int HD = LPK * 8;
-    constexpr int GROUPS = kThreads / LPK;
+    constexpr int GROUPS = THREADS / LPK;
+    constexpr int WAVES = THREADS / 64;
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float* sc = smem;                                          // [max_len]
-    float* part = smem + max_len;                              // [GROUPS][HD]
-    __shared__ float slots[kWaves];
+    float* part = smem + max_len;                              // [WAVES][HD]
+    __shared__ float slots[WAVES];
+    __shared__ __attribute__((aligned(16))) f16 new_k[HD], new_v[HD];
     const int h = blockIdx.x, b = blockIdx.y;
-    int64_t pos = pos_ptr[0];
-    if (pos < 0) return;
+    const int64_t pos = pos_ptr[0];
+    if (pos < 0 || (FUSED && pos >= max_len)) return;          // uniform over the block; nothing is written
     const int n = (int)(pos < max_len ? pos + 1 : max_len);    // keys 0 .. n-1
     const int g = threadIdx.x / LPK, j = threadIdx.x % LPK;
     const size_t head = ((size_t)b * heads + h);
-    const f16* kc = k_cache + head * max_len * HD;
-    const f16* vc = v_cache + head * max_len * HD;
+    f16* kc = k_cache + head * max_len * HD;
+    f16* vc = v_cache + head * max_len * HD;
 
-    const f16x8 qv = *reinterpret_cast<const f16x8*>(q + head * HD + j * 8);
+    f16x8 qv;
+    if constexpr (FUSED) {
+        const f16* row = q_or_qkv + (size_t)b * 3 * heads * HD + (size_t)h * HD + j * 8;
+        float c[4], s[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            c[i] = cos_t[pos * (HD / 2) + j * 4 + i];
+            s[i] = sin_t[pos * (HD / 2) + j * 4 + i];
+        }
+        qv = rotate8(*reinterpret_cast<const f16x8*>(row), c, s);
+        if (g == 0) {
+            const f16x8 kr = rotate8(*reinterpret_cast<const f16x8*>(row + (size_t)heads * HD), c, s);
+            const f16x8 vv = *reinterpret_cast<const f16x8*>(row + (size_t)2 * heads * HD);
+            *reinterpret_cast<f16x8*>(kc + (size_t)pos * HD + j * 8) = kr;
+            *reinterpret_cast<f16x8*>(vc + (size_t)pos * HD + j * 8) = vv;
+            *reinterpret_cast<f16x8*>(new_k + j * 8) = kr;
+            *reinterpret_cast<f16x8*>(new_v + j * 8) = vv;
+        }
+        __syncthreads();
+    } else {
+        qv = *reinterpret_cast<const f16x8*>(q_or_qkv + head * HD + j * 8);
+    }
     float qf[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) qf[e] = (float)qv[e] * scale;
 
     float local_max = -INFINITY;
+#pragma unroll 2
     for (int p0 = 0; p0 < n; p0 += GROUPS) {
         const int p = p0 + g;
         float d = 0.f;
         if (p < n) {
-            const f16x8 kv = *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
+            const f16x8 kv = (FUSED && p == (int)pos) ? *reinterpret_cast<const f16x8*>(new_k + j * 8)
+                                                      : *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
 #pragma unroll
             for (int e = 0; e < 8; e++) d += qf[e] * (float)kv[e];
         }
@@ -175,28 +225,38 @@ __global__ __launch_bounds__(kThreads) void decode_attention_kernel(const f16* _
             local_max = fmaxf(local_max, d);
         }
     }
-    const float mx = block_reduce<true>(local_max, slots);     // also publishes sc[] to the block
+    const float mx = block_reduce<true, WAVES>(local_max, slots);      // also publishes sc[] to the block
     float local_sum = 0.f;
-    for (int p = threadIdx.x; p < n; p += kThreads) {
+    for (int p = threadIdx.x; p < n; p += THREADS) {
         const float e = __expf(sc[p] - mx);
         sc[p] = e;
         local_sum += e;
     }
-    const float total = block_reduce<false>(local_sum, slots);
+    const float total = block_reduce<false, WAVES>(local_sum, slots);
 
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
     for (int p = g; p < n; p += GROUPS) {
         const float w = sc[p];
-        const f16x8 vv = *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
+        const f16x8 vv = (FUSED && p == (int)pos) ? *reinterpret_cast<const f16x8*>(new_v + j * 8)
+                                                  : *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += w * (float)vv[e];
     }
+    // the 64/LPK groups of a wave: lanes that differ in the bits above log2(LPK)
 #pragma unroll
-    for (int e = 0; e < 8; e++) part[g * HD + j * 8 + e] = acc[e];
+    for (int o = LPK; o < 64; o <<= 1)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += __shfl_xor(acc[e], o, 64);
+    if ((threadIdx.x & 63) < LPK) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) part[(threadIdx.x >> 6) * HD + j * 8 + e] = acc[e];
+    }
     __syncthreads();
-    for (int d = threadIdx.x; d < HD; d += kThreads) {
+    for (int d = threadIdx.x; d < HD; d += THREADS) {
         float s = 0.f;
-        for (int gg = 0; gg < GROUPS; gg++) s += part[gg * HD + d];
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) s += part[w * HD + d];
         out[head * HD + d] = (f16)(s / total);
     }
 }
@@ -222,15 +282,40 @@ __global__ __launch_bounds__(kThreads) void silu_mul_kernel(const f16* __restric
     *reinterpret_cast<f16x8*>(out + m * mlp + c) = o;
 }
 
-template <int LPK>
-int launch_attention(const f16* q, const f16* k, const f16* v, const int64_t* pos, f16* out, int batch, int heads,
-                     int max_len, hipStream_t stream) {
+template <int LPK, bool FUSED>
+int launch_attention(const char* fn, const f16* q_or_qkv, f16* k, f16* v, const int64_t* pos, const float* cos_t, const float* sin_t,
+                     f16* out, int batch, int heads, int max_len, hipStream_t stream) {
     constexpr int HD = LPK * 8;
-    const size_t lds = ((size_t)max_len + (size_t)(kThreads / LPK) * HD) * sizeof(float);
-    if (lds > 64 * 1024) return fail("qf_decode_attention", "max_len too large for the score buffer in LDS");
-    hipLaunchKernelGGL(decode_attention_kernel<LPK>, dim3(heads, batch), dim3(kThreads), lds, stream, q, k, v, pos, out,
-                       heads, max_len, 1.0f / sqrtf((float)HD));
-    return launched("qf_decode_attention");
+    const float scale = 1.0f / sqrtf((float)HD);
+    const bool many = (int64_t)batch * heads >= kAttnManyBlocks;
+    const size_t lds = ((size_t)max_len + (size_t)((many ? kAttnThreadsMany : kAttnThreadsFew) / 64) * HD) * sizeof(float);
+    if (lds > 60 * 1024) return fail(fn, "max_len too large for the score buffer in LDS");
+    if (many)
+        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsMany>), dim3(heads, batch), dim3(kAttnThreadsMany), lds,
+                           stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
+    else
+        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsFew>), dim3(heads, batch), dim3(kAttnThreadsFew), lds,
+                           stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
+    return launched(fn);
+}
+
+template <bool FUSED>
+int dispatch_attention(const char* fn, const uint16_t* q_or_qkv, uint16_t* k_cache, uint16_t* v_cache, const int64_t* pos,
+                       const float* cos_t, const float* sin_t, uint16_t* out, int64_t batch, int64_t heads, int64_t head_dim,
+                       int64_t max_len, void* stream) {
+    if (batch <= 0 || heads <= 0 || max_len <= 0 || batch > 65535 || heads > 0x7fffffff || max_len > 0x7fffffff)
+        return fail(fn, "batch in 1..65535, heads and max_len positive");
+    const f16* qp = (const f16*)q_or_qkv;
+    f16 *kp = (f16*)k_cache, *vp = (f16*)v_cache, *op = (f16*)out;
+    hipStream_t s = (hipStream_t)stream;
+    const int B = (int)batch, H = (int)heads, L = (int)max_len;
+    switch (head_dim) {
+        case 32: return launch_attention<4, FUSED>(fn, qp, kp, vp, pos, cos_t, sin_t, op, B, H, L, s);
+        case 64: return launch_attention<8, FUSED>(fn, qp, kp, vp, pos, cos_t, sin_t, op, B, H, L, s);
+        case 128: return launch_attention<16, FUSED>(fn, qp, kp, vp, pos, cos_t, sin_t, op, B, H, L, s);
+        case 256: return launch_attention<32, FUSED>(fn, qp, kp, vp, pos, cos_t, sin_t, op, B, H, L, s);
+        default: return fail(fn, "head_dim must be 32, 64, 128 or 256");
+    }
 }
 
 }  // namespace
@@ -263,16 +348,17 @@ extern "C" int qf_rope_kv_store(const uint16_t* qkv, const int64_t* pos, const f
 extern "C" int qf_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int64_t* pos,
                                    uint16_t* out, int64_t batch, int64_t heads, int64_t head_dim, int64_t max_len, void* stream) {
     if (!q || !k_cache || !v_cache || !pos || !out) return fail("qf_decode_attention", "null pointer");
-    if (batch <= 0 || heads <= 0 || max_len <= 0 || batch > 65535) return fail("qf_decode_attention", "batch in 1..65535, heads and max_len positive");
-    const f16 *qp = (const f16*)q, *kp = (const f16*)k_cache, *vp = (const f16*)v_cache;
-    hipStream_t s = (hipStream_t)stream;
-    switch (head_dim) {
-        case 32: return launch_attention<4>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
-        case 64: return launch_attention<8>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
-        case 128: return launch_attention<16>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
-        case 256: return launch_attention<32>(qp, kp, vp, pos, (f16*)out, (int)batch, (int)heads, (int)max_len, s);
-        default: return fail("qf_decode_attention", "head_dim must be 32, 64, 128 or 256");
-    }
+    // the caches are only read on this path
+    return dispatch_attention<false>("qf_decode_attention", q, const_cast<uint16_t*>(k_cache), const_cast<uint16_t*>(v_cache), pos,
+                                     nullptr, nullptr, out, batch, heads, head_dim, max_len, stream);
+}
+
+extern "C" int qf_rope_decode_attention(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
+                                        uint16_t* k_cache, uint16_t* v_cache, uint16_t* out, int64_t batch, int64_t heads,
+                                        int64_t head_dim, int64_t max_len, void* stream) {
+    if (!qkv || !pos || !cos_table || !sin_table || !k_cache || !v_cache || !out) return fail("qf_rope_decode_attention", "null pointer");
+    return dispatch_attention<true>("qf_rope_decode_attention", qkv, k_cache, v_cache, pos, cos_table, sin_table, out, batch, heads,
+                                    head_dim, max_len, stream);
 }
 
 extern "C" int qf_silu_mul(const uint16_t* gate_up, uint16_t* out, int64_t rows, int64_t mlp, void* stream) {

@@ -11,7 +11,7 @@ The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear 
 regimes through the layers' own row-count dispatch.  Prefill runs everything else (embedding,
 RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch.  A decode
 step runs the steps between the linears as one HIP launch each (residual add + RMSNorm, RoPE + cache
-append, attention of the new position, SiLU * up: libqfactory_hip.so) -- nine launches per layer
+append + attention of the new position, SiLU * up: libqfactory_hip.so) -- eight launches per layer
 instead of about fifty; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
@@ -89,7 +89,7 @@ class QuantLlama:
         self.linear = lambda lin, x: lin(x)                 # hook: tests swap in a dense fp32 evaluation
         # buffers of the fused decode step (one new position per sequence)
         f16 = dict(dtype=torch.float16, device="cuda")
-        self._hdn, self._q, self._att = (torch.empty(batch, h, **f16) for _ in range(3))
+        self._hdn, self._att = (torch.empty(batch, h, **f16) for _ in range(2))
         self._act = torch.empty(batch, shape.mlp, **f16)
 
     def _norm(self, x, w):
@@ -139,8 +139,7 @@ class QuantLlama:
         for li, layer in enumerate(self.layers):
             native.add_rmsnorm(x, delta, layer["norm1"], self._hdn, shape.eps)
             qkv = self.linear(layer["qkv"], self._hdn)
-            native.rope_kv_store(qkv, pos, self.cos, self.sin, self._q, self.k_cache[li], self.v_cache[li])
-            native.decode_attention(self._q, self.k_cache[li], self.v_cache[li], pos, self._att)
+            native.rope_decode_attention(qkv, pos, self.cos, self.sin, self.k_cache[li], self.v_cache[li], self._att)
             delta = self.linear(layer["o"], self._att)
             native.add_rmsnorm(x, delta, layer["norm2"], self._hdn, shape.eps)
             gate_up = self.linear(layer["gate_up"], self._hdn)

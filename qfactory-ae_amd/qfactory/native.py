@@ -30,6 +30,7 @@ SIGNATURES = {
     "qf_add_rmsnorm": (_INT, [_P, _P, _P, _P, _I64, _I64, _F, _P]),
     "qf_rope_kv_store": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_decode_attention": (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    "qf_rope_decode_attention": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_silu_mul": (_INT, [_P, _P, _I64, _I64, _P]),
 }
 
@@ -154,6 +155,20 @@ def decode_attention(q, k_cache, v_cache, pos, out):
     assert pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1
     _check(load().qf_decode_attention(_f16(q), _f16(k_cache), _f16(v_cache), pos.data_ptr(), _f16(out), B, H, hd, max_len,
                                       _stream()), "qf_decode_attention")
+    return out
+
+
+def rope_decode_attention(qkv, pos, cos, sin, k_cache, v_cache, out):
+    """rope_kv_store and decode_attention in one launch: qkv (B, 3*H*hd) of position pos -> out (B, H*hd);
+    rotated k and v are appended to the caches (B, H, max_len, hd)."""
+    import torch
+    B, H, max_len, hd = k_cache.shape
+    assert qkv.shape == (B, 3 * H * hd) and out.shape == (B, H * hd) and v_cache.shape == k_cache.shape
+    assert pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1
+    assert cos.dtype == torch.float32 and cos.is_contiguous() and cos.shape == (max_len, hd // 2)
+    assert sin.dtype == torch.float32 and sin.is_contiguous() and sin.shape == cos.shape
+    _check(load().qf_rope_decode_attention(_f16(qkv), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), _f16(k_cache),
+                                           _f16(v_cache), _f16(out), B, H, hd, max_len, _stream()), "qf_rope_decode_attention")
     return out
 
 

@@ -76,7 +76,7 @@ def test_add_rmsnorm_matches_torch(rows, hidden, with_delta):
 
 
 @pytest.mark.parametrize("B,H,hd,max_len,pos", [(1, 32, 128, 256, 0), (2, 4, 64, 32, 8), (16, 32, 128, 256, 200),
-                                                (3, 5, 32, 40, 39), (2, 2, 256, 300, 299)])
+                                                (3, 5, 32, 40, 39), (2, 2, 256, 300, 299), (40, 32, 64, 64, 50)])
 def test_rope_cache_append_and_attention_match_torch(B, H, hd, max_len, pos):
     import torch.nn.functional as F
     from qfactory import native
@@ -103,8 +103,13 @@ def test_rope_cache_append_and_attention_match_torch(B, H, hd, max_len, pos):
     want_att = want_att[:, :, 0].reshape(B, H * hd)
 
     q_out, att = torch.empty(B, H * hd, dtype=torch.float16, device="cuda"), torch.empty(B, H * hd, dtype=torch.float16, device="cuda")
+    k_before, v_before = k_cache.clone(), v_cache.clone()
     native.rope_kv_store(qkv, pos_t, cos, sin, q_out, k_cache, v_cache)
     native.decode_attention(q_out, k_cache, v_cache, pos_t, att)
+    # the single-launch form gives the same bits as the two steps
+    att_fused = torch.empty_like(att)
+    native.rope_decode_attention(qkv, pos_t, cos, sin, k_before, v_before, att_fused)
+    assert torch.equal(k_before, k_cache) and torch.equal(v_before, v_cache) and torch.equal(att_fused, att)
     # rotation: fp32 products of the same table entries, rounded once to fp16 (a fused multiply-add may differ by one ulp)
     assert (q_out.float() - want_q.reshape(B, -1).float()).abs().max() <= 4e-3
     assert (k_cache.float() - want_kc.float()).abs().max() <= 4e-3
@@ -125,6 +130,8 @@ def test_rope_writes_nothing_for_a_position_outside_the_cache():
     sin = torch.zeros_like(cos)
     q_out = torch.zeros(B, H * hd, dtype=torch.float16, device="cuda")
     native.rope_kv_store(qkv, torch.tensor([max_len], device="cuda"), cos, sin, q_out, k_cache, v_cache)
+    native.rope_decode_attention(qkv, torch.tensor([max_len], device="cuda"), cos, sin, k_cache, v_cache, q_out)
+    native.rope_decode_attention(qkv, torch.tensor([-1], device="cuda"), cos, sin, k_cache, v_cache, q_out)
     torch.cuda.synchronize()
     assert not k_cache.any() and not v_cache.any() and not q_out.any()
 
