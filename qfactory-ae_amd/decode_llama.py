@@ -8,8 +8,9 @@ third_party/vllm-qfactory.patch), which need vLLM and model downloads.
 
 The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear modules; prefill
 (M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
-regimes through the layers' own row-count dispatch.  Prefill runs everything else (embedding,
-RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch.  A decode
+regimes through the layers' own row-count dispatch.  ``forward`` runs everything else (embedding,
+RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch; ``prefill``
+replaces its norm and SiLU steps by single launches.  A decode
 step runs the steps between the linears as one HIP launch each (residual add + RMSNorm, RoPE + cache
 append + attention of the new position, SiLU * up: libqfactory_hip.so) -- eight launches per layer
 instead of about fifty; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
@@ -129,6 +130,33 @@ class QuantLlama:
         last = self._norm(x[:, -1], self.final_norm)
         return last @ self.lm_head.T
 
+    def prefill(self, tokens, pos):
+        """``forward`` with the residual add + RMSNorm and SiLU * up steps as single launches of
+        libqfactory_hip.so (any number of rows); RoPE, the cache update and causal attention stay PyTorch ops."""
+        from qfactory import native
+        shape = self.shape
+        B, T = tokens.shape
+        H, hd = shape.heads, shape.hidden // shape.heads
+        x = self.embed[tokens].reshape(B * T, shape.hidden)                          # residual stream, updated in place
+        hdn = torch.empty_like(x)
+        act = torch.empty(B * T, shape.mlp, dtype=torch.float16, device="cuda")
+        mask = (torch.arange(shape.max_len, device="cuda")[None, :] <= pos[:, None])[None, None]
+        delta = None
+        for li, layer in enumerate(self.layers):
+            native.add_rmsnorm(x, delta, layer["norm1"], hdn, shape.eps)
+            qkv = self.linear(layer["qkv"], hdn).reshape(B, T, 3, H, hd).permute(2, 0, 3, 1, 4)
+            q, k, v = self._rope(qkv[0], pos), self._rope(qkv[1], pos), qkv[2]
+            self.k_cache[li].index_copy_(2, pos, k)
+            self.v_cache[li].index_copy_(2, pos, v)
+            att = F.scaled_dot_product_attention(q, self.k_cache[li], self.v_cache[li], attn_mask=mask)
+            delta = self.linear(layer["o"], att.permute(0, 2, 1, 3).reshape(B * T, shape.hidden))
+            native.add_rmsnorm(x, delta, layer["norm2"], hdn, shape.eps)
+            native.silu_mul(self.linear(layer["gate_up"], hdn), act)
+            delta = self.linear(layer["down"], act)
+        last = (x + delta).reshape(B, T, shape.hidden)[:, -1].contiguous()
+        native.add_rmsnorm(last, None, self.final_norm, last, shape.eps)
+        return last @ self.lm_head.T
+
     def decode_step(self, tok, pos):
         """tok (B, 1) int64, pos one-element int64 device tensor: logits (B, vocab) of the next token, like
         ``forward`` at T = 1, with every step between the linears a single launch of libqfactory_hip.so."""
@@ -185,10 +213,11 @@ def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
     prompt = torch.randint(0, shape.vocab, (batch, prompt_len), device="cuda", generator=gen)
 
     # ---- prefill (eager; also compiles / warms the large-M specialisations on its first call) ----
-    model.forward(prompt, torch.arange(prompt_len, device="cuda"))
+    prefill = model.forward if torch_glue else model.prefill
+    prefill(prompt, torch.arange(prompt_len, device="cuda"))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    logits = model.forward(prompt, torch.arange(prompt_len, device="cuda"))
+    logits = prefill(prompt, torch.arange(prompt_len, device="cuda"))
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
 

@@ -164,6 +164,9 @@ def test_decode_step_matches_the_torch_evaluation_of_the_same_model():
 
     want, want_k, want_v = run(model.forward)
     got, got_k, got_v = run(model.decode_step)
+    # prefill with the norm and SiLU steps as single launches: same logits as the PyTorch evaluation
+    pre = model.prefill(prompt, torch.arange(8, device="cuda")).float()
+    assert ((pre - want[0]).norm() / want[0].norm()).item() <= 3e-3 and torch.equal(pre.argmax(-1), want[0].argmax(-1))
     assert torch.isfinite(got).all()
     assert ((got - want).norm() / want.norm()).item() <= 3e-3
     assert torch.equal(got.argmax(-1), want.argmax(-1))
