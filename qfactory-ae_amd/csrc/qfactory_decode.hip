@@ -134,8 +134,9 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_kernel(const f16* __re
 // ---------------------------------------------------------------------------------------------
 // Attention of one query per (sequence, head) over cache positions 0 .. pos, one block of 16 or 4 waves per
 // (head, sequence).  LPK = hd/8 lanes share a key or value row (16 bytes each), so a block covers
-// 1024/LPK or 256/LPK positions per pass.  Scores -> LDS, block max and sum, then every group of LPK lanes walks its
-// share of the value rows; the groups of a wave are summed by lane shuffles, the waves through LDS.
+// 1024/LPK or 256/LPK positions per pass.  One pass over the cache: every group of LPK lanes walks its share of
+// the positions with a running maximum (key and value row requested together), the groups of a wave are merged
+// by lane shuffles, the waves through LDS.
 //
 // FUSED: q, k, v of the new position come straight from the QKV projection (row b = [3][H][hd]); q and k are
 // rotated here (pairs (2i, 2i+1), angles of table row pos, rounded to fp16 as a separate rotation kernel would
@@ -167,10 +168,7 @@ __global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __
     constexpr int HD = LPK * 8;
     constexpr int GROUPS = THREADS / LPK;
     constexpr int WAVES = THREADS / 64;
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    float* sc = smem;                                          // [max_len]
-    float* part = smem + max_len;                              // [WAVES][HD]
-    __shared__ float slots[WAVES];
+    __shared__ float part[WAVES * HD], part_m[WAVES], part_l[WAVES];
     __shared__ __attribute__((aligned(16))) f16 new_k[HD], new_v[HD];
     const int h = blockIdx.x, b = blockIdx.y;
     const int64_t pos = pos_ptr[0];
@@ -207,57 +205,59 @@ __global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __
 #pragma unroll
     for (int e = 0; e < 8; e++) qf[e] = (float)qv[e] * scale;
 
-    float local_max = -INFINITY;
-#pragma unroll 2
-    for (int p0 = 0; p0 < n; p0 += GROUPS) {
-        const int p = p0 + g;
-        float d = 0.f;
-        if (p < n) {
-            const f16x8 kv = (FUSED && p == (int)pos) ? *reinterpret_cast<const f16x8*>(new_k + j * 8)
-                                                      : *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
-#pragma unroll
-            for (int e = 0; e < 8; e++) d += qf[e] * (float)kv[e];
-        }
-#pragma unroll
-        for (int o = LPK / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
-        if (p < n) {
-            if (j == 0) sc[p] = d;
-            local_max = fmaxf(local_max, d);
-        }
-    }
-    const float mx = block_reduce<true, WAVES>(local_max, slots);      // also publishes sc[] to the block
-    float local_sum = 0.f;
-    for (int p = threadIdx.x; p < n; p += THREADS) {
-        const float e = __expf(sc[p] - mx);
-        sc[p] = e;
-        local_sum += e;
-    }
-    const float total = block_reduce<false, WAVES>(local_sum, slots);
-
+    // one pass over the cache with a running maximum: key and value row of a position are requested together
+    float m = -INFINITY, l = 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll 2
     for (int p = g; p < n; p += GROUPS) {
-        const float w = sc[p];
-        const f16x8 vv = (FUSED && p == (int)pos) ? *reinterpret_cast<const f16x8*>(new_v + j * 8)
-                                                  : *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
+        const bool fresh = FUSED && p == (int)pos;
+        const f16x8 kv = fresh ? *reinterpret_cast<const f16x8*>(new_k + j * 8) : *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
+        const f16x8 vv = fresh ? *reinterpret_cast<const f16x8*>(new_v + j * 8) : *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
+        float d = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] += w * (float)vv[e];
+        for (int e = 0; e < 8; e++) d += qf[e] * (float)kv[e];
+#pragma unroll
+        for (int o = LPK / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);      // stays inside the group: all its lanes are here
+        const float m_new = fmaxf(m, d);
+        const float keep = __expf(m - m_new), w = __expf(d - m_new);           // m = -inf the first time: keep = 0
+        l = l * keep + w;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = acc[e] * keep + w * (float)vv[e];
+        m = m_new;
     }
-    // the 64/LPK groups of a wave: lanes that differ in the bits above log2(LPK)
+    // merge the 64/LPK groups of a wave (lanes that differ in the bits above log2(LPK)) ...
 #pragma unroll
-    for (int o = LPK; o < 64; o <<= 1)
+    for (int o = LPK; o < 64; o <<= 1) {
+        const float m_o = __shfl_xor(m, o, 64), l_o = __shfl_xor(l, o, 64);
+        const float top = fmaxf(m, m_o);
+        const float a = (m == -INFINITY) ? 0.f : __expf(m - top), b = (m_o == -INFINITY) ? 0.f : __expf(m_o - top);
+        l = l * a + l_o * b;
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] += __shfl_xor(acc[e], o, 64);
+        for (int e = 0; e < 8; e++) acc[e] = acc[e] * a + __shfl_xor(acc[e], o, 64) * b;
+        m = top;
+    }
+    // ... and the waves through LDS
     if ((threadIdx.x & 63) < LPK) {
 #pragma unroll
         for (int e = 0; e < 8; e++) part[(threadIdx.x >> 6) * HD + j * 8 + e] = acc[e];
+        if (j == 0) {
+            part_m[threadIdx.x >> 6] = m;
+            part_l[threadIdx.x >> 6] = l;
+        }
     }
     __syncthreads();
     for (int d = threadIdx.x; d < HD; d += THREADS) {
-        float s = 0.f;
+        float top = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) s += part[w * HD + d];
-        out[head * HD + d] = (f16)(s / total);
+        for (int w = 0; w < WAVES; w++) top = fmaxf(top, part_m[w]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) {
+            const float f = (part_m[w] == -INFINITY) ? 0.f : __expf(part_m[w] - top);
+            num += part[w * HD + d] * f;
+            den += part_l[w] * f;
+        }
+        out[head * HD + d] = (f16)(num / den);
     }
 }
 
@@ -288,13 +288,11 @@ int launch_attention(const char* fn, const f16* q_or_qkv, f16* k, f16* v, const 
     constexpr int HD = LPK * 8;
     const float scale = 1.0f / sqrtf((float)HD);
     const bool many = (int64_t)batch * heads >= kAttnManyBlocks;
-    const size_t lds = ((size_t)max_len + (size_t)((many ? kAttnThreadsMany : kAttnThreadsFew) / 64) * HD) * sizeof(float);
-    if (lds > 60 * 1024) return fail(fn, "max_len too large for the score buffer in LDS");
     if (many)
-        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsMany>), dim3(heads, batch), dim3(kAttnThreadsMany), lds,
+        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsMany>), dim3(heads, batch), dim3(kAttnThreadsMany), 0,
                            stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
     else
-        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsFew>), dim3(heads, batch), dim3(kAttnThreadsFew), lds,
+        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsFew>), dim3(heads, batch), dim3(kAttnThreadsFew), 0,
                            stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
     return launched(fn);
 }
