@@ -63,6 +63,16 @@ def parity_cases():
     # chunks, group per lane / per chunk / over two chunks
     cases += [_case(3, 77, 4096, 3, 128), _case(12, 100, 2048, 3, 64), _case(16, 48, 8192, 3, 256, True),
               _case(9, 100, 1024, 3, 512), _case(16, 272, 4864, 3, 128), _case(32, 40, 1024, 3, 128)]
+    # K not a whole number of 128-byte windows of the main plane (GEMM kernel: the last window is moved back to
+    # end at the row's end and its first iterations are skipped): every width, a quarter / half / three quarters
+    # of a window left over, K split over wave groups and not, group per window position and wider
+    cases += [_case(300, 64, 2816, 2, 128, True), _case(40, 100, 2816, 2, 64), _case(64, 80, 11008, 2, 128, True),
+              _case(5, 100, 11008, 3, 128), _case(48, 64, 2816, 3, 64, True), _case(256, 12288, 2816, 3, 128),
+              _case(70, 96, 4224, 4, 32, True), _case(33, 130, 4224, 4, 64), _case(64, 64, 1088, 4, 32, True),
+              _case(64, 64, 1216, 4, 32), _case(512, 4096, 4224, 4, 64),
+              _case(40, 72, 4160, 8, 32), _case(40, 40, 4160, 8, 32, True), _case(128, 8192, 4160, 8, 32)]
+    # eight groups per 128-byte window (4 bits, group 32) on whole windows
+    cases += [_case(70, 96, 4096, 4, 32, True), _case(40, 64, 1024, 4, 32)]
     return cases
 
 

@@ -39,8 +39,11 @@ def regime_for(M, K=None, nbits=None, group_size=None):
         if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
             return "mgemv"
         return "gemm" if gemm_supported(K, nbits, group_size) else "gemv"
-    if K is None or not mfma_supported(K, nbits, group_size):
+    if K is None:
         return "gemv"
+    if not mfma_supported(K, nbits, group_size):
+        # K is not a whole number of 16-byte lane loads: only the GEMM (64-element iterations) and the dot2 GEMV remain
+        return "gemm" if M > GEMV_MAX_M and gemm_supported(K, nbits, group_size) else "gemv"
     if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
         return "mgemv"
     if skinny_preferred(M, K, nbits, group_size):
@@ -199,9 +202,20 @@ def mfma_tiling(M, N, K, nbits, group_size, **pins):
         wn //= 2
     if (N // (wn * bt * 16)) < NUM_CUS and bt > 1:
         bt = 1
+    # the double-buffered activation tile (BM x 4*128/nbits elements) must fit LDS: fewer rows per block at 2 bits
+    while mfma_lds_bytes(at, bt, wm, wn, wk, nbits) > 160 * 1024 and at > 1:
+        at //= 2
+    while mfma_lds_bytes(at, bt, wm, wn, wk, nbits) > 160 * 1024 and wm > 1:
+        wm //= 2
     cfg = {"AT": at, "BT": bt, "WM": wm, "WN": wn, "WK": wk}
     cfg.update(pins)
     return cfg
+
+
+def mfma_lds_bytes(at, bt, wm, wn, wk, nbits):
+    """LDS of qf::mfma_kernel: two activation tiles per K-slice plus the partial tiles of a K split."""
+    bk = 4 * (128 // nbits)
+    return 2 * wk * (at * wm * 16) * (bk + 8) * 2 + ((wk - 1) * wm * wn * at * bt * 1024 if wk > 1 else 0)
 
 
 def mfma_candidates(M, N, K, nbits, group_size):
@@ -213,6 +227,8 @@ def mfma_candidates(M, N, K, nbits, group_size):
         key = tuple(sorted(cfg.items()))
         threads = 64 * cfg["WM"] * cfg["WN"] * cfg["WK"]
         if key in seen or threads > 1024 or cfg["WK"] > iters or cfg["AT"] * cfg["BT"] > 32:
+            return
+        if mfma_lds_bytes(cfg["AT"], cfg["BT"], cfg["WM"], cfg["WN"], cfg["WK"], nbits) > 160 * 1024:
             return
         seen.add(key)
         out.append(cfg)
@@ -499,15 +515,19 @@ def gemm_valid(cfg, K, nbits, group_size):
     bm, nt32, wn, wk, pa = (cfg[k] for k in ("BM", "NT32", "WN", "WK", "PA"))
     if bm <= 0 or bm % 32 or min(nt32, wn, wk) < 1 or 64 * wn * wk > 1024:
         return False
-    if K % supk or K % group_size or group_size % 32:
+    # K: whole 64-element iterations and at least one 128-byte window of the main plane; a partial last
+    # window must be whole 16-byte units in every plane
+    if K % 64 or K < supk or ((K % supk) * pb // 8) % (32 if nbits == 3 else 16):
+        return False
+    if K % group_size or group_size % 32:
         return False
     if (group_size < supk and supk % group_size) or (group_size > supk and group_size % supk):
         return False
     ngs = max(1, supk // group_size)
     if ngs > 8 or ngs * zfb > 32:
         return False
-    if (K // group_size) % (8 // zfb):
-        return False
+    # (asymmetric weights also need K/GS to fill whole zero-point bytes: a property of the packed tensors,
+    # checked where they are built and again by the launcher, not a tiling matter -- symmetric ones do not)
     if (bm * 8) % (64 * wn) or not 3 <= pa <= 12:
         return False
     if (bm // 32) * nt32 * 16 > 256:
@@ -561,7 +581,7 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
         # 8192 x 8192 and 172 against 183 us on 8192 x 28672 at M = 256 (slower than four 64 x 32
         # waves when blocks come in several rounds and there is only one group)
         wn, nt32 = 2, 2
-    nsup = K // (1024 // plane_bits(nbits))
+    nsup = -(-K // (1024 // plane_bits(nbits)))
     wk = max(1, min(wk, nsup))
     pa = 4
     while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):

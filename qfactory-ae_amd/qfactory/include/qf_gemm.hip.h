@@ -71,7 +71,14 @@ struct GemmCfg {
     static constexpr bool HI = NBITS == 3;
     static constexpr int SUPK = 1024 / PB;                     // elements of K in 128 bytes of the main plane
     static constexpr int SUP = SUPK / BK;                      // K-iterations per super
-    static constexpr int NSUP = K / SUPK;
+    // K need not be a whole number of supers: the last one may hold only TAIL_IT of its SUP iterations.  Its
+    // 128-byte window (and those of the 1-bit plane, the scales and the zero-points) is then moved back to end
+    // at the end of the row -- every load stays inside the row -- and iteration q of it reads position
+    // q + TAIL_SHIFT of the window; the iterations past K are skipped.
+    static constexpr int NSUP = (K + SUPK - 1) / SUPK;
+    static constexpr int TAIL_IT = (K % SUPK) / BK;            // 0: K is a whole number of supers
+    static constexpr bool TAIL = TAIL_IT != 0;
+    static constexpr int TAIL_SHIFT = TAIL ? SUP - TAIL_IT : 0;
     static constexpr int SUP_PER_GROUP = (NSUP + WK - 1) / WK;
     static constexpr int ITERS = SUP_PER_GROUP * SUP;          // K-iterations of every group
     static constexpr int UPS = TN * 8 / 64;                    // 16-byte units per lane and super
@@ -195,8 +202,11 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     // past the last super re-reads the last one and drops the products
     auto k_of = [&](int it) {
         const int sup = min((it / SUP) * WK + grp, C::NSUP - 1);
-        return sup * C::SUPK + (it % SUP) * BK;
+        const int k = sup * C::SUPK + (it % SUP) * BK;
+        return C::TAIL ? min(k, C::K - BK) : k;                 // skipped iterations of a partial last super re-read the last tile
     };
+    // does local super P of this group map to the partial last super (groups past the end re-read it)?
+    auto is_tail = [&](int sup_local) { return C::TAIL && sup_local * WK + grp >= C::NSUP - 1; };
 
     // ---- activations: UA 16-byte units per lane and iteration, global memory -> LDS ----
     // Instruction p of wave wn fills the 1 KB of 16-byte slots (p*WN + wn)*64 .. +63 of the tile
@@ -250,14 +260,18 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     auto load_super = [&](WStage& st, int sup_local) {
         if (QF_GEMM_EXPERIMENT & 32) return;
         const int sup = min(sup_local * WK + grp, C::NSUP - 1);
-        const uint8_t* wb = w_rows + (size_t)sup * 128;
+        // byte offset of the super's window in the main plane (half of it in the 1-bit plane); wave-uniform, and
+        // opaque: requests past the end clamp to the same window and must not be merged (see the end of the K loop)
+        uint32_t woff = __builtin_amdgcn_readfirstlane(is_tail(sup_local) ? (uint32_t)(C::K * C::PB / 8 - 128) : (uint32_t)sup * 128u);
+        asm volatile("" : "+s"(woff));
+        const uint8_t* wb = w_rows + woff;
 #pragma unroll
         for (int p = 0; p < UPS; p++) {
             const uint8_t* src = wb + w_off[p];
             st.w[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
         }
         if constexpr (C::HI) {
-            const uint8_t* hb = w_rows + (size_t)sup * 64;
+            const uint8_t* hb = w_rows + woff / 2;
 #pragma unroll
             for (int p = 0; p < C::UPH; p++) {
                 const uint8_t* src = hb + h_off[p];
@@ -268,7 +282,9 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     auto load_quant = [&](Quant& qu, int sup_local) {
         if (QF_GEMM_EXPERIMENT & 32) return;
         const int sup = min(sup_local * WK + grp, C::NSUP - 1);
-        const int g0 = sup * C::SUPK / C::GS;                  // first group of the super
+        // first group of the super's window (a partial last super: the window ends at the last group); opaque, as in load_super
+        int g0 = __builtin_amdgcn_readfirstlane(is_tail(sup_local) ? (C::K - C::SUPK) / C::GS : sup * C::SUPK / C::GS);
+        asm volatile("" : "+s"(g0));
         const uint8_t* sb = s_rows + (size_t)g0 * 2;
         const uint8_t* zb = z_rows + (g0 * C::ZFB) / 8;
 #pragma unroll
@@ -330,8 +346,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     };
     // dequantisation constants of tile j in iteration q of the current super; the group of this
     // lane's 32 fields is a compile-time index unless a group is only 32 wide
-    auto qconst_of = [&](const Quant& qu, int j, int q) {
-        uint32_t sbits, zero;
+    auto qconst_raw = [&](const Quant& qu, int j, int q, uint32_t& sbits, uint32_t& zero) {
         if constexpr (C::GS >= C::SUPK) {
             sbits = qu.s[j][0] & 0xFFFFu;
             zero = qu.z[j] & ZMASK;
@@ -344,6 +359,18 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             zero = (qu.z[j] >> ((2 * q + kb) * C::ZFB)) & ZMASK;
         }
         if constexpr (C::SYM) zero = 1u << (C::NBITS - 1);
+    };
+    // q is a compile-time constant at every call site; in a partial last super (`tail`, wave-uniform) the
+    // window position is q + TAIL_SHIFT: both candidates are extracted and one is selected
+    auto qconst_of = [&](const Quant& qu, int j, int q, bool tail) {
+        uint32_t sbits, zero;
+        qconst_raw(qu, j, q, sbits, zero);
+        if constexpr (C::TAIL) {
+            uint32_t sbits_t, zero_t;
+            qconst_raw(qu, j, min(q + C::TAIL_SHIFT, SUP - 1), sbits_t, zero_t);
+            sbits = tail ? sbits_t : sbits;
+            zero = tail ? zero_t : zero;
+        }
         return make_qconst<C::NBITS>((uint16_t)sbits, zero);
     };
 
@@ -397,8 +424,13 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         // every read of the current super has been issued one iteration ago: the next super
         // (loaded two supers back) takes its place in LDS
         if (q == SUP - 1) store_super(ringW[pslot ^ 1]);
-        read_packed(nxt, (q + 1) % SUP);
-        const bool live = WK == 1 || (P * WK + grp < C::NSUP);
+        const bool tail = is_tail(P);
+        {
+            const int qn = (q + 1) % SUP;                       // the next iteration and the super it belongs to
+            const bool tail_n = is_tail(q == SUP - 1 ? P + 1 : P);
+            read_packed(nxt, C::TAIL && tail_n ? min(qn + C::TAIL_SHIFT, SUP - 1) : qn);
+        }
+        const bool live = (WK == 1 || (P * WK + grp < C::NSUP)) && !(C::TAIL && tail && q >= C::TAIL_IT);
         if (live) {
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
@@ -411,7 +443,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 }
 #pragma unroll
                 for (int j = 0; j < NT32; j++) {
-                    const QConst qc = qconst_of(ringQ[pslot], j, q);
+                    const QConst qc = qconst_of(ringQ[pslot], j, q, tail);
                     if constexpr ((QF_GEMM_EXPERIMENT & 1) != 0) {
                         wf[j] = __builtin_bit_cast(f16x8, u32x4{cur.w[j][0], cur.w[j][1], cur.w[j][2], cur.w[j][3] + (uint32_t)ks});
                     } else if constexpr (C::NBITS == 3) {
@@ -462,7 +494,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     for (int p = 0; p < (C::PREFETCH_A ? C::PA : C::PA - 1); p++) load_a(p, min(p, C::ITERS - 1));
     store_super(ringW[0]);
     load_super(ringW[0], 2);
-    read_packed(cur, 0);
+    read_packed(cur, is_tail(0) ? C::TAIL_SHIFT : 0);
     wait_loads_and_barrier<0>();
     if constexpr (C::PREFETCH_A) read_frags(fcur, 0);
 
@@ -478,6 +510,28 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 b2 = b2 == C::NBUF - 1 ? 0 : b2 + 1;
             }
         });
+    }
+    // The wait counts above assume that every iteration really issues the loads `loads_since` counts.  What
+    // the last iterations load for supers past the end is never used, and a compiler that can see that (a
+    // K loop of a single trip) drops those loads or merges them (they all clamp to the last super): fewer
+    // loads in flight than counted, and the wait lets an activation tile that is about to be read stay in
+    // flight.  The super index is opaque to the compiler where the loads are issued, and naming the ring
+    // registers here keeps every load alive, at no cost (no instruction is emitted; the drain below waits
+    // for them anyway).
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+#pragma unroll
+        for (int p = 0; p < UPS; p++) asm volatile("" ::"v"(ringW[r].w[p]));
+        if constexpr (C::HI) {
+#pragma unroll
+            for (int p = 0; p < C::UPH; p++) asm volatile("" ::"v"(ringW[r].h[p]));
+        }
+#pragma unroll
+        for (int j = 0; j < NT32; j++) {
+#pragma unroll
+            for (int i = 0; i < SREGS; i++) asm volatile("" ::"v"(ringQ[r].s[j][i]));
+            asm volatile("" ::"v"(ringQ[r].z[j]));
+        }
     }
     // the repeated activation requests of the last iterations still target LDS: drain them before
     // the space is reused below or the wave ends
@@ -543,7 +597,8 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8";
     else if (C::BM % 32 != 0 || C::BM <= 0 || C::NT32 < 1 || C::WN < 1 || C::WK < 1) why = "BM must be a multiple of 32; NT32, WN, WK positive";
     else if (C::T > 1024) why = "block too large";
-    else if (C::K % C::SUPK != 0 || C::NSUP < 1) why = "K must be a multiple of 128 packed bytes of the main plane";
+    else if (C::K % C::BK != 0 || C::K < C::SUPK) why = "K must be a multiple of 64 and hold at least 128 packed bytes of the main plane";
+    else if ((C::K % C::SUPK) * C::PB / 8 % (C::HI ? 32 : 16) != 0) why = "a partial last 128-byte window must be whole 16-byte units in every plane";
     else if (C::GS <= 0 || C::K % C::GS != 0) why = "GS must divide K";
     else if (C::GS % 32 != 0) why = "a lane's 32 fields must lie inside one group (GS multiple of 32)";
     else if (C::GS < C::SUPK && C::SUPK % C::GS != 0) why = "GS must divide 1024/NBITS or be a multiple of it";

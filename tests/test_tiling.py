@@ -62,6 +62,9 @@ def test_default_tiling_respects_the_kernel_limits(case):
         assert t["VB"] in (4, 8, 16) and 64 * t["WK"] * t["WN"] <= 1024
     else:
         assert regime == "mfma"
+        t = tiling.mfma_tiling(M, N, K, nbits, gs)
+        assert tiling.mfma_lds_bytes(t["AT"], t["BT"], t["WM"], t["WN"], t["WK"], nbits) <= 160 * 1024
+        assert 64 * t["WM"] * t["WN"] * t["WK"] <= 1024
 
 
 def test_two_bit_k4096_mgemv_fits_lds():
