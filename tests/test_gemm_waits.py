@@ -29,7 +29,7 @@ def _isa_of(qfunc, tmp_path):
 
 @pytest.mark.parametrize("M,N,K,nbits,gs", [(70, 96, 4096, 4, 32), (70, 96, 4224, 4, 32), (64, 80, 2816, 2, 128), (48, 64, 2816, 3, 64),
                                            (256, 57344, 8192, 4, 128), (64, 22016, 4096, 4, 128), (128, 8192, 28672, 4, 128),
-                                           (33, 100, 512, 4, 128), (300, 256, 2048, 4, 128), (40, 96, 512, 8, 32)])
+                                           (33, 100, 512, 4, 128), (300, 256, 2048, 4, 128), (40, 96, 2048, 8, 32)])
 def test_every_counted_load_is_issued(M, N, K, nbits, gs, tmp_path):
     from qfactory.core.qfunc import QMatmulQFunc
     from qfactory.core.qtile import QTile, SymQTile
