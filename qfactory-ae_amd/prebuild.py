@@ -76,6 +76,24 @@ def parity_cases():
     return cases
 
 
+def grid_cases():
+    """Every bit width x group size the packed layout allows, symmetric and asymmetric alternating, at one
+    small shape per kernel family (M = 1 dot2 GEMV, M = 12 small-M matrix-core kernels, M = 40 GEMM), with K a
+    whole number of 128-byte windows and with half a window left over where the group size permits."""
+    cases = []
+    for nbits in (2, 3, 4, 8):
+        zfb = 4 if nbits == 3 else nbits
+        supk = 1024 // (2 if nbits == 3 else nbits)
+        for i, gs in enumerate((32, 64, 128, 256, 512, 1024)):
+            for K in (4096, 4096 + supk // 2):
+                G = K // gs
+                if K % (2 * gs) or G % (8 // zfb):
+                    continue
+                sym = bool(i % 2)
+                cases += [_case(1, 50, K, nbits, gs, sym), _case(12, 72, K, nbits, gs, not sym), _case(40, 72, K, nbits, gs, sym)]
+    return cases
+
+
 def large_parity_cases():
     """W4A16 g128 GEMM at M in {32..256} on Llama-3-70B-style shapes.  The weights are too large to
     build from int32 tensors in a test; the tests fill packed tensors directly (every byte pattern
@@ -118,7 +136,7 @@ def search_cases():
 
 def all_cases():
     seen, out = set(), []
-    for c in (parity_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
+    for c in (parity_cases() + grid_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
               + decode_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:

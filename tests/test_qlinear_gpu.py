@@ -26,7 +26,17 @@ def qf():
     return QLinear
 
 
-@pytest.mark.parametrize("case", prebuild.parity_cases(), ids=_id)
+def _unique(cases):
+    seen, out = set(), []
+    for c in cases:
+        key = tuple(sorted(c.items()))
+        if key not in seen:
+            seen.add(key)
+            out.append(c)
+    return out
+
+
+@pytest.mark.parametrize("case", _unique(prebuild.parity_cases() + prebuild.grid_cases()), ids=_id)
 def test_qlinear_matches_oracle(qf, oracle, case):
     M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
     print(f"[case] {_id(case)}", flush=True)
