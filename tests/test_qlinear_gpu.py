@@ -72,20 +72,21 @@ def test_large_gemm_matches_oracle_on_sampled_columns(qf, oracle, case):
     """Llama-3-70B-style shapes at M = 32..256: packed tensors are filled directly with seeded
     random bytes (any byte pattern is a valid packed weight / zero tensor); 1024 seeded output
     columns are checked against the oracle -- every output column is an independent dot product."""
-    M, N, K, nbits, GS = (case[k] for k in ("M", "N", "K", "NBITS", "GS"))
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
     print(f"[case] {_id(case)}", flush=True)
     g = torch.Generator(device="cuda").manual_seed(N + K + M)
-    layer = qf.empty(M, K, N, nbits, GS, sym=False, compile_flags=NO_SEARCH)
+    layer = qf.empty(M, K, N, nbits, GS, sym=sym, compile_flags=NO_SEARCH)
     layer.w.copy_(torch.randint(-128, 128, layer.w.shape, dtype=torch.int8, device="cuda", generator=g))
     layer.s.copy_((torch.rand(layer.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
-    layer.z.copy_(torch.randint(-128, 128, layer.z.shape, dtype=torch.int8, device="cuda", generator=g))
+    if not sym:
+        layer.z.copy_(torch.randint(-128, 128, layer.z.shape, dtype=torch.int8, device="cuda", generator=g))
     A = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
     out = layer(A)
     torch.cuda.synchronize()
     rows = np.sort(np.random.default_rng(N + M).choice(N, size=1024, replace=False))
     rows_t = torch.from_numpy(rows).cuda()
     ref = oracle.qlinear_np(A.cpu().numpy(), layer.w[rows_t].cpu().numpy(), layer.s[rows_t].cpu().numpy(),
-                            layer.z[rows_t].cpu().numpy(), nbits, GS)
+                            None if sym else layer.z[rows_t].cpu().numpy(), nbits, GS)
     assert_close(oracle, out[:, rows_t].cpu().numpy(), ref, _id(case))
 
 
