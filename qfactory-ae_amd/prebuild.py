@@ -94,6 +94,29 @@ def grid_cases():
     return cases
 
 
+# The reference's shape list (data/nkg_shapes.json, key "all"): [N, K, group size] of the linears of Llama-2
+# 7B / 13B / 70B and Qwen-2.5 7B / 14B / 32B / 72B.  Its accuracy scripts sweep it at M in {1, 16} and 8 / 4 / 2 bits.
+REFERENCE_SHAPES = [[3584, 3584, 128], [4608, 3584, 128], [4096, 4096, 128], [5120, 5120, 128], [7168, 5120, 128],
+                    [4096, 11008, 128], [12288, 4096, 128], [8192, 8192, 128], [3584, 18944, 128], [5120, 13824, 128],
+                    [15360, 5120, 128], [10240, 8192, 128], [22016, 4096, 128], [37888, 3584, 128], [27648, 5120, 128],
+                    [5120, 27648, 128], [8192, 29696, 128], [55296, 5120, 128], [59392, 8192, 128], [57344, 8192, 128],
+                    [8192, 28672, 128]]
+
+
+def reference_sweep_cases():
+    """tests/acc_gptq.py (grouped, asymmetric) and tests/acc_gemv.py (plain integer weights) of the reference:
+    every shape x M in {1, 16} x bits in {8, 4, 2}; the grouped sweep skips K % (GS * 8 / bits) != 0 as the
+    reference does (acc_gptq.py:42-44)."""
+    cases = []
+    for N, K, GS in REFERENCE_SHAPES:
+        for M in (1, 16):
+            for nbits in (8, 4, 2):
+                if K % (GS * 8 // nbits) == 0:
+                    cases.append(_case(M, N, K, nbits, GS))
+                cases.append(_case(M, N, K, nbits, -1))
+    return cases
+
+
 def large_parity_cases():
     """W4A16 g128 GEMM at M in {32..256} on Llama-3-70B-style shapes.  The weights are too large to
     build from int32 tensors in a test; the tests fill packed tensors directly (every byte pattern
@@ -139,7 +162,7 @@ def search_cases():
 
 def all_cases():
     seen, out = set(), []
-    for c in (parity_cases() + grid_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
+    for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
               + decode_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
