@@ -88,7 +88,9 @@ def _pow2_floor(x):
 
 
 def gemv_wave_split(K, nbits, vb, mt, max_waves=8, a_reg_budget=128):
-    """(WK, IT) choices ranked by idle-lane waste, then by fewer chunks per lane (more waves)."""
+    """(WK, IT) choices ranked by idle-lane waste in steps of an eighth, then by fewer chunks per lane (more
+    waves): up to ~12 % of idle lanes cost less than a third pass over the row (8192 x 29696: eight waves x
+    two chunks, 10 % idle, 25.0 us against 34.4 us for five waves x three chunks, 3 % idle)."""
     epc = elements_per_chunk(nbits, vb)
     nch = K // epc
     a_regs_per_chunk = epc // 2
@@ -98,12 +100,12 @@ def gemv_wave_split(K, nbits, vb, mt, max_waves=8, a_reg_budget=128):
         if it * a_regs_per_chunk * mt > a_reg_budget:
             continue
         waste = (64 * wk * it - nch) / nch
-        out.append((round(waste, 3), it, wk, it))
+        out.append((int(waste * 8), it, round(waste, 3), wk, it))
     if not out:
         wk = max_waves
-        out.append((0.0, 0, wk, -(-nch // (64 * wk))))
+        out.append((0, 0, 0.0, wk, -(-nch // (64 * wk))))
     out.sort()
-    return [(wk, it) for _, _, wk, it in out]
+    return [(wk, it) for _, _, _, wk, it in out]
 
 
 def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None, mt=None):
@@ -131,7 +133,7 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
         u = max(1, min(in_flight // it if it <= in_flight else 1, 64 // mt, in_flight))
         u = _pow2_floor(u)
     if wn is None:
-        wn = 1 if big else (2 if wk * 2 <= 16 else 1)
+        wn = 1 if big else (2 if wk * 2 <= 12 else 1)         # 5120 x 13824, seven waves per team: one team 9.2 us, two 10.2
     if steps is None:
         steps = 2 if (big and it >= 2) else 1
         # several activation rows per block: 69 registers instead of 28 leave room for fewer resident
