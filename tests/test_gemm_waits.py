@@ -38,22 +38,19 @@ def test_every_counted_load_is_issued(M, N, K, nbits, gs, tmp_path):
     pa = q.tiling_configs["PA"]
     isa = _isa_of(q, tmp_path)
     loads_in_segment, segments, checked = 0, [], 0
-    pending_wait = None
     for line in isa.splitlines():
         line = line.strip()
         if line.startswith(("global_load", "buffer_load")):
             loads_in_segment += 1
-            pending_wait = None
         m = re.match(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)", line)
-        if m:
-            pending_wait = int(m.group(1))
-        if line.startswith("s_barrier"):
+        if m:                                        # the kernel's explicit wait (with or without a block barrier behind it)
+            allowed = int(m.group(1))
             segments.append(loads_in_segment)
-            if pending_wait == 0:
+            loads_in_segment = 0
+            if allowed == 0:
                 segments = []                        # a full drain (end of the prologue): nothing older is in flight
-            elif pending_wait is not None and len(segments) >= pa - 2:
+            elif len(segments) >= pa - 2:
                 # the loads of the last PA - 2 iterations may stay in flight: they must all exist
-                assert sum(segments[-(pa - 2):]) == pending_wait, (segments, pending_wait)
+                assert sum(segments[-(pa - 2):]) == allowed, (segments, allowed)
                 checked += 1
-            loads_in_segment, pending_wait = 0, None
     assert checked >= 2
