@@ -78,7 +78,7 @@ class QMatmulQFunc(QFunc):
         gs = qtile_b.quant_granularity[1]
 
         # Template-based code generation: which kernel family and how it is tiled
-        self.regime = tiling.regime_for(m, k, qtile_b.nbits, gs)
+        self.regime = tiling.regime_for(m, k, qtile_b.nbits, gs, n)
         self.parallel_strategy = "row"          # teams sweep rows, K split over lanes and waves
         self.tiling_configs = self.default_tiling(self.regime)
         # Computation transformation: "deferred" applies scale and zero once per chunk / group in

@@ -31,7 +31,7 @@ MGEMV_MIN_M = 3         # below: dot2 GEMV; [MGEMV_MIN_M, MGEMV_MAX_M]: A-statio
 MGEMV_MAX_M = 32
 
 
-def regime_for(M, K=None, nbits=None, group_size=None):
+def regime_for(M, K=None, nbits=None, group_size=None, N=None):
     if M < MGEMV_MIN_M or not MFMA_AVAILABLE:
         return "gemv"
     if K is not None and nbits == 3:
@@ -46,7 +46,7 @@ def regime_for(M, K=None, nbits=None, group_size=None):
         return "gemm" if M > GEMV_MAX_M and gemm_supported(K, nbits, group_size) else "gemv"
     if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
         return "mgemv"
-    if skinny_preferred(M, K, nbits, group_size):
+    if skinny_preferred(M, K, nbits, group_size, N):
         return "skinny"
     if M <= GEMV_MAX_M:
         return "gemv"
@@ -375,14 +375,18 @@ SKINNY_MAX_M = 16
 SKINNY_MAX_K = 16384
 
 
-def skinny_preferred(M, K, nbits, group_size):
+def skinny_preferred(M, K, nbits, group_size, N=None):
     """The streaming kernel takes the rows-of-16 problems whose activations the A-stationary kernel
     cannot keep in registers (K = 11008 or 14336 at 4 bits, K = 8192 or 11008 at 8 bits).  Measured at
     M = 4 .. 16 on 4096 x 11008: 10.7 .. 13.2 us against 13.9 .. 21.7 us for the kernels that served it
     before (8-bit: 17.4 against 28.6).  Every block streams all of the activations, M x K x 2 bytes:
     at K = 28672 that is twice the block's weight bytes and the GEMM kernel wins (49 against 109 us),
-    as it does above 16 rows."""
-    if not (MGEMV_MIN_M <= M <= SKINNY_MAX_M) or K > SKINNY_MAX_K:
+    as it does above 16 rows.  Between 16384 and 20480 it still wins where every block has a single tile of
+    16 columns while 32-column GEMM tiles would leave half of the CUs idle (3584 x 18944 at 4 bits: 20.6
+    against 32.0 us)."""
+    if not (MGEMV_MIN_M <= M <= SKINNY_MAX_M):
+        return False
+    if K > SKINNY_MAX_K and not (nbits == 4 and K <= 20480 and N is not None and 0 < N <= 16 * NUM_CUS):
         return False
     return skinny_tiling(M, 16 * NUM_CUS, K, nbits, group_size) is not None
 

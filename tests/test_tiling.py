@@ -35,7 +35,7 @@ def test_regime_routing(M, K, nbits, gs, expected):
 @pytest.mark.parametrize("case", _cases(), ids=_id)
 def test_default_tiling_respects_the_kernel_limits(case):
     M, N, K, nbits, gs = (case[k] for k in ("M", "N", "K", "NBITS", "GS"))
-    regime = tiling.regime_for(M, K, nbits, gs)
+    regime = tiling.regime_for(M, K, nbits, gs, N)
     if regime == "mgemv":
         t = tiling.mgemv_tiling(M, N, K, nbits, gs)
         chunk = 4 * (128 // tiling.plane_bits(nbits))
@@ -65,6 +65,12 @@ def test_default_tiling_respects_the_kernel_limits(case):
         t = tiling.mfma_tiling(M, N, K, nbits, gs)
         assert tiling.mfma_lds_bytes(t["AT"], t["BT"], t["WM"], t["WN"], t["WK"], nbits) <= 160 * 1024
         assert 64 * t["WM"] * t["WN"] * t["WK"] <= 1024
+
+
+def test_skinny_takes_longer_rows_only_with_one_tile_per_block():
+    assert tiling.regime_for(16, 18944, 4, 128, 3584) == "skinny"       # 224 tiles of 16 columns: one per block
+    assert tiling.regime_for(16, 18944, 4, 128, 8192) == "gemm"
+    assert tiling.regime_for(16, 27648, 4, 128, 3584) == "gemm"
 
 
 def test_two_bit_k4096_mgemv_fits_lds():
