@@ -181,7 +181,8 @@ def qlinear_np(A, w, s, z, nbits, GS):
 def gemv_plain_np(A, w, nbits):
     K = A.shape[1]
     q = unpack_weight(w, K, nbits)
-    return (np.asarray(A, dtype=np.float16).astype(np.float64) @ q.astype(np.float64).T).astype(np.float16)
+    with np.errstate(over="ignore"):     # sums past the fp16 range round to infinity, as the fp16 output of the kernel does
+        return (np.asarray(A, dtype=np.float16).astype(np.float64) @ q.astype(np.float64).T).astype(np.float16)
 
 
 # ----------------------------------------------------------------------------------------------
