@@ -37,7 +37,8 @@
 #include "qf_dequant.hip.h"
 
 // Timing experiments (results are wrong when non-zero): bit 0 skips the dequantisation arithmetic,
-// bit 1 the activation fragment reads, bit 2 the MFMAs, bit 5 the global weight / scale / zero loads.
+// bit 1 the activation fragment reads, bit 2 the MFMAs, bit 3 the activation tile requests, bit 4 the block
+// barrier of the K loop, bit 5 the global weight / scale / zero loads.
 #ifndef QF_GEMM_EXPERIMENT
 #define QF_GEMM_EXPERIMENT 0
 #endif
@@ -132,11 +133,11 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
 // Wait until at most ALLOWED of this wave's vector-memory loads (in issue order) and none of its
 // LDS operations are outstanding, then meet the block's other waves.  A bare s_barrier: the
 // fence of __syncthreads() would wait for every outstanding load.
-template <int ALLOWED>
+template <int ALLOWED, bool BARRIER = true>
 __device__ __forceinline__ void wait_loads_and_barrier() {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(ALLOWED, 0));
-    __builtin_amdgcn_s_barrier();
+    if constexpr (BARRIER) __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 }
 
@@ -225,6 +226,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     const uint8_t* a_slab = reinterpret_cast<const uint8_t*>(A + (size_t)m_blk * C::K);
     // tile `it` of the group into LDS buffer `buf`, asynchronously
     auto load_a = [&](int buf, int it) {
+        if (QF_GEMM_EXPERIMENT & 8) return;
         const uint8_t* base = a_slab + (size_t)k_of(it) * 2;
         uint8_t* dst = as_b + (size_t)buf * BM * C::ROWB + (size_t)wn * 1024;
 #pragma unroll
@@ -482,7 +484,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         // wave has issued in those iterations (activation tiles and whole supers) may stay in
         // flight.  Loads return in order; what the requesting iteration itself issued next to the
         // request is not counted, wherever the compiler placed it.
-        wait_loads_and_barrier<loads_since<C>(s, C::PA - 2)>();
+        wait_loads_and_barrier<(QF_GEMM_EXPERIMENT & 8) ? 63 : loads_since<C>(s, C::PA - 2), !(QF_GEMM_EXPERIMENT & 16)>();
     };
 
     // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----
