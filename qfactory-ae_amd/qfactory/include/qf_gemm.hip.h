@@ -38,7 +38,7 @@
 
 // Timing experiments (results are wrong when non-zero): bit 0 skips the dequantisation arithmetic,
 // bit 1 the activation fragment reads, bit 2 the MFMAs, bit 3 the activation tile requests, bit 4 the block
-// barrier of the K loop, bit 5 the global weight / scale / zero loads.
+// barrier of the K loop, bit 5 the global weight / scale / zero loads, bit 6 the wait for the activation tiles.
 #ifndef QF_GEMM_EXPERIMENT
 #define QF_GEMM_EXPERIMENT 0
 #endif
@@ -484,7 +484,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         // wave has issued in those iterations (activation tiles and whole supers) may stay in
         // flight.  Loads return in order; what the requesting iteration itself issued next to the
         // request is not counted, wherever the compiler placed it.
-        wait_loads_and_barrier<(QF_GEMM_EXPERIMENT & 8) ? 63 : loads_since<C>(s, C::PA - 2), !(QF_GEMM_EXPERIMENT & 16)>();
+        wait_loads_and_barrier<(QF_GEMM_EXPERIMENT & (8 | 64)) ? 63 : loads_since<C>(s, C::PA - 2), !(QF_GEMM_EXPERIMENT & 16)>();
     };
 
     // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----
