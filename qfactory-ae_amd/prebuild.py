@@ -122,7 +122,7 @@ def large_parity_cases():
     build from int32 tensors in a test; the tests fill packed tensors directly (every byte pattern
     is a valid packed weight) and check a seeded subset of output columns."""
     return ([_case(M, N, K) for N, K in LLAMA3_70B for M in (32, 64, 128, 256)]
-            + [_case(512, 10240, 8192), _case(1024, 12288, 4096), _case(700, 22016, 4096)]
+            + [_case(512, 10240, 8192), _case(1024, 12288, 4096), _case(700, 22016, 4096), _case(512, 22016, 4096), _case(1024, 10240, 8192)]
             # the large block tiles at the other bit widths, group sizes and with a partial last window
             + [_case(256, 16384, 4096, 2, 64), _case(256, 16384, 4096, 3, 128, True), _case(256, 16384, 4096, 8, 32),
                _case(512, 16384, 4224, 4, 64), _case(256, 57344, 2816, 2, 128, True), _case(1024, 16384, 4096, 3, 128, True)])

@@ -607,8 +607,10 @@ def _gemm_tiling_many_rows(M, N, K, nbits, group_size):
     M = 512 .. 2048 on eight Llama shapes: a tile costs its area plus an overhead worth 6300 outputs
     (per round at K = 8192: 48 us for 64 x 128, 85 for 128 x 128, 140 for 128 x 256, 250 for 256 x 256);
     rounds overlap, so a launch costs its exact number of rounds plus 60 % of the rounding-up, and a
-    single partial round runs a little faster than a full one.  Picks within 4 % of the best of the
-    sweep on 22 of 24 cells (before: 17; worst case 1.35x -> 1.16x).  None when the launch is a
+    single partial round runs faster than a full one (0.6 + 0.4 x the fraction of CUs with a block;
+    with 0.75 + 0.25 the model kept 128 x 128 tiles in 2.5 rounds on 10240 x 8192 at M = 1024, 294 us,
+    where 160 tiles of 256 x 256 take 224 us, and on 22016 x 4096 at M = 512, 146 against 123 us).
+    Picks within 4 % of the best of the sweep on 22 of 24 cells (before: 17; worst case 1.35x -> 1.16x).  None when the launch is a
     single round: the small-M model, which splits K over wave groups, serves those."""
     best = None
     for bm, nt32, wn in ((256, 1, 8), (128, 2, 4), (128, 1, 4), (64, 1, 4)):
@@ -617,7 +619,7 @@ def _gemm_tiling_many_rows(M, N, K, nbits, group_size):
             continue
         bn = 32 * wn * nt32
         exact = (-(-N // bn) * -(-M // bm)) / NUM_CUS
-        rounds = exact + 0.6 * (-(-exact // 1) - exact) if exact >= 1 else 0.75 + 0.25 * exact
+        rounds = exact + 0.6 * (-(-exact // 1) - exact) if exact >= 1 else 0.6 + 0.4 * exact
         cost = rounds * (bm * bn + 6300)
         if best is None or cost < best[0]:
             best = (cost, cfg)
