@@ -43,6 +43,16 @@ int qf_pack_zero(const int32_t* zero, int8_t* out, int64_t G, int64_t N, int nbi
 int qf_transpose_scale(const uint16_t* scale, uint16_t* out, int64_t G, int64_t N, void* stream);
 
 /*
+ * src (n) bf16 -> dst (n) fp16, both 16-byte aligned.  Exact wherever fp16 is normal; magnitudes above
+ * 65504 saturate to +-65504, infinities and NaN pass through.  No reference counterpart: the reference
+ * takes fp16 activations only (qfactory/core/matmul.py:36, :133-136).  The matrix-core GEMM kernel moves
+ * its activation tiles from global memory to LDS without touching registers and cannot convert them on
+ * the way; QMatmul's closure converts bf16 rows with this call first (the other kernels convert in
+ * registers as they load).
+ */
+int qf_bf16_to_f16(const uint16_t* src, uint16_t* dst, int64_t n, void* stream);
+
+/*
  * Calibration kernels (no reference counterpart; the reference times with triton's do_bench only,
  * qfactory/profile.py:5-10).  qf_stream_read reads `bytes` (multiple of 16) with 128-bit loads and
  * writes one checksum word per block to `sink` (>= 4096 uint32); qf_stream_copy copies `bytes`

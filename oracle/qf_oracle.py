@@ -186,6 +186,64 @@ def gemv_plain_np(A, w, nbits):
 
 
 # ----------------------------------------------------------------------------------------------
+# bf16 activations and output.  The reference has no such path (it asserts fp16, qfactory/core/
+# matmul.py:36 and :133-136): this restates the project's own definition -- the activation converted
+# to fp16 (exact wherever fp16 is normal, saturating at +-65504, truncated toward zero on fp16's
+# subnormal grid below 2^-14), the fp16 dequantised weight of dequant_np, the sum carried exactly, one
+# rounding to bf16 (nearest even).  bf16 tensors travel as uint16 bit patterns.  The two conversions are
+# pinned against torch's CPU casts in tests/test_oracle.py; the forward itself is PARITY UNPINNED by the
+# reference.
+# ----------------------------------------------------------------------------------------------
+
+def bf16_bits_to_f32(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16_bits(x):
+    """Round to nearest even; NaN becomes the quiet NaN 0x7FC0."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    rounded = ((u + (0x7FFF + ((u >> 16) & 1))) >> 16).astype(np.uint16)
+    return np.where(np.isnan(x), np.uint16(0x7FC0), rounded)
+
+
+def bf16_bits_to_f16_sat(bits):
+    """bf16 -> fp16 rounding toward zero: finite magnitudes above 65504 become +-65504."""
+    with np.errstate(invalid="ignore"):
+        x = bf16_bits_to_f32(bits).astype(np.float64)
+    mag = np.abs(x)
+    with np.errstate(invalid="ignore", over="ignore"):
+        # truncate to the fp16 grid: spacing 2^(e-10) for normal values, 2^-24 below 2^-14
+        e = np.floor(np.log2(np.where((mag > 0) & np.isfinite(mag), mag, 1.0)))
+        ulp = np.exp2(np.maximum(e, -14.0) - 10.0)
+        trunc = np.floor(mag / ulp) * ulp
+    trunc = np.where(np.isfinite(mag), np.minimum(trunc, 65504.0), mag)
+    return np.copysign(trunc, x).astype(np.float16)
+
+
+def qlinear_bf16_np(A_bits, w, s, z, nbits, GS, rounded=True):
+    """A (M,K) bf16 bit patterns, packed w/s/z -> (M,N) bf16 bit patterns (or the float64 sums before the
+    final rounding)."""
+    K = A_bits.shape[1]
+    dq = dequant_np(w, s, z, K, nbits, GS)
+    acc = bf16_bits_to_f16_sat(A_bits).astype(np.float64) @ dq.astype(np.float64).T
+    if not rounded:
+        return acc
+    with np.errstate(over="ignore"):
+        return f32_to_bf16_bits(acc.astype(np.float32))
+
+
+def gemv_plain_bf16_np(A_bits, w, nbits, rounded=True):
+    K = A_bits.shape[1]
+    q = unpack_weight(w, K, nbits)
+    acc = bf16_bits_to_f16_sat(A_bits).astype(np.float64) @ q.astype(np.float64).T
+    if not rounded:
+        return acc
+    with np.errstate(over="ignore"):
+        return f32_to_bf16_bits(acc.astype(np.float32))
+
+
+# ----------------------------------------------------------------------------------------------
 # Error metrics of the acceptance bar (max relative error 1e-2, normalised RMS error 1e-3).
 # The relative error of an element is taken against max(|ref|, rms(ref)) so that outputs that
 # happen to fall near zero do not dominate; the reference itself only defines MSE < 0.1

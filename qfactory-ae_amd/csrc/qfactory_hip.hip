@@ -150,9 +150,38 @@ __global__ __launch_bounds__(kStreamThreads) void stream_copy_kernel(u32x4* __re
     }
 }
 
+// bf16 -> fp16, eight elements per thread: exact wherever fp16 is normal, magnitudes above 65504 saturate
+// (the conversion rounds toward zero), infinities and NaN pass through -- the conversion the quantized-linear
+// kernels apply to bf16 activations they read themselves.
+__device__ __forceinline__ uint32_t bf16_pair_to_f16_pair(uint32_t v) {
+    const float lo = __builtin_bit_cast(float, v << 16);
+    const float hi = __builtin_bit_cast(float, v & 0xFFFF0000u);
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+
+__global__ __launch_bounds__(256) void bf16_to_f16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                          int64_t n) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i + 8 <= n) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src + i);
+        *reinterpret_cast<u32x4*>(dst + i) = u32x4{bf16_pair_to_f16_pair(v.x), bf16_pair_to_f16_pair(v.y),
+                                                   bf16_pair_to_f16_pair(v.z), bf16_pair_to_f16_pair(v.w)};
+    } else {
+        for (int64_t j = i; j < n; j++) dst[j] = (uint16_t)bf16_pair_to_f16_pair(src[j]);
+    }
+}
+
 }  // namespace
 
-extern "C" int qf_version(void) { return 100; }
+extern "C" int qf_version(void) { return 101; }
+
+extern "C" int qf_bf16_to_f16(const uint16_t* src, uint16_t* dst, int64_t n, void* stream_) {
+    if (!src || !dst) return fail("qf_bf16_to_f16", "null pointer");
+    if (n <= 0) return fail("qf_bf16_to_f16", "n must be positive");
+    if (((uintptr_t)src | (uintptr_t)dst) % 16 != 0) return fail("qf_bf16_to_f16", "src and dst must be 16-byte aligned");
+    hipLaunchKernelGGL(bf16_to_f16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, (hipStream_t)stream_, src, dst, n);
+    return launched("qf_bf16_to_f16");
+}
 
 extern "C" int qf_pack_weight(const int32_t* weight, int8_t* out, int64_t K, int64_t N, int nbits, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;

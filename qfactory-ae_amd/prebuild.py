@@ -128,6 +128,22 @@ def large_parity_cases():
                _case(512, 16384, 4224, 4, 64), _case(256, 57344, 2816, 2, 128, True), _case(1024, 16384, 4096, 3, 128, True)])
 
 
+def bf16_cases():
+    """bf16 activations and output (tests/test_bf16_gpu.py): every kernel family, every bit width, ragged M and N,
+    plain integer weights, a partial last window in the GEMM kernel."""
+    cases = [_case(1, 4096, 4096), _case(2, 100, 256, 4, 64), _case(4, 77, 1024, 3, 128, True),      # dot2 GEMV
+             _case(1, 48, 4096, 2, 128, True), _case(2, 130, 512, 8, 32),
+             _case(1, 4096, 4096, 4, -1), _case(3, 100, 256, 8, -1),                                   # plain integer weights
+             _case(16, 4096, 4096), _case(12, 100, 2048, 3, 64), _case(16, 100, 4096, 2, 128),        # A-stationary
+             _case(7, 1000, 2048, 8, 128),
+             _case(5, 100, 11008, 4, 128), _case(9, 64, 8192, 8, 128), _case(12, 48, 14336, 2, 256),  # streaming skinny
+             _case(33, 100, 512, 4, 128), _case(300, 256, 2048, 4, 128), _case(64, 80, 11008, 2, 128, True),   # GEMM
+             _case(48, 64, 2816, 3, 64, True), _case(40, 72, 4160, 8, 32), _case(256, 4096, 4096),
+             _case(40, 100, 256, 2, 64),                                                               # generic fallback
+             _case(1, 96, 1024), _case(12, 96, 2048), _case(64, 96, 1024), _case(1, 64, 256)]          # range and argument checks
+    return [dict(c, act="bf16") for c in cases]
+
+
 def bench_cases():
     cases = [_case(1, N, K) for N, K in LLAMA2_7B]
     cases += [_case(1, N, K) for N, K in LLAMA3_70B]          # bench.py --small-m
@@ -163,7 +179,7 @@ def search_cases():
 def all_cases():
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases()):
+              + decode_cases() + bf16_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
@@ -176,13 +192,19 @@ def qfuncs_of(case):
     import torch
     from qfactory.core import QMatmul, Matmul
     from qfactory.qlinear import _m_bucket
-    if case["GS"] == -1:
-        op = Matmul(case["N"], case["K"], case["NBITS"], torch.float16, torch.int8)
-    else:
-        op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
-                     torch.float16, torch.int8, case["GS"])
-    op.init_qfuncs()
-    return op.qfuncs
+    dtypes = [torch.float16]                     # a module compiles its fp16 specialisation at construction
+    if case.get("act") == "bf16":
+        dtypes.append(torch.bfloat16)
+    qfuncs = []
+    for dtype in dtypes:
+        if case["GS"] == -1:
+            op = Matmul(case["N"], case["K"], case["NBITS"], dtype, torch.int8)
+        else:
+            op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
+                         dtype, torch.int8, case["GS"])
+        op.init_qfuncs()
+        qfuncs += op.qfuncs
+    return qfuncs
 
 
 def prebuild(cases=None, force=False, workers=None, verbose=True):

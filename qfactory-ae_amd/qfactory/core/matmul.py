@@ -8,7 +8,10 @@ same argument lists and checks.  Differences that matter to callers:
 
 * the closure launches for the *actual* number of activation rows (the reference silently computes
   only the rows it was compiled for, matmul.py:128);
-* supported widths are 2/3/4/8 bits; M may be anything >= 1 (large M runs on the matrix cores).
+* supported widths are 2/3/4/8 bits; M may be anything >= 1 (large M runs on the matrix cores);
+* ``dtype_a`` may be ``torch.bfloat16`` (the reference asserts fp16, matmul.py:36): activations and output
+  are then bf16, scales stay fp16.  The kernels compute on fp16 pairs either way; bf16 activations are
+  converted as they are loaded, or, for the GEMM kernel, by one ``qf_bf16_to_f16`` launch before it.
 """
 import json
 import logging
@@ -92,7 +95,7 @@ class QMatmul:
         self.base_impl = base_impl
         assert self.k % self.group_size == 0, f"Group size {self.group_size} must divide k {self.k}"
         assert self.layout == "nt", f"Layout {layout} is not supported"
-        assert dtype_a == torch.float16, f"Data type {dtype_a} is not supported"
+        assert dtype_a in (torch.float16, torch.bfloat16), f"Data type {dtype_a} is not supported"
         assert dtype_b == torch.int8, f"Data type {dtype_b} is not supported"
         assert nbits in (2, 3, 4, 8), f"{nbits}-bit weights are not supported"
 
@@ -118,10 +121,10 @@ class QMatmul:
 
     def get_dummy_inputs(self):
         require_gpu()
-        activation = torch.zeros((self.m, self.k), dtype=self.dtype_a, device="cuda")
+        activation = torch.zeros((self.m, self.k), dtype=dict(self.qfuncs[0].arg_name_type())["activation"], device="cuda")
         weight = torch.zeros(self.weight_shape, dtype=self.dtype_b, device="cuda")
         output = torch.empty((self.m, self.n), dtype=self.dtype_a, device="cuda")
-        scale = torch.zeros(self.scale_shape, dtype=self.dtype_a, device="cuda")
+        scale = torch.zeros(self.scale_shape, dtype=torch.float16, device="cuda")
         zero = torch.zeros(self.zero_shape, dtype=self.dtype_b, device="cuda")
         return activation, weight, output, scale, zero, torch.cuda.current_stream()
 
@@ -147,11 +150,16 @@ class QMatmul:
         self.runtimes = _compile_all(self.qfuncs)
         dummy = self.get_dummy_inputs() if len(self.runtimes) > 1 else None
         self.best_runtime, self.best_qfunc = _pick_best(self.runtimes, self.qfuncs, dummy, shape)
-        return self._wrap(self.best_runtime)
+        return self._wrap(self.best_runtime, self.best_qfunc)
 
-    def _wrap(self, runtime):
+    def _wrap(self, runtime, qfunc=None):
         n, k = self.n, self.k
         w_shape, s_shape, z_shape = self.weight_shape, self.scale_shape, self.zero_shape
+        dtype_a = self.dtype_a
+        # bf16 rows into a kernel that reads fp16 only (the GEMM kernel): one conversion launch first
+        convert_first = dtype_a == torch.bfloat16 and not (qfunc is not None and qfunc.converts_activations)
+        if convert_first:
+            from .. import native
         zero_empty = None
         if self.sym:
             require_gpu()
@@ -166,9 +174,9 @@ class QMatmul:
             assert scale.shape == s_shape
             assert zero.shape == z_shape
             # tensor dtype check
-            assert activation.dtype == torch.float16
+            assert activation.dtype == dtype_a
             assert weight.dtype == torch.int8
-            assert output.dtype == torch.float16
+            assert output.dtype == dtype_a
             assert scale.dtype == torch.float16
             assert zero.dtype == torch.int8
             # contiguous check
@@ -178,6 +186,8 @@ class QMatmul:
             assert scale.is_contiguous()
             assert zero.is_contiguous()
             assert activation.is_cuda and weight.is_cuda and output.is_cuda
+            if convert_first:
+                activation = native.bf16_to_f16(activation)
             return runtime.run_raw(
                 activation.shape[0],
                 (activation.data_ptr(), weight.data_ptr(), output.data_ptr(), scale.data_ptr(), zero.data_ptr()),
@@ -200,7 +210,7 @@ class Matmul:
         self.dtype_a, self.dtype_b = dtype_a, dtype_b
         self.layout = layout
         assert self.layout == "nt", f"Layout {layout} is not supported"
-        assert dtype_a == torch.float16, f"Data type {dtype_a} is not supported"
+        assert dtype_a in (torch.float16, torch.bfloat16), f"Data type {dtype_a} is not supported"
         assert dtype_b == torch.int8, f"Data type {dtype_b} is not supported"
         assert nbits in (2, 3, 4, 8), f"{nbits}-bit weights are not supported"
 
@@ -246,15 +256,16 @@ class Matmul:
 
     def _wrap(self, runtime):
         n, k, w_shape = self.n, self.k, self.weight_shape
+        dtype_a = self.dtype_a
 
         def inner(activation, weight, output):
             m = activation.shape[0]
             assert activation.shape == (m, k)
             assert weight.shape == w_shape
             assert output.shape == (m, n)
-            assert activation.dtype == torch.float16
+            assert activation.dtype == dtype_a
             assert weight.dtype == torch.int8
-            assert output.dtype == torch.float16
+            assert output.dtype == dtype_a
             assert activation.is_contiguous()
             assert weight.is_contiguous()
             assert output.is_contiguous()

@@ -25,6 +25,7 @@ from . import tiling
 Python2CppTypes = {  # python-side type -> (type in the C signature, type used inside)
     int: ("int", "int"),
     torch.float16: ("void*", "uint16_t*"),
+    torch.bfloat16: ("void*", "uint16_t*"),
     torch.int8: ("void*", "uint8_t*"),
     torch.cuda.streams.Stream: ("void*", "hipStream_t"),
 }
@@ -67,7 +68,10 @@ def _problem_of(qtile_a, qtile_b):
 
 
 class QMatmulQFunc(QFunc):
-    """activation (M,K) fp16  x  quantized weight (N,K), per-group scale (and zero)  ->  (M,N) fp16."""
+    """activation (M,K) fp16  x  quantized weight (N,K), per-group scale (and zero)  ->  (M,N) fp16.
+
+    Beyond the reference (fp16 only, matmul.py:36): a bf16 activation tile gives a bf16 output; scales
+    stay fp16, the packed tensors are the same."""
 
     def __init__(self, qtile_a, qtile_b, layout, base_impl=False):
         self.qtile_a, self.qtile_b, self.layout = qtile_a, qtile_b, layout
@@ -90,6 +94,17 @@ class QMatmulQFunc(QFunc):
         self.smem_quant = False                 # stage scales/zeros through LDS
         self.base_impl = base_impl
         self._gs = gs
+        assert qtile_a.dtype in (torch.float16, torch.bfloat16), f"Data type {qtile_a.dtype} is not supported for A"
+
+    @property
+    def act_dtype(self):
+        return self.qtile_a.dtype
+
+    @property
+    def converts_activations(self):
+        """Does the kernel read bf16 activations itself?  The GEMM kernel cannot (its activation tiles go
+        from global memory to LDS untouched): its caller converts the rows to fp16 first."""
+        return self.act_dtype == torch.bfloat16 and self.regime != "gemm"
 
     # -- description ------------------------------------------------------------------------
     @property
@@ -113,7 +128,8 @@ class QMatmulQFunc(QFunc):
 
     def arg_name_type(self):
         return [
-            ("activation", torch.float16), ("weight", torch.int8), ("output", torch.float16),
+            ("activation", self.act_dtype if self.converts_activations else torch.float16),
+            ("weight", torch.int8), ("output", self.act_dtype),
             ("scale", torch.float16), ("zero", torch.int8),
             ("stream", torch.cuda.streams.Stream),
         ]
@@ -156,6 +172,10 @@ class QMatmulQFunc(QFunc):
         if self.regime == "gemv" and p["NBITS"] == 2:
             # sixteen fields per word make the 2-bit GEMV decode-bound: measured 7.6 -> 6.9 us at 8192 x 8192
             defines.setdefault("QF_FUSED_AND_OR", 1)
+        if self.act_dtype == torch.bfloat16:
+            defines["QF_OUT_BF16"] = 1
+            if self.converts_activations:
+                defines["QF_IN_BF16"] = 1
         for name, value in sorted(defines.items()):
             code += f"#define {name} {value}\n"
         if self.regime == "gemv":
@@ -190,6 +210,7 @@ class QMatmulQFunc(QFunc):
         code += f"\t__return_code = {call}({args}, m, (hipStream_t)_stream);\n}}\n\n"
         desc = (f"regime={self.regime} M={p['M']} N={p['N']} K={p['K']} NBITS={p['NBITS']} GS={p['GS']} "
                 f"SYM={int(p['SYM'])} decode={self.decode_strategy} nt_b={int(not self.l2cache_b)} "
+                + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
         code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
         return code
@@ -209,6 +230,11 @@ class MatmulQFunc(QFunc):
         self.tiling_configs = tiling.gemv_tiling(1, qtile_b.shape[0], qtile_b.shape[1], qtile_b.nbits, None)
         self.l2cache_a = True
         self.l2cache_b = False
+        assert qtile_a.dtype in (torch.float16, torch.bfloat16), f"Data type {qtile_a.dtype} is not supported for A"
+
+    @property
+    def act_dtype(self):
+        return self.qtile_a.dtype
 
     @property
     def problem(self):
@@ -217,7 +243,7 @@ class MatmulQFunc(QFunc):
     def arg_name_type(self):
         return [
             ("m", int),
-            ("activation", torch.float16), ("weight", torch.int8), ("output", torch.float16),
+            ("activation", self.act_dtype), ("weight", torch.int8), ("output", self.act_dtype),
             ("stream", torch.cuda.streams.Stream),
         ]
 
@@ -234,6 +260,8 @@ class MatmulQFunc(QFunc):
         t = self.tiling_configs
         b = lambda x: "true" if x else "false"
         code = "// QFactory-HIP generated translation unit\n\n"
+        if self.act_dtype == torch.bfloat16:
+            code += "#define QF_IN_BF16 1\n#define QF_OUT_BF16 1\n"
         code += '#include "qf_gemv.hip.h"\n'
         code += '#if __has_include("qfactory_launch.h")\n#define QF_LAUNCH_PLAIN 1\n#include "qfactory_launch.h"\n#endif\n\n'
         code += (f"using Cfg = qf::GemvCfg<{p['NBITS']}, 0, false, false, {p['N']}, {p['K']}, "
@@ -242,6 +270,7 @@ class MatmulQFunc(QFunc):
         code += ("\t__return_code = qf::gemv_launch<Cfg>(_activation, _weight, _output, nullptr, nullptr, m, "
                  "(hipStream_t)_stream);\n}\n\n")
         desc = (f"regime=gemv-plain N={p['N']} K={p['K']} NBITS={p['NBITS']} nt_b={int(not self.l2cache_b)} "
+                + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
         code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
         return code

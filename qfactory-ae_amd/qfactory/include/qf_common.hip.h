@@ -53,6 +53,43 @@ __device__ __forceinline__ f16x2 as_f16x2(uint32_t v) { return __builtin_bit_cas
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
 
+// ---- element type of the activations and of the output ----
+// The reference computes on fp16 activations only (qfactory/core/matmul.py:36, :133-136).  A
+// translation unit compiled with QF_IN_BF16 reads bf16 activations, one with QF_OUT_BF16 writes a
+// bf16 output (fp32 accumulator rounded to nearest even, once).  Inside, every kernel keeps
+// computing on fp16 pairs against fp16 dequantised weights: a bf16 value has 8 significant bits
+// and is exact in fp16 wherever fp16 is normal (2^-14 <= |a| <= 65504); larger magnitudes saturate
+// to +-65504 and smaller ones are truncated to fp16's subnormal grid (the conversion rounds toward
+// zero), infinities and NaN pass through.
+#ifndef QF_IN_BF16
+#define QF_IN_BF16 0
+#endif
+#ifndef QF_OUT_BF16
+#define QF_OUT_BF16 0
+#endif
+
+// two activations as loaded (32 bits) -> the fp16 pair the kernels compute with
+__device__ __forceinline__ uint32_t act_pair(uint32_t v) {
+#if QF_IN_BF16
+    const float lo = __builtin_bit_cast(float, v << 16);
+    const float hi = __builtin_bit_cast(float, v & 0xFFFF0000u);
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+#else
+    return v;
+#endif
+}
+__device__ __forceinline__ u32x4 act_unit(u32x4 v) {
+    return u32x4{act_pair(v.x), act_pair(v.y), act_pair(v.z), act_pair(v.w)};
+}
+// fp32 result -> the 16 bits stored in the output
+__device__ __forceinline__ uint16_t f32_to_out_bits(float f) {
+#if QF_OUT_BF16
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+#else
+    return f32_to_f16_bits(f);
+#endif
+}
+
 // ---- global loads of NW 32-bit words (NW in {1,2,4}); NT = streaming (non-temporal) ----
 template <int NW, bool NT>
 __device__ __forceinline__ void load_words(const void* p, uint32_t (&dst)[NW]) {

@@ -50,6 +50,10 @@
 #define QF_GEMM_XCD_MAP 0
 #endif
 
+// The activation tiles go from global memory to LDS without passing through registers, so this kernel
+// cannot convert them on the way: it reads fp16 activations only (its output may be bf16).
+static_assert(!QF_IN_BF16, "the GEMM kernel takes fp16 activations: convert bf16 rows before the launch");
+
 namespace qf {
 
 template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int BM_, int NT32_, int WN_, int WK_, int PA_, bool NT_B_>
@@ -579,7 +583,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 const int n = n_wave + j * 32 + 8 * q + 4 * kb;
                 uint16_t h[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) h[e] = f32_to_f16_bits(acc[j][i][4 * q + e]);
+                for (int e = 0; e < 4; e++) h[e] = f32_to_out_bits(acc[j][i][4 * q + e]);
                 uint16_t* dst = Cout + (size_t)m * C::N + n;
                 if constexpr (C::N % 4 == 0) {
                     if (n < C::N) *reinterpret_cast<u32x2*>(dst) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};

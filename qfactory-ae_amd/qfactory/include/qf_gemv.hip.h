@@ -183,7 +183,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
             for (int c2 = 0; c2 < NCLS; c2++) cls_sum[c2] = 0.0f;
 #pragma unroll
             for (int r = 0; r < AR; r++) {
-                const uint32_t val = cvalid[it] ? a[m][it][r] : 0u;
+                const uint32_t val = cvalid[it] ? act_pair(a[m][it][r]) : 0u;   // once per block: the activations stay in registers
                 a[m][it][r] = val;
                 // sum of the pair in one instruction: dot2 with (1, 1)
                 cls_sum[D::cls(r % PAIRS)] = __builtin_amdgcn_fdot2(
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 const int u = v / MT, m = v % MT;
                 const int row = row_base + step * U + u;
                 if (row < C::N && m0 + m < m_total)
-                    Cout[(size_t)(m0 + m) * C::N + row] = f32_to_f16_bits(part[0]);
+                    Cout[(size_t)(m0 + m) * C::N + row] = f32_to_out_bits(part[0]);
             } else {
                 red[team][wk][step * V + v] = part[0];
             }
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         const int step = j / V, v = j % V;
         const int u = v / MT, m = v % MT;
         const int row = row_base + step * U + u;
-        if (row < C::N && m0 + m < m_total) Cout[(size_t)(m0 + m) * C::N + row] = f32_to_f16_bits(total);
+        if (row < C::N && m0 + m < m_total) Cout[(size_t)(m0 + m) * C::N + row] = f32_to_out_bits(total);
     }
 }
 

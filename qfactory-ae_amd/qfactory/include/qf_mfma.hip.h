@@ -129,7 +129,7 @@ __global__ __launch_bounds__(C::THREADS) void mfma_kernel(
         for (int p = 0; p < UPT; p++) {
             const int u = tpk + p * C::TPK;
             const int row = u / UNITS_PER_ROW, col = (u % UNITS_PER_ROW) * 8;
-            if (u < C::UNITS) *reinterpret_cast<u32x4*>(base + (size_t)row * PITCH + col) = regs[p];
+            if (u < C::UNITS) *reinterpret_cast<u32x4*>(base + (size_t)row * PITCH + col) = act_unit(regs[p]);
         }
     };
 
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(C::THREADS) void mfma_kernel(
             const int n = n0 + j * 16 + kb * 4;
             uint16_t h[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) h[e] = f32_to_f16_bits(acc[i][j][e]);
+            for (int e = 0; e < 4; e++) h[e] = f32_to_out_bits(acc[i][j][e]);
             uint16_t* dst = Cout + (size_t)m * C::N + n;
             if constexpr (C::N % 4 == 0) {
                 if (n < C::N) *reinterpret_cast<u32x2*>(dst) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};

@@ -207,7 +207,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                 for (int i = 0; i < LPC; i++) {
                     const int row = i * RPIA + lane / LPRA;
                     const int m = m0 + 16 * mt + row;
-                    u32x4 v = raw[mt][c][i];
+                    u32x4 v = act_unit(raw[mt][c][i]);
                     if (!(own && m < m_total)) v = u32x4{0, 0, 0, 0};
                     *reinterpret_cast<u32x4*>(wbuf + row * PITCH_A + (lane % LPRA) * 16) = v;
                 }
@@ -375,7 +375,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
             const int m = m0 + 16 * mt + ml;
             const int n = tile * 16 + nl;
-            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_f16_bits(total);
+            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_out_bits(total);
         }
         if (batch + 1 < C::NBATCH) __syncthreads();           // LDS slots are reused by the next batch
     };

@@ -156,7 +156,7 @@ __global__ __launch_bounds__(C::THREADS) void skinny_kernel(
         for (int mt = 0; mt < MT16; mt++)
 #pragma unroll
             for (int i = 0; i < NA; i++)
-                *reinterpret_cast<u32x4*>(abuf + (mt * 16 + i * C::A_RPI + a_row) * C::A_PITCH + a_col * 16) = raw.v[mt][i];
+                *reinterpret_cast<u32x4*>(abuf + (mt * 16 + i * C::A_RPI + a_row) * C::A_PITCH + a_col * 16) = act_unit(raw.v[mt][i]);
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int mt = 0; mt < MT16; mt++)
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(C::THREADS) void skinny_kernel(
             for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
             const int m = m0 + 16 * mt + ml;
             const int n = tile * 16 + nl;
-            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_f16_bits(total);
+            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_out_bits(total);
         }
     };
 

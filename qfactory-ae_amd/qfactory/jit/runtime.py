@@ -14,6 +14,7 @@ import torch
 
 _TYPE_NAMES = {
     "float16": torch.float16,
+    "bfloat16": torch.bfloat16,
     "int8": torch.int8,
     "stream": torch.cuda.streams.Stream,
     "int": int,
@@ -22,6 +23,7 @@ _NAME_OF_TYPE = {v: k for k, v in _TYPE_NAMES.items()}
 
 Python2CTypes = {
     torch.float16: ctypes.c_void_p,
+    torch.bfloat16: ctypes.c_void_p,
     torch.int8: ctypes.c_void_p,
     torch.cuda.streams.Stream: ctypes.c_void_p,
     int: ctypes.c_int,

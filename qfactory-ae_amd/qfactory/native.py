@@ -25,6 +25,7 @@ SIGNATURES = {
     "qf_pack_weight": (_INT, [_P, _P, _I64, _I64, _INT, _P]),
     "qf_pack_zero": (_INT, [_P, _P, _I64, _I64, _INT, _P]),
     "qf_transpose_scale": (_INT, [_P, _P, _I64, _I64, _P]),
+    "qf_bf16_to_f16": (_INT, [_P, _P, _I64, _P]),
     "qf_stream_read": (_INT, [_P, _SZ, _P, _P]),
     "qf_stream_copy": (_INT, [_P, _P, _SZ, _P]),
     "qf_add_rmsnorm": (_INT, [_P, _P, _P, _P, _I64, _I64, _F, _P]),
@@ -106,6 +107,18 @@ def transpose_scale(scale):
     G, N = scale.shape
     out = torch.empty(N, G, dtype=torch.float16, device=scale.device)
     _check(load().qf_transpose_scale(scale.data_ptr(), out.data_ptr(), G, N, _stream()), "qf_transpose_scale")
+    return out
+
+
+def bf16_to_f16(src, out=None):
+    """bf16 device tensor -> fp16 tensor of the same shape (saturating; see include/qfactory_hip.h)."""
+    import torch
+    assert src.is_cuda and src.dtype == torch.bfloat16 and src.is_contiguous()
+    if out is None:
+        out = torch.empty(src.shape, dtype=torch.float16, device=src.device)
+    assert out.is_cuda and out.dtype == torch.float16 and out.is_contiguous() and out.numel() == src.numel()
+    if src.numel():
+        _check(load().qf_bf16_to_f16(src.data_ptr(), out.data_ptr(), src.numel(), _stream()), "qf_bf16_to_f16")
     return out
 
 

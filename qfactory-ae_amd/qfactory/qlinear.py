@@ -9,7 +9,9 @@ the compiled closure for the constructor's ``batch_size``).
 Beyond the reference: ``forward`` accepts any number of rows.  The specialisation compiled at
 construction is tuned for ``batch_size``; other row counts get their own specialisation (per M
 bucket) on first use, because the best kernel family changes with M (register-resident GEMV for a
-few rows, matrix-core GEMM for many).
+few rows, matrix-core GEMM for many).  ``forward`` also accepts bf16 activations (the reference asserts
+fp16, qfactory/core/matmul.py:133-136) and then returns bf16; those specialisations are compiled on first
+use as well.  Scales stay fp16.
 """
 import torch
 
@@ -68,32 +70,32 @@ class GPTQLinear(torch.nn.Module):
 
         self._funcs = {}
         self.func = self._compile(batch_size, self.compile_flags)
-        self._funcs[_m_bucket(batch_size)] = self.func
+        self._funcs[(_m_bucket(batch_size), torch.float16)] = self.func
 
-    def _compile(self, m, compile_flags):
+    def _compile(self, m, compile_flags, dtype=torch.float16):
         matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
-                         torch.float16, torch.int8, self.group_size, base_impl=self.base_impl)
+                         dtype, torch.int8, self.group_size, base_impl=self.base_impl)
         func = matmul.compile_profile(**compile_flags)
         # One launch now: the first call of a specialisation loads its code object and may raise its
         # LDS limit (hipFuncSetAttribute), neither of which should happen inside a HIP-graph capture.
         if self.w.is_cuda:
-            x = torch.zeros(m, self.in_features, dtype=torch.float16, device=self.w.device)
-            out = torch.empty(m, self.out_features, dtype=torch.float16, device=self.w.device)
+            x = torch.zeros(m, self.in_features, dtype=dtype, device=self.w.device)
+            out = torch.empty(m, self.out_features, dtype=dtype, device=self.w.device)
             rc = func(x, self.w, out, self.s, self.z) if self.z is not None else func(x, self.w, out, self.s)
             if rc != 0:
                 raise RuntimeError(f"quantized linear launch failed with return code {rc}")
         return func
 
-    def func_for(self, m):
-        bucket = _m_bucket(m)
-        func = self._funcs.get(bucket)
+    def func_for(self, m, dtype=torch.float16):
+        key = (_m_bucket(m), dtype)
+        func = self._funcs.get(key)
         if func is None:
-            func = self._funcs[bucket] = self._compile(bucket, self.compile_flags)
+            func = self._funcs[key] = self._compile(key[0], self.compile_flags, dtype)
         return func
 
     def forward(self, x: torch.Tensor):
-        output = torch.empty(x.shape[0], self.w.shape[0], dtype=torch.float16, device=x.device)
-        func = self.func_for(x.shape[0])
+        output = torch.empty(x.shape[0], self.w.shape[0], dtype=x.dtype, device=x.device)
+        func = self.func_for(x.shape[0], x.dtype)
         if self.z is not None:
             rc = func(x, self.w, output, self.s, self.z)
         else:
@@ -126,12 +128,21 @@ class GEMVLinear(torch.nn.Module):
         self.in_features, self.out_features, self.n_bits = in_features, out_features, n_bits
         self.w = w
 
+        self.compile_flags = dict(compile_flags)
         matmul = Matmul(out_features, in_features, n_bits, torch.float16, torch.int8)
         self.func = matmul.compile_profile(**compile_flags)
+        self._funcs = {torch.float16: self.func}
+
+    def func_for(self, dtype):
+        func = self._funcs.get(dtype)
+        if func is None:
+            matmul = Matmul(self.out_features, self.in_features, self.n_bits, dtype, torch.int8)
+            func = self._funcs[dtype] = matmul.compile_profile(**self.compile_flags)
+        return func
 
     def forward(self, x: torch.Tensor):
-        output = torch.empty(x.shape[0], self.w.shape[0], dtype=torch.float16, device=x.device)
-        rc = self.func(x, self.w, output)
+        output = torch.empty(x.shape[0], self.w.shape[0], dtype=x.dtype, device=x.device)
+        rc = self.func_for(x.dtype)(x, self.w, output)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")
         return output

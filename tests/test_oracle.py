@@ -7,6 +7,7 @@ independent rounding routine, and closed-form special cases of the forward.
 """
 import numpy as np
 import pytest
+import torch
 
 
 # ---------------------------------------------------------------- packers: known answers
@@ -253,3 +254,58 @@ def test_torch_cpu_port_agrees_with_oracle(oracle):
                                        None if z is None else torch.from_numpy(z), nbits, GS).numpy()
         m = oracle.error_metrics(got, oracle.qlinear(A, w, s, z, nbits, GS))
         assert m["max_rel"] < 2e-3 and m["nrms"] < 5e-4
+
+
+# ---- bf16 activations / output (no reference counterpart; the oracle's conversions against torch's CPU casts) ----
+
+def _all_bf16_bits():
+    return np.arange(65536, dtype=np.uint32).astype(np.uint16)
+
+
+def test_bf16_widening_equals_torch_on_every_bit_pattern(oracle):
+    bits = _all_bf16_bits()
+    t = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    assert np.array_equal(oracle.bf16_bits_to_f32(bits).view(np.uint32), t.float().numpy().view(np.uint32))
+
+
+def test_bf16_rounding_equals_torch(oracle):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(200000, generator=g) * torch.exp(torch.randn(200000, generator=g) * 8)
+    x = torch.cat([x, torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 3.3895314e38, 3.4e38, 1e-40,
+                                    1.00390625, 1.01171875])])          # the last two are ties: to even
+    ref = x.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(oracle.f32_to_bf16_bits(x.numpy()), ref)
+    assert oracle.f32_to_bf16_bits(np.array([np.nan], dtype=np.float32))[0] == 0x7FC0
+
+
+def test_bf16_to_fp16_is_exact_where_fp16_is_normal_and_saturates_above(oracle):
+    bits = _all_bf16_bits()
+    f = oracle.bf16_bits_to_f32(bits)
+    h = oracle.bf16_bits_to_f16_sat(bits)
+    t = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).to(torch.float16).numpy()
+    mag = np.abs(f)
+    normal = (mag >= 2.0 ** -14) & (mag <= 65504)
+    assert np.array_equal(h[normal].view(np.uint16), t[normal].view(np.uint16))       # torch's cast, exact there
+    big = np.isfinite(f) & (mag > 65504)
+    assert np.array_equal(h[big], np.sign(f[big]).astype(np.float16) * np.float16(65504))
+    assert np.isposinf(h[bits == 0x7F80]) and np.isneginf(h[bits == 0xFF80]) and np.isnan(h[bits == 0x7FC0])
+    small = (mag < 2.0 ** -14) & (mag > 0)
+    err = np.abs(h[small].astype(np.float64)) - mag[small].astype(np.float64)
+    assert np.all(err <= 0) and np.all(err > -(2.0 ** -24))                           # toward zero, on the 2^-24 grid
+
+
+def test_bf16_forward_one_hot_selects_dequantised_column(oracle):
+    """A = one-hot row: the output is the dequantised weight column rounded to bf16."""
+    rng = np.random.default_rng(3)
+    N, K, nbits, GS = 24, 256, 4, 64
+    weight = rng.integers(0, 16, (K, N), dtype=np.int32)
+    scale = (rng.random((K // GS, N)) * 0.019 + 0.001).astype(np.float16)
+    zero = rng.integers(0, 16, (K // GS, N), dtype=np.int32)
+    w, s, z = oracle.pack_weight(weight, nbits), oracle.transpose_scale(scale), oracle.pack_zero(zero, nbits)
+    dq = oracle.dequant(w, s, z, K, nbits, GS)
+    A = np.zeros((3, K), dtype=np.uint16)
+    for m, k in enumerate((0, 77, 255)):
+        A[m, k] = 0x3F80                                                              # 1.0
+    out = oracle.qlinear_bf16_np(A, w, s, z, nbits, GS)
+    for m, k in enumerate((0, 77, 255)):
+        assert np.array_equal(out[m], oracle.f32_to_bf16_bits(dq[:, k].astype(np.float32)))
