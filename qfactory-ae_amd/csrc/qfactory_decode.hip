@@ -276,8 +276,11 @@ __global__ __launch_bounds__(kThreads) void silu_mul_kernel(const f16* __restric
     f16x8 o;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
+        // the hardware's exp2 and reciprocal (one ulp each in fp32): the same expression as the GEMV kernel's
+        // fused form of this step (qf_gemv.hip.h, QF_GEMV_SILU_MUL), so that the two give the same bits
         const float x = (float)gv[e];
-        o[e] = (f16)(x / (1.f + expf(-x))) * uv[e];
+        const float s = x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+        o[e] = (f16)s * uv[e];
     }
     *reinterpret_cast<f16x8*>(out + m * mlp + c) = o;
 }

@@ -91,7 +91,6 @@ class QuantLlama:
         # buffers of the fused decode step (one new position per sequence)
         f16 = dict(dtype=torch.float16, device="cuda")
         self._hdn, self._att = (torch.empty(batch, h, **f16) for _ in range(2))
-        self._act = torch.empty(batch, shape.mlp, **f16)
 
     def _norm(self, x, w):
         xf = x.float()
@@ -170,9 +169,9 @@ class QuantLlama:
             native.rope_decode_attention(qkv, pos, self.cos, self.sin, self.k_cache[li], self.v_cache[li], self._att)
             delta = self.linear(layer["o"], self._att)
             native.add_rmsnorm(x, delta, layer["norm2"], self._hdn, shape.eps)
-            gate_up = self.linear(layer["gate_up"], self._hdn)
-            native.silu_mul(gate_up, self._act)
-            delta = self.linear(layer["down"], self._act)
+            # SiLU(gate) * up: in the gate+up projection's final sum for few rows, else one launch behind it
+            act = layer["gate_up"].forward_silu_mul(self._hdn)
+            delta = self.linear(layer["down"], act)
         native.add_rmsnorm(x, delta, self.final_norm, self._hdn, shape.eps)
         return self._hdn @ self.lm_head.T
 

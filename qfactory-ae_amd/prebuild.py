@@ -168,7 +168,17 @@ def decode_cases():
     plus the tiny model tests/test_decode_gpu.py runs."""
     cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 1024)]
     cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
-    return cases
+    return cases + silu_mul_cases()
+
+
+def silu_mul_cases():
+    """Fused gate+up projections that write silu(gate) * up (GPTQLinear.forward_silu_mul, few rows): the decode
+    loop's at batch 1 and 2, the tiny test model's, and the shapes of tests/test_qlinear_gpu.py (ragged N/2,
+    every bit width, one wave per team and several)."""
+    cases = [_case(1, 22016, 4096), _case(2, 22016, 4096), _case(2, 1024, 256, 4, 64),
+             _case(1, 100, 1024, 2, 128, True), _case(2, 154, 512, 3, 64), _case(1, 260, 2048, 8, 128),
+             _case(1, 36, 256, 4, 128), _case(2, 8192, 11008, 4, 128)]
+    return [dict(c, epilogue="silu_mul") for c in cases]
 
 
 def search_cases():
@@ -202,6 +212,11 @@ def qfuncs_of(case):
         else:
             op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
                          dtype, torch.int8, case["GS"])
+        op.init_qfuncs()
+        qfuncs += op.qfuncs
+    if case.get("epilogue") == "silu_mul":
+        op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
+                     torch.float16, torch.int8, case["GS"], output_epilogue="silu_mul")
         op.init_qfuncs()
         qfuncs += op.qfuncs
     return qfuncs

@@ -86,8 +86,13 @@ def _pick_best(runtimes, qfuncs, dummy_inputs, what):
 
 class QMatmul:
     def __init__(self, m: int, n: int, k: int, nbits: int, sym: bool, dtype_a, dtype_b,
-                 group_size: int = -1, layout: str = "nt", base_impl: bool = False):
+                 group_size: int = -1, layout: str = "nt", base_impl: bool = False,
+                 output_epilogue: str = "none"):
         self.m, self.n, self.k = m, n, k
+        # "silu_mul" (beyond the reference): the weight is a fused gate+up projection and the closure's output is
+        # the (M, N/2) SwiGLU activation fp16(silu(gate)) * up; few rows only (the dot2 GEMV kernel), fp16 only
+        self.output_epilogue = output_epilogue
+        assert output_epilogue in ("none", "silu_mul")
         self.nbits, self.sym = nbits, sym
         self.dtype_a, self.dtype_b = dtype_a, dtype_b
         self.group_size = k if group_size == -1 else group_size
@@ -118,12 +123,13 @@ class QMatmul:
             QTile((self.m, self.k), self.dtype_a, 16),
             tile_b((self.n, self.k), self.dtype_b, self.nbits, (1, self.group_size)),
             "nt", self.base_impl)]
+        self.qfuncs[0].output_epilogue = self.output_epilogue
 
     def get_dummy_inputs(self):
         require_gpu()
         activation = torch.zeros((self.m, self.k), dtype=dict(self.qfuncs[0].arg_name_type())["activation"], device="cuda")
         weight = torch.zeros(self.weight_shape, dtype=self.dtype_b, device="cuda")
-        output = torch.empty((self.m, self.n), dtype=self.dtype_a, device="cuda")
+        output = torch.empty((self.m, self.n // 2 if self.output_epilogue == "silu_mul" else self.n), dtype=self.dtype_a, device="cuda")
         scale = torch.zeros(self.scale_shape, dtype=torch.float16, device="cuda")
         zero = torch.zeros(self.zero_shape, dtype=self.dtype_b, device="cuda")
         return activation, weight, output, scale, zero, torch.cuda.current_stream()
@@ -156,6 +162,7 @@ class QMatmul:
         n, k = self.n, self.k
         w_shape, s_shape, z_shape = self.weight_shape, self.scale_shape, self.zero_shape
         dtype_a = self.dtype_a
+        n_out = n // 2 if self.output_epilogue == "silu_mul" else n         # columns of the output
         # bf16 rows into a kernel that reads fp16 only (the GEMM kernel): one conversion launch first
         convert_first = dtype_a == torch.bfloat16 and not (qfunc is not None and qfunc.converts_activations)
         if convert_first:
@@ -169,7 +176,7 @@ class QMatmul:
             # tensor shape check
             assert activation.shape[1] == k
             assert weight.shape == w_shape
-            assert output.shape[1] == n
+            assert output.shape[1] == n_out
             assert activation.shape[0] == output.shape[0]
             assert scale.shape == s_shape
             assert zero.shape == z_shape

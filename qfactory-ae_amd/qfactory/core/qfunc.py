@@ -94,6 +94,9 @@ class QMatmulQFunc(QFunc):
         self.smem_quant = False                 # stage scales/zeros through LDS
         self.base_impl = base_impl
         self._gs = gs
+        # "silu_mul": the weight is a fused gate+up projection and the kernel writes the (M, N/2) SwiGLU activation
+        # fp16(silu(gate)) * up instead of the (M, N) projection (dot2 GEMV kernel only; not in the reference)
+        self.output_epilogue = "none"
         assert qtile_a.dtype in (torch.float16, torch.bfloat16), f"Data type {qtile_a.dtype} is not supported for A"
 
     @property
@@ -176,6 +179,10 @@ class QMatmulQFunc(QFunc):
             defines["QF_OUT_BF16"] = 1
             if self.converts_activations:
                 defines["QF_IN_BF16"] = 1
+        if self.output_epilogue != "none":
+            assert self.output_epilogue == "silu_mul" and self.regime == "gemv" and self.act_dtype == torch.float16, \
+                "only the dot2 GEMV kernel, on fp16, writes silu(gate) * up"
+            defines["QF_GEMV_GATE_UP_SILU"] = 1
         for name, value in sorted(defines.items()):
             code += f"#define {name} {value}\n"
         if self.regime == "gemv":
@@ -211,6 +218,7 @@ class QMatmulQFunc(QFunc):
         desc = (f"regime={self.regime} M={p['M']} N={p['N']} K={p['K']} NBITS={p['NBITS']} GS={p['GS']} "
                 f"SYM={int(p['SYM'])} decode={self.decode_strategy} nt_b={int(not self.l2cache_b)} "
                 + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
+                + ("epilogue=silu_mul " if self.output_epilogue == "silu_mul" else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
         code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
         return code

@@ -69,6 +69,23 @@ struct GemvCfg {
 #define QF_GEMV_A_FIRST 1
 #endif
 
+// 1: the weight matrix is a fused gate+up projection (rows 0 .. N/2-1 gate, rows N/2 .. N-1 up) and the
+// kernel writes the (M, N/2) SwiGLU activation out[m][i] = fp16(silu(gate[m][i])) * up[m][i] instead of
+// the (M, N) projection: a team's rows alternate between a gate row and its up row, and the pair meets in
+// the block's final sum.  Same roundings as the projection followed by qf_silu_mul of libqfactory_hip.so
+// (both results rounded to fp16 first; silu(x) = x * rcp(1 + exp2(-x * log2(e)))), which it replaces for
+// few rows.  The reference has no such fusion; its end-to-end runs leave the step to vLLM's SiluAndMul.
+#ifndef QF_GEMV_GATE_UP_SILU
+#define QF_GEMV_GATE_UP_SILU 0
+#endif
+
+__device__ __forceinline__ uint16_t silu_mul_f16(float gate_sum, float up_sum) {
+    const _Float16 g = (_Float16)gate_sum, u = (_Float16)up_sum;
+    const float x = (float)g;
+    const float s = x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+    return __builtin_bit_cast(uint16_t, (_Float16)((_Float16)s * u));
+}
+
 // Lower bound on resident waves per SIMD the register allocator must leave room for (0: no bound).
 #ifndef QF_GEMV_WAVES_PER_EU
 #define QF_GEMV_WAVES_PER_EU 0
@@ -91,6 +108,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     constexpr int P8 = 8 / C::ZFB;                     // zero-point fields per byte
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
     constexpr int NWH = C::NWH;
+    constexpr bool SILU = QF_GEMV_GATE_UP_SILU != 0;
 
     __shared__ float red[C::WN][WK][STEPS * V];
 
@@ -129,7 +147,9 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     auto load_stage = [&](Stage& st, int step) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int row = min(row_base + step * U + u, C::N - 1);
+            const int lrow = min(row_base + step * U + u, C::N - 1);
+            // gate+up: even positions of the sweep are gate rows, odd ones the up rows of the same output
+            const int row = SILU ? (lrow >> 1) + (lrow & 1) * (C::N / 2) : lrow;
             const uint8_t* wrow = W + (size_t)row * C::RB;
             const uint8_t* srow = reinterpret_cast<const uint8_t*>(S) + (size_t)row * C::G * 2;
             const uint8_t* zrow = Zp + (size_t)row * C::ZRB;
@@ -261,7 +281,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         wave_reduce_many<V>(part, lane);
         if (reduce_owner<V>(lane)) {
             const int v = reduce_index<V>(lane);
-            if constexpr (WK == 1) {          // one wave owns the rows: store straight from the lane
+            if constexpr (WK == 1 && !SILU) { // one wave owns the rows: store straight from the lane
                 const int u = v / MT, m = v % MT;
                 const int row = row_base + step * U + u;
                 if (row < C::N && m0 + m < m_total)
@@ -289,8 +309,25 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         }
     }
 
-    if constexpr (WK == 1) return;
+    if constexpr (WK == 1 && !SILU) return;
     __syncthreads();
+
+    if constexpr (SILU) {
+        // ---- cross-wave sums of a gate row and its up row, one store of their SwiGLU product ----
+        for (int j = tt; j < STEPS * V / 2; j += T) {
+            const int step = j / (V / 2), r = j % (V / 2);
+            const int u2 = r / MT, m = r % MT;
+            float gate = 0.0f, up = 0.0f;
+#pragma unroll
+            for (int w2 = 0; w2 < WK; w2++) {
+                gate += red[team][w2][step * V + (2 * u2) * MT + m];
+                up += red[team][w2][step * V + (2 * u2 + 1) * MT + m];
+            }
+            const int lrow = row_base + step * U + 2 * u2;
+            if (lrow < C::N && m0 + m < m_total) Cout[(size_t)(m0 + m) * (C::N / 2) + (lrow >> 1)] = silu_mul_f16(gate, up);
+        }
+        return;
+    }
 
     // ---- cross-wave sum and the single store of every output element ----
     for (int j = tt; j < STEPS * V; j += T) {
@@ -318,6 +355,8 @@ int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::QPARAM && !C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if ((C::V & (C::V - 1)) != 0 || C::V > 64) why = "U*MT must be a power of two <= 64";
     else if (C::THREADS > 1024) why = "block too large";
+    else if (QF_GEMV_GATE_UP_SILU && (C::N % 2 != 0 || C::U % 2 != 0)) why = "gate+up rows come in pairs: N and U must be even";
+    else if (QF_GEMV_GATE_UP_SILU && (QF_IN_BF16 || QF_OUT_BF16)) why = "the SwiGLU epilogue is fp16 only";
     else if (C::WN * C::WK * C::STEPS * C::V * 4 > 64 * 1024) why = "reduction scratch exceeds LDS";
     if (why) {
         fprintf(stderr, "qfactory gemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT=%d WK=%d WN=%d U=%d STEPS=%d VB=%d)\n",

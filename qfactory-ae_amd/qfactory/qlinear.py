@@ -72,15 +72,15 @@ class GPTQLinear(torch.nn.Module):
         self.func = self._compile(batch_size, self.compile_flags)
         self._funcs[(_m_bucket(batch_size), torch.float16)] = self.func
 
-    def _compile(self, m, compile_flags, dtype=torch.float16):
+    def _compile(self, m, compile_flags, dtype=torch.float16, epilogue="none"):
         matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
-                         dtype, torch.int8, self.group_size, base_impl=self.base_impl)
+                         dtype, torch.int8, self.group_size, base_impl=self.base_impl, output_epilogue=epilogue)
         func = matmul.compile_profile(**compile_flags)
         # One launch now: the first call of a specialisation loads its code object and may raise its
         # LDS limit (hipFuncSetAttribute), neither of which should happen inside a HIP-graph capture.
         if self.w.is_cuda:
             x = torch.zeros(m, self.in_features, dtype=dtype, device=self.w.device)
-            out = torch.empty(m, self.out_features, dtype=dtype, device=self.w.device)
+            out = torch.empty(m, self.out_features // (2 if epilogue == "silu_mul" else 1), dtype=dtype, device=self.w.device)
             rc = func(x, self.w, out, self.s, self.z) if self.z is not None else func(x, self.w, out, self.s)
             if rc != 0:
                 raise RuntimeError(f"quantized linear launch failed with return code {rc}")
@@ -100,6 +100,35 @@ class GPTQLinear(torch.nn.Module):
             rc = func(x, self.w, output, self.s, self.z)
         else:
             rc = func(x, self.w, output, self.s)
+        if rc != 0:
+            raise RuntimeError(f"quantized linear launch failed with return code {rc}")
+        return output
+
+
+    def fuses_silu_mul(self, m, dtype=torch.float16):
+        """Does ``forward_silu_mul`` on ``m`` rows run as one launch?  Where the dot2 GEMV kernel serves and its
+        rows come in pairs."""
+        bucket = _m_bucket(m)
+        if dtype != torch.float16 or self.out_features % 2 or tiling.regime_for(
+                bucket, self.in_features, self.n_bits, self.group_size, self.out_features) != "gemv":
+            return False
+        return tiling.gemv_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)["U"] % 2 == 0
+
+    def forward_silu_mul(self, x: torch.Tensor):
+        """For a fused gate+up projection (rows 0 .. N/2-1 gate, the rest up): the SwiGLU activation
+        ``silu(gate) * up`` of shape (M, N/2), i.e. ``silu_mul(self(x))``.  For few rows the product is formed in
+        the GEMV kernel's final sum (one launch); otherwise by ``forward`` followed by ``qf_silu_mul``.  Both give
+        the same bits.  Not in the reference, whose end-to-end runs leave the step to vLLM's ``SiluAndMul``."""
+        m, half = x.shape[0], self.out_features // 2
+        output = torch.empty(m, half, dtype=x.dtype, device=x.device)
+        if not self.fuses_silu_mul(m, x.dtype):
+            from . import native
+            return native.silu_mul(self.forward(x), output)
+        key = (_m_bucket(m), x.dtype, "silu_mul")
+        func = self._funcs.get(key)
+        if func is None:
+            func = self._funcs[key] = self._compile(key[0], self.compile_flags, x.dtype, "silu_mul")
+        rc = func(x, self.w, output, self.s, self.z) if self.z is not None else func(x, self.w, output, self.s)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")
         return output

@@ -175,3 +175,33 @@ def test_repeated_launches_give_identical_bits(qf, M, N, K, nbits):
             scrub.fill_(i)                        # push the operands out of L2 now and then
         out = layer(A)
         assert torch.equal(out, first), f"launch {i} differs"
+
+
+@pytest.mark.parametrize("case", prebuild.silu_mul_cases() + [dict(prebuild._case(16, 1024, 256, 4, 64), epilogue="silu_mul")], ids=_id)
+def test_gate_up_projection_with_swiglu_epilogue(qf, oracle, case):
+    """``forward_silu_mul`` of a fused gate+up projection: in the GEMV kernel's final sum for few rows (one
+    launch), through ``qf_silu_mul`` otherwise; both equal ``silu_mul(forward(x))`` bit for bit, and
+    fp16(silu(gate)) * up formed with PyTorch ops from the oracle's projection."""
+    from qfactory import native
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
+    print(f"[case] silu_mul {_id(case)}", flush=True)
+    A, weight, scale, zero = make_problem(321 + N + K + M, M, N, K, nbits, GS, sym)
+    if scale is not None:
+        scale = scale * (0.1 if nbits == 8 else 4)             # projections of a few units: SiLU across its bend, products in range
+    layer = qf.init(M, K, N, nbits, weight.cuda(), GS, scale.cuda(), None if zero is None else zero.cuda(),
+                    compile_flags=NO_SEARCH)
+    x = A.cuda()
+    out = layer.forward_silu_mul(x)
+    proj = layer(x)
+    torch.cuda.synchronize()
+    assert out.shape == (M, N // 2) and out.dtype == torch.float16
+    assert layer.fuses_silu_mul(M) == (M < 3)
+    if layer.fuses_silu_mul(M):
+        desc = layer._funcs[(M, torch.float16, "silu_mul")].runtime.description
+        assert "epilogue=silu_mul" in desc and "regime=gemv" in desc
+    if (N // 2) % 8 == 0:                                      # qf_silu_mul works in units of eight columns
+        assert torch.equal(out, native.silu_mul(proj, torch.empty(M, N // 2, dtype=torch.float16, device="cuda")))
+    ref = torch.from_numpy(reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS))
+    want = torch.nn.functional.silu(ref[:, : N // 2].float()).to(torch.float16) * ref[:, N // 2:]
+    # the projection itself is within the bar of the oracle (tested above); here the product of two such values
+    assert_close(oracle, out.cpu().numpy(), want.numpy(), _id(case))
