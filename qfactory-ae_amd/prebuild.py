@@ -177,7 +177,11 @@ def silu_mul_cases():
     every bit width, one wave per team and several)."""
     cases = [_case(1, 22016, 4096), _case(2, 22016, 4096), _case(2, 1024, 256, 4, 64),
              _case(1, 100, 1024, 2, 128, True), _case(2, 154, 512, 3, 64), _case(1, 260, 2048, 8, 128),
-             _case(1, 36, 256, 4, 128), _case(2, 8192, 11008, 4, 128)]
+             _case(1, 36, 256, 4, 128), _case(2, 8192, 11008, 4, 128),
+             # the A-stationary kernel: the decode loop's at batch 16, ragged M, one pair per block and many,
+             # every bit width, a last block with fewer pairs
+             _case(16, 22016, 4096), _case(16, 1024, 256, 4, 64), _case(5, 96, 1024, 4, 128), _case(12, 4128, 2048, 3, 64),
+             _case(32, 160, 4096, 2, 128, True), _case(7, 18016, 2048, 8, 128)]
     return [dict(c, epilogue="silu_mul") for c in cases]
 
 

@@ -90,7 +90,7 @@ class QMatmul:
                  output_epilogue: str = "none"):
         self.m, self.n, self.k = m, n, k
         # "silu_mul" (beyond the reference): the weight is a fused gate+up projection and the closure's output is
-        # the (M, N/2) SwiGLU activation fp16(silu(gate)) * up; few rows only (the dot2 GEMV kernel), fp16 only
+        # the (M, N/2) SwiGLU activation fp16(silu(gate)) * up; M <= 32 only (dot2 GEMV and A-stationary kernels), fp16 only
         self.output_epilogue = output_epilogue
         assert output_epilogue in ("none", "silu_mul")
         self.nbits, self.sym = nbits, sym

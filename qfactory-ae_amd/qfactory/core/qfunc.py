@@ -95,7 +95,7 @@ class QMatmulQFunc(QFunc):
         self.base_impl = base_impl
         self._gs = gs
         # "silu_mul": the weight is a fused gate+up projection and the kernel writes the (M, N/2) SwiGLU activation
-        # fp16(silu(gate)) * up instead of the (M, N) projection (dot2 GEMV kernel only; not in the reference)
+        # fp16(silu(gate)) * up instead of the (M, N) projection (the kernels for M <= 32; not in the reference)
         self.output_epilogue = "none"
         assert qtile_a.dtype in (torch.float16, torch.bfloat16), f"Data type {qtile_a.dtype} is not supported for A"
 
@@ -180,9 +180,9 @@ class QMatmulQFunc(QFunc):
             if self.converts_activations:
                 defines["QF_IN_BF16"] = 1
         if self.output_epilogue != "none":
-            assert self.output_epilogue == "silu_mul" and self.regime == "gemv" and self.act_dtype == torch.float16, \
-                "only the dot2 GEMV kernel, on fp16, writes silu(gate) * up"
-            defines["QF_GEMV_GATE_UP_SILU"] = 1
+            assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
+                "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, write silu(gate) * up"
+            defines["QF_GEMV_GATE_UP_SILU" if self.regime == "gemv" else "QF_MGEMV_GATE_UP_SILU"] = 1
         for name, value in sorted(defines.items()):
             code += f"#define {name} {value}\n"
         if self.regime == "gemv":

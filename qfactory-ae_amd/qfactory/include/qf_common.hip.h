@@ -90,6 +90,17 @@ __device__ __forceinline__ uint16_t f32_to_out_bits(float f) {
 #endif
 }
 
+// SwiGLU on two fp32 sums of a fused gate+up projection: both are rounded to fp16 as the projection's output
+// would be, then fp16(silu(gate)) * up with silu(x) = x * rcp(1 + exp2(-x * log2(e))) on the hardware's exp2 and
+// reciprocal -- the expression of qf_silu_mul in libqfactory_hip.so, so that a kernel's fused epilogue and the
+// projection followed by that call give the same bits.
+__device__ __forceinline__ uint16_t silu_mul_f16(float gate_sum, float up_sum) {
+    const _Float16 g = (_Float16)gate_sum, u = (_Float16)up_sum;
+    const float x = (float)g;
+    const float s = x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+    return __builtin_bit_cast(uint16_t, (_Float16)((_Float16)s * u));
+}
+
 // ---- global loads of NW 32-bit words (NW in {1,2,4}); NT = streaming (non-temporal) ----
 template <int NW, bool NT>
 __device__ __forceinline__ void load_words(const void* p, uint32_t (&dst)[NW]) {

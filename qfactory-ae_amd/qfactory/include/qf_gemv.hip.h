@@ -79,13 +79,6 @@ struct GemvCfg {
 #define QF_GEMV_GATE_UP_SILU 0
 #endif
 
-__device__ __forceinline__ uint16_t silu_mul_f16(float gate_sum, float up_sum) {
-    const _Float16 g = (_Float16)gate_sum, u = (_Float16)up_sum;
-    const float x = (float)g;
-    const float s = x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
-    return __builtin_bit_cast(uint16_t, (_Float16)((_Float16)s * u));
-}
-
 // Lower bound on resident waves per SIMD the register allocator must leave room for (0: no bound).
 #ifndef QF_GEMV_WAVES_PER_EU
 #define QF_GEMV_WAVES_PER_EU 0

@@ -29,6 +29,14 @@
 #define QF_MGEMV_SB 4
 #endif
 
+// 1: the weight matrix is a fused gate+up projection (rows 0 .. N/2-1 gate, the rest up) and the kernel writes
+// the (M, N/2) SwiGLU activation fp16(silu(gate)) * up instead of the (M, N) projection: a block's tiles
+// alternate between a gate tile and the up tile of the same outputs, and the two meet in the batch's final sum
+// (same bits as the projection followed by qf_silu_mul of libqfactory_hip.so).  Not in the reference.
+#ifndef QF_MGEMV_GATE_UP_SILU
+#define QF_MGEMV_GATE_UP_SILU 0
+#endif
+
 // Timing experiments (results are wrong when non-zero): bit 0 skips the activation loads, bit 1 the
 // dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores, bit 3 the weight loads.
 #ifndef QF_MGEMV_EXPERIMENT
@@ -66,8 +74,11 @@ struct MGemvCfg {
     static constexpr int THREADS = 64 * WK;
     static constexpr int BM = 16 * MT16;
     static constexpr int NT = (N + 15) / 16;       // 16-row weight tiles
-    static constexpr int GRID_X = NT < PB ? NT : PB;
-    static constexpr int SLOTS = (NT + GRID_X - 1) / GRID_X;               // tiles per block
+    static constexpr bool SILU = QF_MGEMV_GATE_UP_SILU != 0;
+    static constexpr int NPAIR = NT / 2;           // gate+up: pairs of a gate tile and its up tile
+    static constexpr int NUNIT = SILU ? NPAIR : NT;                        // what the blocks deal among themselves
+    static constexpr int GRID_X = NUNIT < PB ? NUNIT : PB;
+    static constexpr int SLOTS = (NUNIT + GRID_X - 1) / GRID_X * (SILU ? 2 : 1);   // tiles per block
     static constexpr int PF = PF_;                 // weight tiles in flight per wave (ring of stages): 2 or 4
     // tiles per batch (partials are reduced and stored per batch): no more than the block has
     static constexpr int SB = SLOTS < QF_MGEMV_SB ? (SLOTS + PF - 1) / PF * PF : QF_MGEMV_SB;
@@ -121,6 +132,13 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     const int m0 = blockIdx.y * C::BM;
     const int team_id = blockIdx.x;
     constexpr int TEAM_STRIDE = C::GRID_X;
+    // weight tile of the block's slot: plain, teams deal the tiles round-robin; gate+up, they deal pairs, and
+    // slots 2i and 2i + 1 are the gate tile and the up tile of pair i
+    auto unit_of = [&](int slot) { return team_id + (C::SILU ? slot >> 1 : slot) * TEAM_STRIDE; };
+    auto tile_ok = [&](int slot) { return unit_of(slot) < C::NUNIT; };
+    auto tile_clamped = [&](int slot) {
+        return min(unit_of(slot), C::NUNIT - 1) + (C::SILU ? (slot & 1) * C::NPAIR : 0);
+    };
 
     // chunks [lo, lo + CH) are read by this wave; it owns [own_from, own_from + CH) (a clamped last
     // wave re-reads chunks of its neighbours with zeroed activations: every address stays in bounds)
@@ -171,7 +189,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     WStage ring[PF];
 #pragma unroll
     for (int p = 0; p < PF; p++)
-        if (p < SLOTS) load_tile(ring[p], min(team_id + p * TEAM_STRIDE, C::NT - 1));
+        if (p < SLOTS) load_tile(ring[p], tile_clamped(p));
 
     // ---- resident activations, brought into MFMA fragment order through the wave's LDS buffer:
     //      fragment (mt, c, t) = A[m0 + 16*mt + r][(lo+c)*CHUNK + kb*EPL + 8t .. +8] ----
@@ -237,7 +255,6 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         mg_static_for<0, SB>([&](auto sb_tag) {
             constexpr int sb = decltype(sb_tag)::value;
             const int slot = batch * SB + sb;
-            const int tile = team_id + slot * TEAM_STRIDE;
             WStage& cur = ring[sb % PF];
             f32x4 acc[MT16];
 #pragma unroll
@@ -277,12 +294,12 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 #pragma unroll
                 for (int j = 0; j < NZI; j++) qz[j] = C::SYM ? 0u : cur.z[j];
                 if constexpr (STATIC_BATCH) {
-                    if constexpr (BT::value * SB + sb + PF < SLOTS) load_tile(cur, min(tile + PF * TEAM_STRIDE, C::NT - 1));
+                    if constexpr (BT::value * SB + sb + PF < SLOTS) load_tile(cur, tile_clamped(slot + PF));
                 } else {
-                    if (slot + PF < SLOTS) load_tile(cur, min(tile + PF * TEAM_STRIDE, C::NT - 1));
+                    if (slot + PF < SLOTS) load_tile(cur, tile_clamped(slot + PF));
                 }
             }
-            if (have_slot && tile < C::NT && !(QF_MGEMV_EXPERIMENT & 2)) {               // wave-uniform
+            if (have_slot && tile_ok(slot) && !(QF_MGEMV_EXPERIMENT & 2)) {              // wave-uniform
 #pragma unroll
                 for (int c = 0; c < CH; c++) {
                     const int g = ((lo + c) * CHUNK + kb * EPL) / C::GS;     // group of this lane's fields
@@ -362,12 +379,32 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         //      (m = o/16, n = o%16 inside a tile): sixteen neighbouring lanes read sixteen different
         //      banks and store 32 contiguous bytes, and the WK-deep sums are spread over all waves
         //      instead of one wave per tile. ----
-        constexpr int OUTPUTS = SB * MT16 * 256;
+        if constexpr (C::SILU) {
+            // a gate tile (even slot) and its up tile (odd slot): both sums, one store of their SwiGLU product
+            constexpr int OUTPUTS_P = SB / 2 * MT16 * 256;
+            for (int o = tid; o < OUTPUTS_P; o += 64 * WK) {
+                const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
+                const int sp = p / MT16, mt = p % MT16;
+                const int slot = batch * SB + 2 * sp;
+                if (slot >= SLOTS || !tile_ok(slot)) continue;
+                const float* base = redf + (((size_t)(2 * sp) * MT16 + mt) * 64 + nl + 16 * (ml >> 2)) * 4 + (ml & 3);
+                float gate = 0.f, up = 0.f;
+#pragma unroll
+                for (int k2 = 0; k2 < WK; k2++) {
+                    gate += base[(size_t)k2 * SB * MT16 * 256];
+                    up += base[(size_t)k2 * SB * MT16 * 256 + MT16 * 256];
+                }
+                const int m = m0 + 16 * mt + ml;
+                const int n = unit_of(slot) * 16 + nl;
+                if (m < m_total) Cout[(size_t)m * (C::N / 2) + n] = silu_mul_f16(gate, up);
+            }
+        }
+        constexpr int OUTPUTS = C::SILU ? 0 : SB * MT16 * 256;
         for (int o = tid; o < OUTPUTS && !(QF_MGEMV_EXPERIMENT & 4); o += 64 * WK) {
             const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
             const int sb = p / MT16, mt = p % MT16;
             const int slot = batch * SB + sb;
-            const int tile = team_id + slot * TEAM_STRIDE;
+            const int tile = unit_of(slot);
             if (slot >= SLOTS || tile >= C::NT) continue;
             const float* base = redf + (((size_t)sb * MT16 + mt) * 64 + nl + 16 * (ml >> 2)) * 4 + (ml & 3);
             float total = 0.f;
@@ -403,6 +440,8 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
     else if (C::GS % C::CHUNK != 0 && C::CHUNK % C::GS != 0) why = "GS must divide the chunk or be a multiple of it";
     else if (C::PF != 1 && C::PF != 2 && C::PF != 4) why = "PF must be 1, 2 or 4";
     else if (C::LDS_BYTES > 160 * 1024) why = "partial tiles exceed the 160 KB of LDS";
+    else if (C::SILU && (C::N % 32 != 0 || C::SB % 2 != 0)) why = "gate+up: N/2 must be whole 16-row tiles and a batch whole pairs";
+    else if (C::SILU && (QF_IN_BF16 || QF_OUT_BF16)) why = "the SwiGLU epilogue is fp16 only";
     if (why) {
         fprintf(stderr, "qfactory mgemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT16=%d WK=%d CH=%d PB=%d PF=%d)\n",
                 why, C::NBITS, C::GS, C::N, C::K, C::MT16, C::WK, C::CH, C::PB, C::PF);

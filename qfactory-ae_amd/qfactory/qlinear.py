@@ -107,17 +107,21 @@ class GPTQLinear(torch.nn.Module):
 
     def fuses_silu_mul(self, m, dtype=torch.float16):
         """Does ``forward_silu_mul`` on ``m`` rows run as one launch?  Where the dot2 GEMV kernel serves and its
-        rows come in pairs."""
+        rows come in pairs, or the A-stationary kernel and gate and up are whole 16-row tiles."""
         bucket = _m_bucket(m)
-        if dtype != torch.float16 or self.out_features % 2 or tiling.regime_for(
-                bucket, self.in_features, self.n_bits, self.group_size, self.out_features) != "gemv":
+        if dtype != torch.float16 or self.out_features % 2:
+            return False
+        regime = tiling.regime_for(bucket, self.in_features, self.n_bits, self.group_size, self.out_features)
+        if regime == "mgemv":
+            return self.out_features % 32 == 0
+        if regime != "gemv":
             return False
         return tiling.gemv_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)["U"] % 2 == 0
 
     def forward_silu_mul(self, x: torch.Tensor):
         """For a fused gate+up projection (rows 0 .. N/2-1 gate, the rest up): the SwiGLU activation
-        ``silu(gate) * up`` of shape (M, N/2), i.e. ``silu_mul(self(x))``.  For few rows the product is formed in
-        the GEMV kernel's final sum (one launch); otherwise by ``forward`` followed by ``qf_silu_mul``.  Both give
+        ``silu(gate) * up`` of shape (M, N/2), i.e. ``silu_mul(self(x))``.  Up to 32 rows the product is formed in
+        the kernel's final sum (one launch); otherwise by ``forward`` followed by ``qf_silu_mul``.  Both give
         the same bits.  Not in the reference, whose end-to-end runs leave the step to vLLM's ``SiluAndMul``."""
         m, half = x.shape[0], self.out_features // 2
         output = torch.empty(m, half, dtype=x.dtype, device=x.device)
