@@ -128,6 +128,22 @@ def kernel_event_time_us(lins, x, reps=64):
     return best[len(best) // 2]
 
 
+def module_time_us(lins, x, reps=256):
+    """Average time of one eager ``layer(x)`` call -- output allocation, Python checks, ctypes and the launch, as the
+    reference's latency harness times it (qfactory/testing.py:31-35) -- rotating over the layers' weight copies;
+    wall clock around `reps` calls with a synchronisation on both sides.  At small M this is bound by the host
+    (the kernel is shorter than its enqueue), which is why the decode loop replays HIP graphs."""
+    import torch
+    for i in range(16):
+        lins[i % len(lins)](x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(reps):
+        lins[i % len(lins)](x)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps * 1e6
+
+
 def dense_fp16_time_us(M, N, K, total_bytes=600e6):
     """The vendor library's dense fp16 GEMM of the same shape (torch.matmul on hipBLASLt / rocBLAS), cold
     weights: the comparison the reference's own evaluation makes against cuBLAS
@@ -366,9 +382,11 @@ def main():
         b = algorithmic_bytes(M, N, K)
         rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
                "TFLOP/s": round(2 * M * N * K / us / 1e6, 3), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
-               "bytes": int(b), "kernel": layers[0][name].func.runtime.description}
+               "bytes": int(b), "kernel": layers[0][name].func.runtime.description,
+               "module_us": round(module_time_us([layer[name] for layer in layers], acts[K]), 2)}
         shapes_report.append(rec)
-        log(f"[bench] {name:8s} N={N:6d} K={K:6d}  {us:7.2f} us  {rec['GB/s']:7.1f} GB/s  {100 * rec['hbm_frac']:5.1f}% of HBM peak")
+        log(f"[bench] {name:8s} N={N:6d} K={K:6d}  {us:7.2f} us  {rec['GB/s']:7.1f} GB/s  {100 * rec['hbm_frac']:5.1f}% of HBM peak"
+            f"  (eager layer(x): {rec['module_us']:.2f} us per call)")
         if name == DOMINANT:
             dominant = rec
 
