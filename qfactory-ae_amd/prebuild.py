@@ -144,6 +144,15 @@ def bf16_cases():
     return [dict(c, act="bf16") for c in cases]
 
 
+def smem_quant_cases():
+    """The dot2 GEMV kernel with the scales and zero-points of a block's rows staged through LDS (the schedule
+    search's other choice; tests/test_qlinear_gpu.py): every bit width, symmetric and not, a last block past N,
+    several stages per block, one wave per team and several."""
+    cases = [_case(1, 100, 1024), _case(2, 77, 512, 3, 64, True), _case(1, 130, 2048, 8, 128, True),
+             _case(2, 22016, 4096), _case(1, 4096, 11008), _case(1, 48, 4096, 2, 128), _case(4, 50, 512, 4, 16)]
+    return [dict(c, smem_quant=True) for c in cases]
+
+
 def bench_cases():
     cases = [_case(1, N, K) for N, K in LLAMA2_7B]
     cases += [_case(1, N, K) for N, K in LLAMA3_70B]          # bench.py --small-m
@@ -193,7 +202,7 @@ def search_cases():
 def all_cases():
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases() + bf16_cases()):
+              + decode_cases() + bf16_cases() + smem_quant_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
@@ -218,6 +227,11 @@ def qfuncs_of(case):
                          dtype, torch.int8, case["GS"])
         op.init_qfuncs()
         qfuncs += op.qfuncs
+    if case.get("smem_quant"):
+        op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
+                     torch.float16, torch.int8, case["GS"])
+        op.init_qfuncs()
+        qfuncs += [q.clone(smem_quant=True) for q in op.qfuncs]
     if case.get("epilogue") == "silu_mul":
         op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
                      torch.float16, torch.int8, case["GS"], output_epilogue="silu_mul")

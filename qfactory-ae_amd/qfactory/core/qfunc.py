@@ -91,7 +91,8 @@ class QMatmulQFunc(QFunc):
         # Load-path scheduling
         self.l2cache_a = True                   # activations: normal (cached) loads
         self.l2cache_b = False                  # weights: streaming (non-temporal) loads
-        self.smem_quant = False                 # stage scales/zeros through LDS
+        self.smem_quant = False                 # scales / zero-points of a block's rows through LDS (dot2 GEMV kernel);
+        #                                         measured slower at M = 1 (a barrier in a one-shot block), 3 % faster at M = 2
         self.base_impl = base_impl
         self._gs = gs
         # "silu_mul": the weight is a fused gate+up projection and the kernel writes the (M, N/2) SwiGLU activation
@@ -144,7 +145,8 @@ class QMatmulQFunc(QFunc):
         return [self.clone()]
 
     def schedule(self) -> List[QFunc]:
-        return [self.clone(l2cache_a=True, l2cache_b=b) for b in (False, True)]
+        smem = (False, True) if self.regime == "gemv" and self.output_epilogue == "none" else (False,)
+        return [self.clone(l2cache_a=True, l2cache_b=b, smem_quant=s) for b in (False, True) for s in smem]
 
     def lower(self) -> List[QFunc]:
         p = self.problem
@@ -183,6 +185,8 @@ class QMatmulQFunc(QFunc):
             assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
                 "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, write silu(gate) * up"
             defines["QF_GEMV_GATE_UP_SILU" if self.regime == "gemv" else "QF_MGEMV_GATE_UP_SILU"] = 1
+        if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none":
+            defines["QF_GEMV_SMEM_QUANT"] = 1
         for name, value in sorted(defines.items()):
             code += f"#define {name} {value}\n"
         if self.regime == "gemv":
@@ -219,6 +223,7 @@ class QMatmulQFunc(QFunc):
                 f"SYM={int(p['SYM'])} decode={self.decode_strategy} nt_b={int(not self.l2cache_b)} "
                 + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
                 + ("epilogue=silu_mul " if self.output_epilogue == "silu_mul" else "")
+                + ("smem_quant=1 " if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none" else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
         code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
         return code

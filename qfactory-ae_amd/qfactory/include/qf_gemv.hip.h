@@ -79,6 +79,14 @@ struct GemvCfg {
 #define QF_GEMV_GATE_UP_SILU 0
 #endif
 
+// 1: the scales and zero-points of the block's rows go through LDS (the reference's SMEM_QUANT choice,
+// qfactory/include/gptq_gemv.h:62-82): the rows of a block are contiguous in both tensors, so the block fetches
+// them with coalesced loads issued ahead of everything else, and a lane reads its group's pair from LDS instead
+// of issuing two narrow global loads behind every 16 bytes of weights.
+#ifndef QF_GEMV_SMEM_QUANT
+#define QF_GEMV_SMEM_QUANT 0
+#endif
+
 // Lower bound on resident waves per SIMD the register allocator must leave room for (0: no bound).
 #ifndef QF_GEMV_WAVES_PER_EU
 #define QF_GEMV_WAVES_PER_EU 0
@@ -102,7 +110,11 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
     constexpr int NWH = C::NWH;
     constexpr bool SILU = QF_GEMV_GATE_UP_SILU != 0;
+    constexpr bool SMEMQ = QF_GEMV_SMEM_QUANT != 0 && C::QPARAM;
+    constexpr int SQ_WORDS = SMEMQ ? (C::RPB * C::G * 2 + 3) / 4 : 1;           // 32-bit words of the block's scales
+    constexpr int ZQ_WORDS = SMEMQ && !C::SYM ? (C::RPB * C::ZRB + 3) / 4 : 1;  // and of its zero-points
 
+    __shared__ uint32_t sq_s[SQ_WORDS], sq_z[ZQ_WORDS];
     __shared__ float red[C::WN][WK][STEPS * V];
 
     const int tid = threadIdx.x;
@@ -115,6 +127,29 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     const int tt = wk * 64 + lane;
     const int m0 = blockIdx.y * MT;
     const int row_base = blockIdx.x * C::RPB + team * C::RPT;
+
+    // ---- scales / zero-points of the block's RPB rows: requested before anything else (SMEM_QUANT) ----
+    constexpr int SQ_PER = (SQ_WORDS + C::THREADS - 1) / C::THREADS, ZQ_PER = (ZQ_WORDS + C::THREADS - 1) / C::THREADS;
+    uint32_t sq_reg[SQ_PER], zq_reg[ZQ_PER];
+    if constexpr (SMEMQ) {
+        // rows past N (last block) clamp to the end of the tensor: loaded, never used
+        const size_t s_words = ((size_t)C::N * C::G * 2) / 4, z_words = ((size_t)C::N * C::ZRB) / 4;
+        const uint32_t* sg = reinterpret_cast<const uint32_t*>(S) + ((size_t)blockIdx.x * C::RPB * C::G * 2) / 4;
+        const uint32_t* zg = reinterpret_cast<const uint32_t*>(Zp) + ((size_t)blockIdx.x * C::RPB * C::ZRB) / 4;
+        const size_t s_first = ((size_t)blockIdx.x * C::RPB * C::G * 2) / 4, z_first = ((size_t)blockIdx.x * C::RPB * C::ZRB) / 4;
+#pragma unroll
+        for (int i = 0; i < SQ_PER; i++) {
+            const int wd = tid + i * C::THREADS;
+            sq_reg[i] = sg[min((size_t)wd, s_words - 1 - s_first)];
+        }
+        if constexpr (!C::SYM) {
+#pragma unroll
+            for (int i = 0; i < ZQ_PER; i++) {
+                const int wd = tid + i * C::THREADS;
+                zq_reg[i] = zg[min((size_t)wd, z_words - 1 - z_first)];
+            }
+        }
+    }
 
     // ---- per-lane chunk bookkeeping ----
     int coff[IT];            // byte offset of the chunk inside a packed weight row
@@ -150,7 +185,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
             for (int it = 0; it < IT; it++) {
                 load_words<NW, C::NT_B>(wrow + (uint32_t)coff[it], st.w[u][it]);
                 if constexpr (NWH > 0) load_words<NWH, C::NT_B>(wrow + (uint32_t)(C::HI_OFF + coff[it] / 2), st.h[u][it]);
-                if constexpr (C::QPARAM && !(QF_GEMV_EXPERIMENT & 4)) {
+                if constexpr (C::QPARAM && !SMEMQ && !(QF_GEMV_EXPERIMENT & 4)) {
                     st.s[u][it] = *reinterpret_cast<const uint16_t*>(srow + (uint32_t)(goff[it] * 2));
                     if constexpr (!C::SYM) st.z[u][it] = zrow[(uint32_t)(goff[it] / P8)];
                 }
@@ -186,6 +221,17 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         }
     }
     if constexpr (QF_GEMV_A_FIRST) load_stage(st0, 0);
+    if constexpr (SMEMQ) {
+#pragma unroll
+        for (int i = 0; i < SQ_PER; i++)
+            if (tid + i * C::THREADS < SQ_WORDS) sq_s[tid + i * C::THREADS] = sq_reg[i];
+        if constexpr (!C::SYM) {
+#pragma unroll
+            for (int i = 0; i < ZQ_PER; i++)
+                if (tid + i * C::THREADS < ZQ_WORDS) sq_z[tid + i * C::THREADS] = zq_reg[i];
+        }
+        __syncthreads();
+    }
     // ---- and their per-chunk sums ----
 #pragma unroll
     for (int it = 0; it < IT; it++) {
@@ -249,11 +295,14 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 }
                 float sc = 1.0f, zf = 0.0f;
                 if constexpr (C::QPARAM) {
-                    sc = f16_bits_to_f32((uint16_t)st.s[u][it]);
+                    const int brow = team * C::RPT + step * U + u;            // row inside the block
+                    if constexpr (SMEMQ) sc = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(sq_s)[brow * C::G + goff[it]]);
+                    else sc = f16_bits_to_f32((uint16_t)st.s[u][it]);
                     if constexpr (C::SYM) {
                         zf = (float)(1 << (C::NBITS - 1));
                     } else {
-                        zf = (float)((st.z[u][it] >> ((goff[it] % P8) * C::ZFB)) & ZMASK);
+                        const uint32_t zbyte = SMEMQ ? reinterpret_cast<const uint8_t*>(sq_z)[brow * C::ZRB + goff[it] / P8] : st.z[u][it];
+                        zf = (float)((zbyte >> ((goff[it] % P8) * C::ZFB)) & ZMASK);
                     }
                 }
 #pragma unroll
@@ -350,6 +399,10 @@ int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::THREADS > 1024) why = "block too large";
     else if (QF_GEMV_GATE_UP_SILU && (C::N % 2 != 0 || C::U % 2 != 0)) why = "gate+up rows come in pairs: N and U must be even";
     else if (QF_GEMV_GATE_UP_SILU && (QF_IN_BF16 || QF_OUT_BF16)) why = "the SwiGLU epilogue is fp16 only";
+    else if (QF_GEMV_SMEM_QUANT && QF_GEMV_GATE_UP_SILU) why = "scales through LDS need a block's rows contiguous: not with the gate+up row order";
+    else if (QF_GEMV_SMEM_QUANT && C::QPARAM && ((C::N * C::G * 2) % 4 != 0 || (!C::SYM && (C::N * C::ZRB) % 4 != 0 )|| (C::RPB * C::G * 2) % 4 != 0 || (!C::SYM && (C::RPB * C::ZRB) % 4 != 0)))
+        why = "scales through LDS: a block's scales and zero-points must be whole 32-bit words";
+    else if (QF_GEMV_SMEM_QUANT && C::QPARAM && (size_t)C::RPB * C::G * 2 + (size_t)C::RPB * C::ZRB + sizeof(float) * C::WN * C::WK * C::STEPS * C::V > 64 * 1024) why = "scales through LDS exceed LDS";
     else if (C::WN * C::WK * C::STEPS * C::V * 4 > 64 * 1024) why = "reduction scratch exceeds LDS";
     if (why) {
         fprintf(stderr, "qfactory gemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT=%d WK=%d WN=%d U=%d STEPS=%d VB=%d)\n",

@@ -208,3 +208,29 @@ def test_gate_up_projection_with_swiglu_epilogue(qf, oracle, case):
     want = torch.nn.functional.silu(ref[:, : N // 2].float()).to(torch.float16) * ref[:, N // 2:]
     # the projection itself is within the bar of the oracle (tested above); here the product of two such values
     assert_close(oracle, out.cpu().numpy(), want.numpy(), _id(case))
+
+
+@pytest.mark.parametrize("case", prebuild.smem_quant_cases(), ids=_id)
+def test_gemv_with_scales_through_lds(oracle, case):
+    """The schedule search's other choice for the dot2 GEMV kernel (``smem_quant``, the reference's SMEM_QUANT):
+    scales and zero-points of a block's rows staged through LDS.  Same results as the default to the bar."""
+    from qfactory.convert import convert_params
+    from qfactory.core import QMatmul
+    from qfactory.jit import jit
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
+    print(f"[case] smem_quant {_id(case)}", flush=True)
+    A, weight, scale, zero = make_problem(555 + N + K + M, M, N, K, nbits, GS, sym)
+    w, s, z = convert_params({"K": K, "N": N, "NBITS": nbits, "GS": GS},
+                             (weight.cuda(), scale.cuda(), None if zero is None else zero.cuda()))
+    op = QMatmul(M, N, K, nbits, sym, torch.float16, torch.int8, GS)
+    op.init_qfuncs()
+    qfunc = op.qfuncs[0].clone(smem_quant=True)
+    assert qfunc.regime == "gemv"
+    func = op._wrap(jit.compile(qfunc), qfunc)
+    assert "smem_quant=1" in func.runtime.description
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    rc = func(A.cuda(), w, out, s) if sym else func(A.cuda(), w, out, s, z)
+    torch.cuda.synchronize()
+    assert rc == 0
+    ref = reference_output(oracle, A, w, s, z, nbits, GS)
+    assert_close(oracle, out.cpu().numpy(), ref, _id(case))
