@@ -320,6 +320,8 @@ def main():
     ap.add_argument("--layers", type=int, default=8, help="distinct resident weight copies cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=256 GEMM report")
+    ap.add_argument("--no-module-time", action="store_true",
+                    help="skip the eager layer(x) timing (its launches would mix into a kernel trace's averages)")
     ap.add_argument("--small-m", action="store_true",
                     help="also report configs[1] at M = 4, 16 and the configs[2] bit-width sweep (not part of `value`)")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
@@ -382,11 +384,12 @@ def main():
         b = algorithmic_bytes(M, N, K)
         rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
                "TFLOP/s": round(2 * M * N * K / us / 1e6, 3), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
-               "bytes": int(b), "kernel": layers[0][name].func.runtime.description,
-               "module_us": round(module_time_us([layer[name] for layer in layers], acts[K]), 2)}
+               "bytes": int(b), "kernel": layers[0][name].func.runtime.description}
+        if not args.no_module_time:
+            rec["module_us"] = round(module_time_us([layer[name] for layer in layers], acts[K]), 2)
         shapes_report.append(rec)
         log(f"[bench] {name:8s} N={N:6d} K={K:6d}  {us:7.2f} us  {rec['GB/s']:7.1f} GB/s  {100 * rec['hbm_frac']:5.1f}% of HBM peak"
-            f"  (eager layer(x): {rec['module_us']:.2f} us per call)")
+            + (f"  (eager layer(x): {rec['module_us']:.2f} us per call)" if "module_us" in rec else ""))
         if name == DOMINANT:
             dominant = rec
 
