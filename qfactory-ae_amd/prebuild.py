@@ -165,7 +165,7 @@ def smoke_cases():
 
 def misc_test_cases():
     """Other modules the GPU tests construct (row-count dispatch, argument checks)."""
-    return ([_case(M, 96, 512, 4, 128) for M in (1, 2, 3, 6)] + [_case(1, 64, 256, 4, 128)]
+    return ([_case(M, 96, 512, 4, 128) for M in (1, 2, 3, 6)] + [_case(1, 64, 256, 4, 128), _case(1, 96, 512, 4, -1)]
             + [_case(1, 384, 1024, 4, 128), _case(16, 384, 1024, 4, 128), _case(64, 384, 1024, 4, 128)])
 
 

@@ -95,6 +95,8 @@ class GPTQLinear(torch.nn.Module):
 
     def forward(self, x: torch.Tensor):
         output = torch.empty(x.shape[0], self.w.shape[0], dtype=x.dtype, device=x.device)
+        if x.shape[0] == 0:
+            return output                                  # no rows: nothing to launch
         func = self.func_for(x.shape[0], x.dtype)
         if self.z is not None:
             rc = func(x, self.w, output, self.s, self.z)
@@ -125,6 +127,8 @@ class GPTQLinear(torch.nn.Module):
         the same bits.  Not in the reference, whose end-to-end runs leave the step to vLLM's ``SiluAndMul``."""
         m, half = x.shape[0], self.out_features // 2
         output = torch.empty(m, half, dtype=x.dtype, device=x.device)
+        if m == 0:
+            return output
         if not self.fuses_silu_mul(m, x.dtype):
             from . import native
             return native.silu_mul(self.forward(x), output)
@@ -175,6 +179,8 @@ class GEMVLinear(torch.nn.Module):
 
     def forward(self, x: torch.Tensor):
         output = torch.empty(x.shape[0], self.w.shape[0], dtype=x.dtype, device=x.device)
+        if x.shape[0] == 0:
+            return output
         rc = self.func_for(x.dtype)(x, self.w, output)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")

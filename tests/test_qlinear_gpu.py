@@ -115,6 +115,18 @@ def test_forward_with_other_row_counts_than_constructed(qf, oracle):
         assert_close(oracle, out.cpu().numpy(), ref, f"M={M}")
 
 
+def test_forward_without_rows_returns_an_empty_result(qf):
+    N, K, nbits, GS = 96, 512, 4, 128
+    _, weight, scale, zero = make_problem(5, 1, N, K, nbits, GS)
+    layer = qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
+    for dtype in (torch.float16, torch.bfloat16):
+        out = layer(torch.empty(0, K, dtype=dtype, device="cuda"))
+        assert out.shape == (0, N) and out.dtype == dtype
+    assert layer.forward_silu_mul(torch.empty(0, K, dtype=torch.float16, device="cuda")).shape == (0, N // 2)
+    plain = qf.init(1, K, N, nbits, weight.cuda(), compile_flags={"enable_schedule": False, "enable_lower": False})
+    assert plain(torch.empty(0, K, dtype=torch.float16, device="cuda")).shape == (0, N)
+
+
 def test_closure_rejects_bad_tensors(qf):
     N, K, nbits, GS = 64, 256, 4, 128
     A, weight, scale, zero = make_problem(6, 1, N, K, nbits, GS)
