@@ -110,8 +110,10 @@ class QFactoryLinearMethod(LinearMethodBase):
         cfg = self.quant_config
         input_size = layer.qweight.shape[0] * cfg.pack_factor
         output_size = layer.qweight.shape[1]
+        # the loaded g_idx decides: only the trivial k // group_size is computed correctly here, anything else
+        # (an activation-reordered, desc_act checkpoint) raises NotImplementedError instead of loading
         weight, scale, zero = gptq_to_qlinear_inputs(layer.qweight.data, layer.qzeros.data, layer.scales.data,
-                                                     cfg.weight_bits, cfg.group_size, g_idx=None)
+                                                     cfg.weight_bits, cfg.group_size, g_idx=layer.g_idx.data)
         layer.qlinear = QLinear.init(
             1, input_size, output_size, cfg.weight_bits, weight, cfg.group_size, scale, zero,
             compile_flags={"enable_transform": False, "enable_schedule": False, "enable_lower": False})

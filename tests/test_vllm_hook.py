@@ -77,6 +77,25 @@ def test_gptq_word_format_round_trip(bits):
         gf.check_trivial_g_idx(torch.arange(K, dtype=torch.int32).flip(0) // GS, GS)
 
 
+def test_activation_reordered_checkpoint_is_rejected_at_load(plugin):
+    """A desc_act checkpoint (g_idx is a permutation of the groups) must not load: the kernels assume group
+    k // group_size.  The check runs on the loaded ``layer.g_idx`` before any device work."""
+    from qfactory.integrations import gptq_format as gf
+    g = torch.Generator().manual_seed(9)
+    K, N, GS, bits = 512, 64, 128, 4
+    cfg = plugin.QFactoryConfig(bits, GS)
+    method = cfg.get_quant_method(vllm_stub.LinearBase(), "o_proj")
+    layer = vllm_stub.LinearBase()
+    method.create_weights(layer, K, [N], K, N, torch.float16, weight_loader=None)
+    layer.qweight.data.copy_(gf.pack_qweight(torch.randint(0, 16, (K, N), dtype=torch.int32, generator=g), bits))
+    layer.qzeros.data.copy_(gf.pack_qzeros(torch.randint(0, 16, (K // GS, N), dtype=torch.int32, generator=g), bits))
+    layer.scales.data.fill_(0.01)
+    layer.g_idx.data.copy_((torch.arange(K, dtype=torch.int32) // GS)[torch.randperm(K, generator=g)])
+    with pytest.raises(NotImplementedError):
+        method.process_weights_after_loading(layer)
+    assert layer.qweight is not None                       # nothing was torn down
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("rows", [1, 40])
 def test_loaded_layer_matches_oracle(plugin, oracle, rows):
@@ -94,6 +113,7 @@ def test_loaded_layer_matches_oracle(plugin, oracle, rows):
     layer.qweight.data.copy_(gf.pack_qweight(W, bits))
     layer.qzeros.data.copy_(gf.pack_qzeros(Z, bits))
     layer.scales.data.copy_(S)
+    layer.g_idx.data.copy_(torch.arange(K, dtype=torch.int32) // GS)
     method.process_weights_after_loading(layer)
     assert layer.qweight is None and layer.qzeros is None
     x = torch.randn(2, rows // 2 if rows > 1 else 1, K, generator=g).to(torch.float16)[: (2 if rows > 1 else 1)]
