@@ -153,6 +153,19 @@ def smem_quant_cases():
     return [dict(c, smem_quant=True) for c in cases]
 
 
+def eager_cases():
+    """The other decode strategy of the kernels that have two (``transform()``: the dot2 GEMV in packed fp16, the
+    A-stationary and streaming matrix-core kernels with every field scaled before the contraction) where the
+    default is the deferred one: every bit width, symmetric and not, ragged shapes, the SwiGLU epilogue."""
+    cases = [_case(1, 100, 1024), _case(2, 77, 512, 3, 64, True), _case(1, 130, 2048, 8, 128, True),
+             _case(1, 48, 4096, 2, 128), _case(4, 50, 512, 4, 16), _case(1, 4096, 4096), _case(1, 256, 11008),
+             _case(16, 384, 1024, 4, 128), _case(12, 100, 2048, 3, 256), _case(16, 100, 4096, 2, 256, True),     # A-stationary
+             _case(7, 1000, 2048, 8, 128),
+             _case(5, 100, 11008, 4, 128), _case(16, 272, 14336, 4, 256), _case(9, 64, 8192, 8, 128, True),     # streaming skinny
+             _case(12, 48, 14336, 2, 256)]
+    return [dict(c, decode="eager") for c in cases]
+
+
 def bench_cases():
     cases = [_case(1, N, K) for N, K in LLAMA2_7B]
     cases += [_case(1, N, K) for N, K in LLAMA3_70B]          # bench.py --small-m
@@ -199,14 +212,33 @@ def search_cases():
     return [_case(1, 64, 256, 4, 128)]
 
 
-def all_cases():
+def drain_cases(base=None):
+    """One problem (the cheapest) per distinct GEMM tiling x bit width among the problems above: the GEMM kernel
+    with counted waits is compared bit for bit with its full-drain build (tests/test_gemm_drain_gpu.py)."""
+    best = {}
+    for c in (base if base is not None else all_cases(with_drain=False)):
+        if c.get("act") or c.get("smem_quant") or c.get("epilogue") or c.get("drain") or c["GS"] == -1:
+            continue
+        for q in qfuncs_of(c):
+            if getattr(q, "regime", None) != "gemm":
+                continue
+            key = (tuple(sorted(q.tiling_configs.items())), c["NBITS"])
+            cost = c["M"] * c["N"] * c["K"]
+            if key not in best or cost < best[key][0]:
+                best[key] = (cost, c)
+    return [dict(c, drain=True) for _, c in sorted(best.values(), key=lambda t: t[0])]
+
+
+def all_cases(with_drain=True):
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases() + bf16_cases() + smem_quant_cases()):
+              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
             out.append(c)
+    if with_drain:
+        out += drain_cases(out)
     return out
 
 
@@ -232,12 +264,34 @@ def qfuncs_of(case):
                      torch.float16, torch.int8, case["GS"])
         op.init_qfuncs()
         qfuncs += [q.clone(smem_quant=True) for q in op.qfuncs]
+    if case.get("decode"):
+        eager = [q.clone(decode_strategy=case["decode"]) for q in qfuncs if case["decode"] in q.decode_strategies()
+                 and q.decode_strategy != case["decode"]]
+        assert eager, f"{case}: the kernel has no second decode strategy"
+        qfuncs += eager
+    if case.get("drain"):
+        qfuncs += [q.clone(defines={"QF_GEMM_FULL_DRAIN": 1}) for q in list(qfuncs) if q.regime == "gemm"]
     if case.get("epilogue") == "silu_mul":
         op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
                      torch.float16, torch.int8, case["GS"], output_epilogue="silu_mul")
         op.init_qfuncs()
         qfuncs += op.qfuncs
     return qfuncs
+
+
+def prune(keep):
+    """Remove cached objects of the in-tree cache that no listed problem compiles to any more (older header
+    or generator versions): the cache travels with the tree, stale objects are dead weight."""
+    import shutil
+    root = os.path.join(os.environ["QFACTORY_CACHE_DIR"], "runtimes")
+    removed = 0
+    for name in (os.listdir(root) if os.path.isdir(root) else []):
+        path = os.path.join(root, name)
+        if path not in keep:
+            shutil.rmtree(path, ignore_errors=True)
+            removed += 1
+    shutil.rmtree(os.path.join(os.environ["QFACTORY_CACHE_DIR"], "tmp"), ignore_errors=True)
+    return removed
 
 
 def prebuild(cases=None, force=False, workers=None, verbose=True):
@@ -257,6 +311,10 @@ def prebuild(cases=None, force=False, workers=None, verbose=True):
                     if path not in seen:
                         seen.add(path)
                         qfuncs.append(cand)
+    if cases is None and os.path.abspath(os.environ["QFACTORY_CACHE_DIR"]) == os.path.join(HERE, "jit_cache"):
+        removed = prune(seen)
+        if verbose and removed:
+            print(f"[prebuild] removed {removed} stale objects", flush=True)
     workers = workers or min(16, os.cpu_count() or 4)
     done = 0
     with ThreadPoolExecutor(max_workers=workers) as pool:

@@ -22,7 +22,7 @@ from itertools import chain
 import torch
 
 from .qtile import QTile, SymQTile, AsymQTile
-from .qfunc import QMatmulQFunc, MatmulQFunc
+from .qfunc import QMatmulQFunc, MatmulQFunc, apply_config
 from ..convert import weight_row_bytes, zero_row_bytes
 from ..jit import jit
 
@@ -141,10 +141,7 @@ class QMatmul:
         predefined = _load_predefined(shape)
         if predefined is not None:
             logger.info(f"[Profile] Using predefined config for {shape}")
-            qfunc = self.qfuncs[0]
-            for key, value in predefined.items():
-                setattr(qfunc, key, value)
-            self.qfuncs = [qfunc]
+            self.qfuncs = [apply_config(self.qfuncs[0], predefined)]
         else:
             if enable_transform:
                 self.qfuncs = list(chain.from_iterable(q.transform() for q in self.qfuncs))
@@ -172,27 +169,29 @@ class QMatmul:
             require_gpu()
             zero_empty = torch.empty(z_shape, dtype=torch.int8, device="cuda")
 
-        def inner(activation, weight, output, scale, zero):
-            # tensor shape check
-            assert activation.shape[1] == k
+        def check_packed(weight, scale, zero):
             assert weight.shape == w_shape
-            assert output.shape[1] == n_out
-            assert activation.shape[0] == output.shape[0]
             assert scale.shape == s_shape
             assert zero.shape == z_shape
-            # tensor dtype check
-            assert activation.dtype == dtype_a
             assert weight.dtype == torch.int8
-            assert output.dtype == dtype_a
             assert scale.dtype == torch.float16
             assert zero.dtype == torch.int8
-            # contiguous check
-            assert activation.is_contiguous()
             assert weight.is_contiguous()
-            assert output.is_contiguous()
             assert scale.is_contiguous()
             assert zero.is_contiguous()
-            assert activation.is_cuda and weight.is_cuda and output.is_cuda
+            assert weight.is_cuda and scale.is_cuda and zero.is_cuda
+
+        def inner(activation, weight, output, scale, zero):
+            # tensor shape / dtype / contiguity checks (reference: matmul.py:124-144)
+            assert activation.shape[1] == k
+            assert output.shape[1] == n_out
+            assert activation.shape[0] == output.shape[0]
+            assert activation.dtype == dtype_a
+            assert output.dtype == dtype_a
+            assert activation.is_contiguous()
+            assert output.is_contiguous()
+            assert activation.is_cuda and output.is_cuda
+            check_packed(weight, scale, zero)
             if convert_first:
                 activation = native.bf16_to_f16(activation)
             return runtime.run_raw(
@@ -203,8 +202,38 @@ class QMatmul:
         def inner_sym(activation, weight, output, scale):
             return inner(activation, weight, output, scale, zero_empty)
 
+        def bind(weight, scale, zero=None):
+            """The packed tensors of a layer never change between calls: validate them once and return
+            ``launch(activation, output) -> rc`` that checks only what changes per call (the activation and the
+            output) and passes raw addresses.  The bound tensors must stay alive and in place; rebinding is
+            the caller's business when it replaces them."""
+            if zero is None:
+                zero = zero_empty
+            check_packed(weight, scale, zero)
+            device_index = weight.device.index
+            fn = runtime._launch_m if runtime._launch_m is not None else runtime.lib.launch
+            rc, rc_ref = runtime._rc, runtime._rc_ref
+            wp, sp, zp = weight.data_ptr(), scale.data_ptr(), zero.data_ptr()
+            get_stream = _get_raw_stream
+
+            def launch(activation, output):
+                m = activation.shape[0]
+                if (activation.dim() != 2 or activation.shape[1] != k or output.shape != (m, n_out)
+                        or activation.dtype != dtype_a or output.dtype != dtype_a
+                        or not activation.is_contiguous() or not output.is_contiguous()
+                        or activation.device.index != device_index or output.device.index != device_index):
+                    return inner(activation, weight, output, scale, zero)       # the full checks name the problem
+                if convert_first:
+                    activation = native.bf16_to_f16(activation)
+                stream = get_stream(device_index) if get_stream is not None else _raw_stream(activation)
+                fn(m, activation.data_ptr(), wp, output.data_ptr(), sp, zp, stream, rc_ref)
+                return rc.value
+
+            return launch
+
         func = inner_sym if self.sym else inner
         func.runtime = runtime
+        func.bind = bind
         return func
 
 
@@ -246,10 +275,7 @@ class Matmul:
         predefined = _load_predefined(shape)
         if predefined is not None:
             logger.info(f"[Profile] Using predefined config for {shape}")
-            qfunc = self.qfuncs[0]
-            for key, value in predefined.items():
-                setattr(qfunc, key, value)
-            self.qfuncs = [qfunc]
+            self.qfuncs = [apply_config(self.qfuncs[0], predefined)]
         else:
             if enable_schedule:
                 self.qfuncs = list(chain.from_iterable(q.schedule() for q in self.qfuncs))
@@ -280,5 +306,28 @@ class Matmul:
             return runtime.run_raw(m, (activation.data_ptr(), weight.data_ptr(), output.data_ptr()),
                                    _raw_stream(activation))
 
+        def bind(weight):
+            """Validate the layer's packed weight once; ``launch(activation, output) -> rc`` then checks only the
+            two tensors that change per call (see ``QMatmul``'s closure)."""
+            assert weight.shape == w_shape and weight.dtype == torch.int8 and weight.is_contiguous() and weight.is_cuda
+            device_index = weight.device.index
+            fn, rc, rc_ref = runtime.lib.launch, runtime._rc, runtime._rc_ref
+            wp = weight.data_ptr()
+            get_stream = _get_raw_stream
+
+            def launch(activation, output):
+                m = activation.shape[0]
+                if (activation.dim() != 2 or activation.shape[1] != k or output.shape != (m, n)
+                        or activation.dtype != dtype_a or output.dtype != dtype_a
+                        or not activation.is_contiguous() or not output.is_contiguous()
+                        or activation.device.index != device_index or output.device.index != device_index):
+                    return inner(activation, weight, output)
+                stream = get_stream(device_index) if get_stream is not None else _raw_stream(activation)
+                fn(m, activation.data_ptr(), wp, output.data_ptr(), stream, rc_ref)
+                return rc.value
+
+            return launch
+
         inner.runtime = runtime
+        inner.bind = bind
         return inner

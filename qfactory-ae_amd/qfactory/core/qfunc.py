@@ -31,6 +31,30 @@ Python2CppTypes = {  # python-side type -> (type in the C signature, type used i
 }
 
 
+# Attributes of a QFunc that a tuned-config JSON ($QFACTORY_CONFIG) may set: the reference's file sets attributes
+# verbatim (qfactory/core/matmul.py:76-77); here anything outside this list is an error, so a config file can choose
+# among valid specialisations but cannot inject preprocessor definitions or other state.
+CONFIG_ATTRIBUTES = ("regime", "parallel_strategy", "tiling_configs", "decode_strategy",
+                     "l2cache_a", "l2cache_b", "smem_quant")
+
+# Preprocessor knobs of the kernel headers that change how a kernel is scheduled, never what it computes; the only
+# names `QFunc.defines` may hold.  (The headers' QF_*_EXPERIMENT timing knobs give wrong results and refuse to
+# compile unless the translation unit itself asks for them; the generator cannot.)
+TUNING_DEFINES = ("QF_FUSED_AND_OR", "QF_SCHED_FENCE_MODE", "QF_WIDE_HOLDERS", "QF_GEMV_A_FIRST",
+                  "QF_GEMV_WAVES_PER_EU", "QF_MGEMV_SB", "QF_GEMM_FULL_DRAIN")
+
+
+def apply_config(qfunc, entry):
+    """Set the attributes of a tuned-config entry on ``qfunc``; unknown names raise."""
+    for key, value in entry.items():
+        if key not in CONFIG_ATTRIBUTES:
+            raise ValueError(f"config attribute {key!r} is not one of {CONFIG_ATTRIBUTES}")
+        if key == "regime" and value != qfunc.regime:
+            raise ValueError(f"config entry is for the {value!r} kernel family, the problem runs on {qfunc.regime!r}")
+        setattr(qfunc, key, value)
+    return qfunc
+
+
 class QFunc:
     regime = "gemv"
 
@@ -85,16 +109,16 @@ class QMatmulQFunc(QFunc):
         self.regime = tiling.regime_for(m, k, qtile_b.nbits, gs, n)
         self.parallel_strategy = "row"          # teams sweep rows, K split over lanes and waves
         self.tiling_configs = self.default_tiling(self.regime)
-        # Computation transformation: "deferred" applies scale and zero once per chunk / group in
-        # fp32 after the integer dot product; "eager" dequantises every element to fp16 first.
-        self.decode_strategy = "deferred" if self.regime == "gemv" else "eager"
+        # Computation transformation (reference: qfunc.py:85-91): "deferred" applies scale and zero once per
+        # chunk / group in fp32 after the integer dot product; "eager" dequantises every element to fp16 first.
+        self._gs = gs
+        self.decode_strategy = self.decode_strategies()[0]
         # Load-path scheduling
         self.l2cache_a = True                   # activations: normal (cached) loads
         self.l2cache_b = False                  # weights: streaming (non-temporal) loads
         self.smem_quant = False                 # scales / zero-points of a block's rows through LDS (dot2 GEMV kernel);
         #                                         measured slower at M = 1 (a barrier in a one-shot block), 3 % faster at M = 2
         self.base_impl = base_impl
-        self._gs = gs
         # "silu_mul": the weight is a fused gate+up projection and the kernel writes the (M, N/2) SwiGLU activation
         # fp16(silu(gate)) * up instead of the (M, N) projection (the kernels for M <= 32; not in the reference)
         self.output_epilogue = "none"
@@ -139,10 +163,25 @@ class QMatmulQFunc(QFunc):
         ]
 
     # -- search space -------------------------------------------------------------------------
+    def decode_strategies(self):
+        """Decode strategies this problem's kernel family implements, its default first.
+
+        * dot2 GEMV: deferred (default) and eager in packed fp16.
+        * A-stationary and streaming matrix-core kernels: deferred where a chunk of 512/b fields lies inside one
+          group (the group sum is formed on the matrix core and scaled once in fp32), eager always.
+        * GEMM and the generic matrix-core kernel: eager only (dequantised fp16 fragments feed the MFMA)."""
+        nbits, gs = self.qtile_b.nbits, self._gs
+        chunk = 4 * (128 // tiling.plane_bits(nbits))
+        if self.regime == "gemv":
+            return ["deferred", "eager"]
+        if self.regime == "mgemv":
+            return ["deferred", "eager"] if gs % chunk == 0 else ["eager"]
+        if self.regime == "skinny":
+            return ["deferred", "eager"] if (gs >= 2 * chunk or gs == chunk) else ["eager"]
+        return ["eager"]
+
     def transform(self) -> List[QFunc]:
-        # one decode strategy per kernel family today: the dot2 GEMV defers scale/zero to fp32,
-        # the matrix-core kernels dequantise eagerly (bit-identical weights to the reference)
-        return [self.clone()]
+        return [self.clone(decode_strategy=d) for d in self.decode_strategies()]
 
     def schedule(self) -> List[QFunc]:
         smem = (False, True) if self.regime == "gemv" and self.output_epilogue == "none" else (False,)
@@ -169,6 +208,14 @@ class QMatmulQFunc(QFunc):
         b = lambda x: "true" if x else "false"
         code = "// QFactory-HIP generated translation unit\n\n"
         defines = dict(getattr(self, "defines", {}))                        # kernel-header tuning knobs
+        for name in defines:
+            if name not in TUNING_DEFINES:
+                raise ValueError(f"{name} is not a tuning knob of the kernel headers ({', '.join(TUNING_DEFINES)})")
+        if self.decode_strategy not in self.decode_strategies():
+            raise ValueError(f"decode_strategy {self.decode_strategy!r} is not implemented by the {self.regime!r} kernel "
+                             f"for {p['NBITS']}-bit weights in groups of {p['GS']} (available: {self.decode_strategies()})")
+        if self.decode_strategy == "eager" and self.regime in ("gemv", "mgemv", "skinny"):
+            defines[{"gemv": "QF_GEMV_EAGER", "mgemv": "QF_MGEMV_EAGER", "skinny": "QF_SKINNY_EAGER"}[self.regime]] = 1
         if self.regime in ("gemm", "mgemv", "skinny"):
             # the matrix-core kernels expose their dequantisation's vector-instruction issue and have
             # registers to spare: the one-instruction mask-and-merge decode pays there (2 - 7 %
@@ -225,7 +272,8 @@ class QMatmulQFunc(QFunc):
                 + ("epilogue=silu_mul " if self.output_epilogue == "silu_mul" else "")
                 + ("smem_quant=1 " if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none" else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
-        code += f'extern "C" const char* qf_describe() {{ return "{desc}"; }}\n'
+        wait_desc = " QF_GEMM_WAIT_DESC" if self.regime == "gemm" else ""    # string literal from the header: counted / drain
+        code += f'extern "C" const char* qf_describe() {{ return "{desc}"{wait_desc}; }}\n'
         return code
 
 
@@ -241,6 +289,7 @@ class MatmulQFunc(QFunc):
         self.regime = "gemv"
         self.parallel_strategy = "row"
         self.tiling_configs = tiling.gemv_tiling(1, qtile_b.shape[0], qtile_b.shape[1], qtile_b.nbits, None)
+        self.decode_strategy = "deferred"       # raw fields: there is no scale or zero-point to apply early
         self.l2cache_a = True
         self.l2cache_b = False
         assert qtile_a.dtype in (torch.float16, torch.bfloat16), f"Data type {qtile_a.dtype} is not supported for A"
@@ -272,6 +321,9 @@ class MatmulQFunc(QFunc):
         p = self.problem
         t = self.tiling_configs
         b = lambda x: "true" if x else "false"
+        if self.decode_strategy != "deferred":
+            raise ValueError(f"decode_strategy {self.decode_strategy!r}: the group_size == -1 kernel has no scale or "
+                             "zero-point to apply early (available: ['deferred'])")
         code = "// QFactory-HIP generated translation unit\n\n"
         if self.act_dtype == torch.bfloat16:
             code += "#define QF_IN_BF16 1\n#define QF_OUT_BF16 1\n"

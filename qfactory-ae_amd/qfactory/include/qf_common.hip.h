@@ -158,6 +158,7 @@ template <> struct Decode<4> {
     static constexpr int NCLS = 2;    // field offsets 0 and 4
     __host__ __device__ static constexpr int cls(int pair) { return pair & 1; }
     __host__ __device__ static constexpr float inv_scale(int c) { return c == 0 ? 1.0f : 0.0625f; }
+    __host__ __device__ static constexpr int shift(int c) { return 4 * c; }     // bit offset o of a class: inv_scale = 2^-o
     __device__ __forceinline__ static void word(uint32_t w, uint32_t (&x)[PAIRS]) {
         const uint32_t w8 = w >> 8;
         const uint32_t mg = magic_register();
@@ -175,6 +176,7 @@ template <> struct Decode<2> {
     __host__ __device__ static constexpr float inv_scale(int c) {
         return c == 0 ? 1.0f : c == 1 ? 0.25f : c == 2 ? 0.0625f : 0.015625f;
     }
+    __host__ __device__ static constexpr int shift(int c) { return 2 * c; }
     __device__ __forceinline__ static void word(uint32_t w, uint32_t (&x)[PAIRS]) {
         const uint32_t w8 = w >> 8;
         const uint32_t mg = magic_register();
@@ -199,6 +201,7 @@ template <> struct Decode<3> {
     static constexpr int NCLS = 4;
     __host__ __device__ static constexpr int cls(int pair) { return pair & 3; }
     __host__ __device__ static constexpr float inv_scale(int c) { return Decode<2>::inv_scale(c); }
+    __host__ __device__ static constexpr int shift(int c) { return 2 * c; }
     template <int R>
     __device__ __forceinline__ static void word(uint32_t w, uint32_t h, uint32_t (&x)[PAIRS]) {
         const uint32_t w8 = w >> 8;
@@ -226,6 +229,7 @@ template <> struct Decode<8> {
     static constexpr int NCLS = 1;
     __host__ __device__ static constexpr int cls(int) { return 0; }
     __host__ __device__ static constexpr float inv_scale(int) { return 1.0f; }
+    __host__ __device__ static constexpr int shift(int) { return 0; }
     __device__ __forceinline__ static void word(uint32_t w, uint32_t (&x)[PAIRS]) {
         // 8-bit fields are stored in natural byte order (PERMUTE_ORDER[8] is the identity):
         // byte-permute (b0, 0x64, b1, 0x64) and (b2, 0x64, b3, 0x64) in one instruction each.

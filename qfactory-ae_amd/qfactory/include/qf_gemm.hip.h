@@ -42,6 +42,22 @@
 #ifndef QF_GEMM_EXPERIMENT
 #define QF_GEMM_EXPERIMENT 0
 #endif
+#if QF_GEMM_EXPERIMENT != 0 && !defined(QF_ALLOW_TIMING_EXPERIMENTS)
+#error "QF_GEMM_EXPERIMENT gives wrong results: timing builds only (define QF_ALLOW_TIMING_EXPERIMENTS)"
+#endif
+
+// 1: the wait in front of the K loop's barrier drains every vector-memory load of the wave (vmcnt(0)) instead of
+// letting the counted younger loads stay in flight.  The counted wait is only right if the compiled code issues
+// exactly the loads `loads_since` counts, in order; the JIT checks that on the generated ISA of every object and
+// falls back to this conservative form when the check fails.
+#ifndef QF_GEMM_FULL_DRAIN
+#define QF_GEMM_FULL_DRAIN 0
+#endif
+#if QF_GEMM_FULL_DRAIN
+#define QF_GEMM_WAIT_DESC " waits=drain"
+#else
+#define QF_GEMM_WAIT_DESC " waits=counted"
+#endif
 
 // 1: block -> tile map that keeps the slabs of one column of tiles together on one XCD (see the
 // kernel), 0: plain blockIdx order.  Measured no faster (358 vs 365 us on 57344 x 8192 at M = 256, slower
@@ -488,7 +504,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         // wave has issued in those iterations (activation tiles and whole supers) may stay in
         // flight.  Loads return in order; what the requesting iteration itself issued next to the
         // request is not counted, wherever the compiler placed it.
-        wait_loads_and_barrier<(QF_GEMM_EXPERIMENT & (8 | 64)) ? 63 : loads_since<C>(s, C::PA - 2), !(QF_GEMM_EXPERIMENT & 16)>();
+        wait_loads_and_barrier<QF_GEMM_FULL_DRAIN ? 0 : ((QF_GEMM_EXPERIMENT & (8 | 64)) ? 63 : loads_since<C>(s, C::PA - 2)), !(QF_GEMM_EXPERIMENT & 16)>();
     };
 
     // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----

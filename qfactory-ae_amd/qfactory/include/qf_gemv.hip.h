@@ -61,8 +61,21 @@ struct GemvCfg {
 
 // Timing experiments (results are wrong when non-zero): bit 0 replaces the decode + dot products by
 // an xor of the loaded words, bit 1 skips the activation loads, bit 2 the scale / zero-point loads.
+// A translation unit that sets it must also define QF_ALLOW_TIMING_EXPERIMENTS; the code generator never does.
 #ifndef QF_GEMV_EXPERIMENT
 #define QF_GEMV_EXPERIMENT 0
+#endif
+#if QF_GEMV_EXPERIMENT != 0 && !defined(QF_ALLOW_TIMING_EXPERIMENTS)
+#error "QF_GEMV_EXPERIMENT gives wrong results: timing builds only (define QF_ALLOW_TIMING_EXPERIMENTS)"
+#endif
+
+// Decode strategy (the reference's search dimension, qfactory/core/qfunc.py:85-91; utils.h:46-62 against :193-213).
+// 0, "deferred": integer dot products per chunk, then s * (sum a*q - Z * sum a) once per chunk in fp32.
+// 1, "eager": every field pair becomes the fp16 weight first -- (x - (1024 + 2^o Z)) * s with packed fp16 adds and
+// multiplies, i.e. 2^o * fp16_rn((q - Z) * s) -- and the dot product runs on those; the 2^-o of a class is applied
+// to its fp32 sum.  Two more packed instructions per pair; no per-chunk activation sums.
+#ifndef QF_GEMV_EAGER
+#define QF_GEMV_EAGER 0
 #endif
 
 #ifndef QF_GEMV_A_FIRST
@@ -110,6 +123,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
     constexpr int NWH = C::NWH;
     constexpr bool SILU = QF_GEMV_GATE_UP_SILU != 0;
+    constexpr bool EAGER = QF_GEMV_EAGER != 0 && C::QPARAM;
     constexpr bool SMEMQ = QF_GEMV_SMEM_QUANT != 0 && C::QPARAM;
     constexpr int SQ_WORDS = SMEMQ ? (C::RPB * C::G * 2 + 3) / 4 : 1;           // 32-bit words of the block's scales
     constexpr int ZQ_WORDS = SMEMQ && !C::SYM ? (C::RPB * C::ZRB + 3) / 4 : 1;  // and of its zero-points
@@ -272,6 +286,25 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 for (int m = 0; m < MT; m++)
 #pragma unroll
                     for (int c2 = 0; c2 < NCLS; c2++) acc[m][c2] = 0.0f;
+                uint32_t sbits = 0x3C00u, zint = 0u;               // scale (fp16 bits) and zero-point of this chunk's group
+                if constexpr (C::QPARAM) {
+                    const int brow = team * C::RPT + step * U + u;            // row inside the block
+                    if constexpr (SMEMQ) sbits = reinterpret_cast<const uint16_t*>(sq_s)[brow * C::G + goff[it]];
+                    else sbits = (uint16_t)st.s[u][it];
+                    if constexpr (C::SYM) {
+                        zint = 1u << (C::NBITS - 1);
+                    } else {
+                        const uint32_t zbyte = SMEMQ ? reinterpret_cast<const uint8_t*>(sq_z)[brow * C::ZRB + goff[it] / P8] : st.z[u][it];
+                        zint = (zbyte >> ((goff[it] % P8) * C::ZFB)) & ZMASK;
+                    }
+                }
+                // eager: per class the fp16 pair -(1024 + 2^o Z) (exact: below 2048) and the scale pair
+                f16x2 off[NCLS];
+                const f16x2 s2 = as_f16x2(sbits * 0x00010001u);
+                if constexpr (EAGER) {
+#pragma unroll
+                    for (int c2 = 0; c2 < NCLS; c2++) off[c2] = as_f16x2((0xE400u + (zint << D::shift(c2))) * 0x00010001u);
+                }
                 if constexpr ((QF_GEMV_EXPERIMENT & 1) != 0) {
                     uint32_t t = 0;
                     for (int j = 0; j < NW; j++) t ^= st.w[u][it][j];
@@ -287,35 +320,31 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                         D::word(st.w[u][it][j], x);
                     }
 #pragma unroll
-                    for (int p = 0; p < PAIRS; p++)
+                    for (int p = 0; p < PAIRS; p++) {
+                        f16x2 wv = as_f16x2(x[p]);
+                        if constexpr (EAGER) wv = (wv + off[D::cls(p)]) * s2;     // 2^o * fp16((q - Z) * s)
 #pragma unroll
                         for (int m = 0; m < MT; m++)
                             acc[m][D::cls(p)] = __builtin_amdgcn_fdot2(
-                                as_f16x2(a[m][it][j * PAIRS + p]), as_f16x2(x[p]), acc[m][D::cls(p)], false);
-                }
-                float sc = 1.0f, zf = 0.0f;
-                if constexpr (C::QPARAM) {
-                    const int brow = team * C::RPT + step * U + u;            // row inside the block
-                    if constexpr (SMEMQ) sc = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(sq_s)[brow * C::G + goff[it]]);
-                    else sc = f16_bits_to_f32((uint16_t)st.s[u][it]);
-                    if constexpr (C::SYM) {
-                        zf = (float)(1 << (C::NBITS - 1));
-                    } else {
-                        const uint32_t zbyte = SMEMQ ? reinterpret_cast<const uint8_t*>(sq_z)[brow * C::ZRB + goff[it] / P8] : st.z[u][it];
-                        zf = (float)((zbyte >> ((goff[it] % P8) * C::ZFB)) & ZMASK);
+                                as_f16x2(a[m][it][j * PAIRS + p]), wv, acc[m][D::cls(p)], false);
                     }
                 }
+                const float sc = f16_bits_to_f32((uint16_t)sbits), zf = (float)zint;
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     float t = acc[m][0];
 #pragma unroll
                     for (int c2 = 1; c2 < NCLS; c2++) t = __builtin_fmaf(acc[m][c2], D::inv_scale(c2), t);
-                    t -= c1[m][it];                              // = sum a*q over the chunk
-                    if constexpr (C::QPARAM) {
-                        t = __builtin_fmaf(-zf, sa[m][it], t);   // sum a*(q - Z)
-                        part[u * MT + m] = __builtin_fmaf(sc, t, part[u * MT + m]);
+                    if constexpr (EAGER) {
+                        part[u * MT + m] += t;                   // the weights were dequantised before the dot product
                     } else {
-                        part[u * MT + m] += t;
+                        t -= c1[m][it];                          // = sum a*q over the chunk
+                        if constexpr (C::QPARAM) {
+                            t = __builtin_fmaf(-zf, sa[m][it], t);   // sum a*(q - Z)
+                            part[u * MT + m] = __builtin_fmaf(sc, t, part[u * MT + m]);
+                        } else {
+                            part[u * MT + m] += t;
+                        }
                     }
                 }
             }

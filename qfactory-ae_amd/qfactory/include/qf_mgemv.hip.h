@@ -42,6 +42,16 @@
 #ifndef QF_MGEMV_EXPERIMENT
 #define QF_MGEMV_EXPERIMENT 0
 #endif
+#if QF_MGEMV_EXPERIMENT != 0 && !defined(QF_ALLOW_TIMING_EXPERIMENTS)
+#error "QF_MGEMV_EXPERIMENT gives wrong results: timing builds only (define QF_ALLOW_TIMING_EXPERIMENTS)"
+#endif
+
+// Decode strategy (the reference's search dimension, qfactory/core/qfunc.py:85-91).  0: "deferred" wherever a chunk
+// lies inside one group (integer sums on the matrix core, one fp32 scale per chunk), "eager" elsewhere.
+// 1: "eager" everywhere -- every field becomes fp16_rn((q - Z) * s) before the contraction.
+#ifndef QF_MGEMV_EAGER
+#define QF_MGEMV_EAGER 0
+#endif
 
 namespace qf {
 
@@ -87,7 +97,7 @@ struct MGemvCfg {
     static constexpr int G = K / GS;
     static constexpr int ZRB = G * ZFB / 8;
     static constexpr int HI_OFF = K / 4;           // byte offset of the 1-bit plane in a 3-bit row
-    static constexpr bool DEFERRED = (GS % CHUNK == 0);      // a chunk lies inside one group
+    static constexpr bool DEFERRED = (GS % CHUNK == 0) && !QF_MGEMV_EAGER;   // a chunk lies inside one group
     static constexpr int LPR = CH * 4;             // lanes covering one row's K-slice (CH*64 bytes)
     static constexpr int RPI = 64 / LPR;           // rows per coalesced weight load
     // groups and zero-point bytes of one row inside a wave's K-slice

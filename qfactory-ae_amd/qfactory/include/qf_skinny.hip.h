@@ -43,6 +43,16 @@
 #ifndef QF_SKINNY_EXPERIMENT
 #define QF_SKINNY_EXPERIMENT 0
 #endif
+#if QF_SKINNY_EXPERIMENT != 0 && !defined(QF_ALLOW_TIMING_EXPERIMENTS)
+#error "QF_SKINNY_EXPERIMENT gives wrong results: timing builds only (define QF_ALLOW_TIMING_EXPERIMENTS)"
+#endif
+
+// Decode strategy (the reference's search dimension, qfactory/core/qfunc.py:85-91).  0: "deferred" wherever the group
+// geometry allows (integer sums on the matrix core, one fp32 scale per group), 1: "eager" everywhere (scale mode 2
+// below: every field becomes fp16_rn((q - Z) * s) before the contraction).
+#ifndef QF_SKINNY_EAGER
+#define QF_SKINNY_EAGER 0
+#endif
 
 namespace qf {
 
@@ -95,7 +105,7 @@ struct SkinnyCfg {
     static constexpr int ZRB = G * NBITS / 8;
     // 0: a step lies inside one group; 1: one group per chunk; 2: groups narrower than a chunk
     // (a lane's 128/NBITS fields still share one): the weights are scaled before the contraction
-    static constexpr int SMODE = GS >= STEPK ? 0 : (GS == CHUNK ? 1 : 2);
+    static constexpr int SMODE = QF_SKINNY_EAGER ? 2 : (GS >= STEPK ? 0 : (GS == CHUNK ? 1 : 2));
     // scales of one row for the wave's SPW steps: SMODE 1 keeps a dword (two groups) per step and
     // fetches VS steps per load; the other modes fetch a half-word per step (and chunk)
     static constexpr int VS = SMODE != 1 ? 1 : ((SPW % 4 == 0 && NSTEP % 4 == 0) ? 4 : ((SPW % 2 == 0 && NSTEP % 2 == 0) ? 2 : 1));

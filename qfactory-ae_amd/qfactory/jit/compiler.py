@@ -17,6 +17,7 @@ import threading
 import uuid
 
 from .runtime import Runtime, RuntimeCache, dump_args
+from .verify import gemm_waits_hold
 
 logger = logging.getLogger(__name__)
 
@@ -43,20 +44,43 @@ def include_dirs():
     return dirs
 
 
-def get_qfactory_version() -> str:
-    """md5 over every header the generated code can include."""
-    with _lock:
-        if "version" in _memo:
-            return _memo["version"]
-    md5 = hashlib.md5()
+_INCLUDE_RE = re.compile(r'^[ \t]*#[ \t]*include[ \t]*"([^"]+)"', re.MULTILINE)
+
+
+def _read_header(name):
+    """(path, text) of a quoted include found in the include directories, or None (a system header)."""
     for d in include_dirs():
-        for root, _, files in sorted(os.walk(d)):
-            for filename in sorted(f for f in files if f.endswith(".h")):
-                with open(os.path.join(root, filename), "rb") as f:
-                    md5.update(f.read())
-    with _lock:
-        _memo["version"] = md5.hexdigest()[0:12]
-        return _memo["version"]
+        path = os.path.join(d, name)
+        if os.path.exists(path):
+            with _lock:
+                hit = _memo.get(("header", path))
+            if hit is None:
+                with open(path) as f:
+                    hit = f.read()
+                with _lock:
+                    _memo[("header", path)] = hit
+            return path, hit
+    return None
+
+
+def get_qfactory_version(code: str = None) -> str:
+    """md5 over the package headers a translation unit includes, directly or through other headers (the
+    reference hashes its whole include directory, compiler.py:16-28; hashing what a unit can see keeps the
+    objects of the other kernel families valid when one header changes).  Without ``code``: every header."""
+    if code is None:
+        code = "".join(f'#include "{f}"\n' for d in include_dirs() for f in sorted(os.listdir(d)) if f.endswith(".h"))
+    seen, queue = {}, [code]
+    while queue:
+        for name in _INCLUDE_RE.findall(queue.pop()):
+            found = _read_header(name)
+            if found is not None and found[0] not in seen:
+                seen[found[0]] = found[1]
+                queue.append(found[1])
+    md5 = hashlib.md5()
+    for path in sorted(seen):
+        md5.update(os.path.basename(path).encode())
+        md5.update(seen[path].encode())
+    return md5.hexdigest()[0:12]
 
 
 def get_hipcc_compiler():
@@ -101,12 +125,14 @@ def compile_flags(arch):
 
 
 class JITCompiler:
+    check_gemm_waits = staticmethod(gemm_waits_hold)
+
     def runtime_path_of(self, qfunc):
         """(runtime directory, source) the given QFunc compiles to, without compiling."""
         code = qfunc.emit()
         arch = os.getenv("QFACTORY_ARCH", DEFAULT_ARCH)
         flags = compile_flags(arch)
-        signature = f"{code}$${get_hipcc_compiler()}$${get_qfactory_version()}$${flags}$${arch}"
+        signature = f"{code}$${get_hipcc_compiler()}$${get_qfactory_version(code)}$${flags}$${arch}"
         runtime_name = f"kernel.{arch}.{hash_to_hex(signature)}"
         return os.path.join(get_cache_dir(), "runtimes", runtime_name), code
 
@@ -133,10 +159,31 @@ class JITCompiler:
         write_file(tmp_dir, src_path, code)
         command = [get_hipcc_compiler()[0], "-x", "hip", src_path, "-o", tmp_so_path, *flags,
                    *[f"-I{d}" for d in include_dirs()]]
+        # GEMM objects wait on counted loads: keep the device ISA of this compile and re-count (verify.py)
+        counted_waits = getattr(qfunc, "regime", None) == "gemm" and "QF_GEMM_FULL_DRAIN 1" not in code
+        work_dir = None
+        if counted_waits:
+            work_dir = os.path.join(tmp_dir, f"temps.{uuid.uuid4()}")
+            os.makedirs(work_dir)
+            command.append("-save-temps")
         logger.info(f"Compiling kernel with command: {' '.join(command)}")
-        proc = subprocess.run(command, capture_output=True, text=True)
-        if proc.returncode != 0:
-            raise RuntimeError(f"hipcc failed for {src_path} (exit {proc.returncode}):\n{proc.stderr[-4000:]}")
+        try:
+            proc = subprocess.run(command, capture_output=True, text=True, cwd=work_dir)
+            if proc.returncode != 0:
+                raise RuntimeError(f"hipcc failed for {src_path} (exit {proc.returncode}):\n{proc.stderr[-4000:]}")
+            if counted_waits:
+                isa = "".join(open(os.path.join(work_dir, f)).read() for f in sorted(os.listdir(work_dir))
+                              if f.endswith(".s") and "amdgcn" in f)
+                ok, detail = self.check_gemm_waits(isa, qfunc.tiling_configs["PA"])
+                if not ok:
+                    logger.warning(f"GEMM object {runtime_path}: {detail}; rebuilding with a full drain per K-iteration")
+                    command = [c for c in command if c != "-save-temps"] + ["-DQF_GEMM_FULL_DRAIN=1"]
+                    proc = subprocess.run(command, capture_output=True, text=True)
+                    if proc.returncode != 0:
+                        raise RuntimeError(f"hipcc failed for {src_path} (exit {proc.returncode}):\n{proc.stderr[-4000:]}")
+        finally:
+            if work_dir is not None:
+                shutil.rmtree(work_dir, ignore_errors=True)
 
         dump_args(qfunc.arg_name_type(), tmp_args_path)
         os.replace(tmp_args_path, args_path)

@@ -69,8 +69,14 @@ class GPTQLinear(torch.nn.Module):
         self.batch_size = batch_size
 
         self._funcs = {}
+        self._launchers = {}            # (rows, dtype) -> launch(activation, output) bound to this layer's packed tensors
         self.func = self._compile(batch_size, self.compile_flags)
         self._funcs[(_m_bucket(batch_size), torch.float16)] = self.func
+
+    def __setattr__(self, name, value):
+        if name in ("w", "s", "z") and getattr(self, "_launchers", None):
+            self._launchers.clear()     # bound launchers hold the addresses of the tensors they were made for
+        super().__setattr__(name, value)
 
     def _compile(self, m, compile_flags, dtype=torch.float16, epilogue="none"):
         matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
@@ -93,18 +99,30 @@ class GPTQLinear(torch.nn.Module):
             func = self._funcs[key] = self._compile(key[0], self.compile_flags, dtype)
         return func
 
-    def forward(self, x: torch.Tensor):
-        output = torch.empty(x.shape[0], self.w.shape[0], dtype=x.dtype, device=x.device)
-        if x.shape[0] == 0:
-            return output                                  # no rows: nothing to launch
-        func = self.func_for(x.shape[0], x.dtype)
-        if self.z is not None:
-            rc = func(x, self.w, output, self.s, self.z)
-        else:
-            rc = func(x, self.w, output, self.s)
+    def _launcher(self, m, dtype):
+        """``launch(x, out)`` for ``m`` rows of ``dtype``: the bucket's closure with this layer's packed tensors
+        validated once and bound (the reference re-checks all five tensors on every call, matmul.py:124-144; the
+        three that belong to the layer cannot change between calls)."""
+        launch = self._launchers[(m, dtype)] = self.func_for(m, dtype).bind(self.w, self.s, self.z)
+        return launch
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor = None):
+        """``(M, K)`` -> ``(M, N)`` in ``x``'s dtype on ``x``'s device.  ``out`` (beyond the reference, which always
+        allocates, qlinear.py:53): a preallocated contiguous ``(M, N)`` tensor to write into, e.g. under HIP-graph
+        capture or in a loop that reuses its buffers."""
+        m, dtype = x.shape[0], x.dtype
+        if out is None:
+            out = torch.empty((m, self.out_features), dtype=dtype, device=x.device)
+        if m == 0:
+            assert out.shape == (0, self.out_features)
+            return out                                     # no rows: nothing to launch
+        launch = self._launchers.get((m, dtype))
+        if launch is None:
+            launch = self._launcher(m, dtype)
+        rc = launch(x, out)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")
-        return output
+        return out
 
 
     def fuses_silu_mul(self, m, dtype=torch.float16):
@@ -130,8 +148,12 @@ class GPTQLinear(torch.nn.Module):
         if m == 0:
             return output
         if not self.fuses_silu_mul(m, x.dtype):
+            y = self.forward(x)
+            if x.dtype != torch.float16:
+                # qf_silu_mul is an fp16 kernel: other activation types take the same expression in torch ops
+                return torch.mul(torch.nn.functional.silu(y[:, :half]), y[:, half:], out=output)
             from . import native
-            return native.silu_mul(self.forward(x), output)
+            return native.silu_mul(y, output)
         key = (_m_bucket(m), x.dtype, "silu_mul")
         func = self._funcs.get(key)
         if func is None:
@@ -166,9 +188,15 @@ class GEMVLinear(torch.nn.Module):
         self.w = w
 
         self.compile_flags = dict(compile_flags)
+        self._launchers = {}
         matmul = Matmul(out_features, in_features, n_bits, torch.float16, torch.int8)
         self.func = matmul.compile_profile(**compile_flags)
         self._funcs = {torch.float16: self.func}
+
+    def __setattr__(self, name, value):
+        if name == "w" and getattr(self, "_launchers", None):
+            self._launchers.clear()
+        super().__setattr__(name, value)
 
     def func_for(self, dtype):
         func = self._funcs.get(dtype)
@@ -177,14 +205,20 @@ class GEMVLinear(torch.nn.Module):
             func = self._funcs[dtype] = matmul.compile_profile(**self.compile_flags)
         return func
 
-    def forward(self, x: torch.Tensor):
-        output = torch.empty(x.shape[0], self.w.shape[0], dtype=x.dtype, device=x.device)
-        if x.shape[0] == 0:
-            return output
-        rc = self.func_for(x.dtype)(x, self.w, output)
+    def forward(self, x: torch.Tensor, out: torch.Tensor = None):
+        m, dtype = x.shape[0], x.dtype
+        if out is None:
+            out = torch.empty((m, self.out_features), dtype=dtype, device=x.device)
+        if m == 0:
+            assert out.shape == (0, self.out_features)
+            return out
+        launch = self._launchers.get(dtype)
+        if launch is None:
+            launch = self._launchers[dtype] = self.func_for(dtype).bind(self.w)
+        rc = launch(x, out)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")
-        return output
+        return out
 
 
 class QLinear():

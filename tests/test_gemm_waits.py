@@ -1,29 +1,33 @@
 """The GEMM kernel waits for its activation tiles with explicit counts of the vector-memory loads that may
 stay in flight.  The counts are computed from how many loads every K-iteration issues, so the compiled code
 must really issue them -- also in the last iterations, whose loads (for 128-byte windows past the end of K)
-are never used and which a compiler may drop or merge when the K loop has a single trip.  Checked here on
-the generated ISA of such a specialisation, without a GPU."""
+are never used and which a compiler may drop or merge when the K loop has a single trip.  The JIT re-counts
+the loads on the ISA of every GEMM object it builds (qfactory/jit/verify.py) and rebuilds with a full drain
+when the count does not hold; checked here without a GPU."""
+import ctypes
 import os
-import re
 import subprocess
 
 import pytest
 import torch
 
 
+def _gemm_qfunc(M, N, K, nbits, gs):
+    from qfactory.core.qfunc import QMatmulQFunc
+    from qfactory.core.qtile import QTile, SymQTile
+    q = QMatmulQFunc(QTile((M, K), torch.float16, 16), SymQTile((N, K), torch.int8, nbits, (1, gs)), "nt")
+    assert q.regime == "gemm"
+    return q
+
+
 def _isa_of(qfunc, tmp_path):
-    from qfactory.jit.compiler import compile_flags, get_hipcc_compiler
+    from qfactory.jit.compiler import compile_flags, get_hipcc_compiler, include_dirs
     src = tmp_path / "kernel.hip"
     src.write_text(qfunc.emit())
-    flags = compile_flags("gfx950")
-    flags = flags.split() if isinstance(flags, str) else list(flags)
-    flags = [f for f in flags if f not in ("-shared", "-fPIC")]
+    flags = [f for f in compile_flags("gfx950") if f not in ("-shared", "-fPIC")]
     out = tmp_path / "kernel.s"
-    from qfactory.jit import compiler
-    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(compiler.__file__))), "include")
-    abi = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
-    subprocess.run([get_hipcc_compiler()[0], *flags, f"-I{include}", f"-I{abi}", "--cuda-device-only", "-S", str(src), "-o", str(out)],
-                   check=True, capture_output=True)
+    subprocess.run([get_hipcc_compiler()[0], *flags, *[f"-I{d}" for d in include_dirs()], "--cuda-device-only", "-S",
+                    str(src), "-o", str(out)], check=True, capture_output=True)
     return out.read_text()
 
 
@@ -31,26 +35,41 @@ def _isa_of(qfunc, tmp_path):
                                            (256, 57344, 8192, 4, 128), (64, 22016, 4096, 4, 128), (128, 8192, 28672, 4, 128),
                                            (33, 100, 512, 4, 128), (300, 256, 2048, 4, 128), (40, 96, 2048, 8, 32)])
 def test_every_counted_load_is_issued(M, N, K, nbits, gs, tmp_path):
-    from qfactory.core.qfunc import QMatmulQFunc
-    from qfactory.core.qtile import QTile, SymQTile
-    q = QMatmulQFunc(QTile((M, K), torch.float16, 16), SymQTile((N, K), torch.int8, nbits, (1, gs)), "nt")
-    assert q.regime == "gemm"
-    pa = q.tiling_configs["PA"]
-    isa = _isa_of(q, tmp_path)
-    loads_in_segment, segments, checked = 0, [], 0
-    for line in isa.splitlines():
-        line = line.strip()
-        if line.startswith(("global_load", "buffer_load")):
-            loads_in_segment += 1
-        m = re.match(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)", line)
-        if m:                                        # the kernel's explicit wait (with or without a block barrier behind it)
-            allowed = int(m.group(1))
-            segments.append(loads_in_segment)
-            loads_in_segment = 0
-            if allowed == 0:
-                segments = []                        # a full drain (end of the prologue): nothing older is in flight
-            elif len(segments) >= pa - 2:
-                # the loads of the last PA - 2 iterations may stay in flight: they must all exist
-                assert sum(segments[-(pa - 2):]) == allowed, (segments, allowed)
-                checked += 1
-    assert checked >= 2
+    from qfactory.jit.verify import gemm_waits_hold
+    q = _gemm_qfunc(M, N, K, nbits, gs)
+    ok, detail = gemm_waits_hold(_isa_of(q, tmp_path), q.tiling_configs["PA"])
+    assert ok, detail
+
+
+def test_checker_rejects_a_missing_load():
+    from qfactory.jit.verify import gemm_waits_hold
+    body = ["global_load_dwordx4 v[0:3], v4, s[0:1]"] * 3 + ["s_waitcnt vmcnt(3) lgkmcnt(0)"]
+    good = "\n".join(["s_waitcnt vmcnt(0) lgkmcnt(0)"] + body * 4)
+    assert gemm_waits_hold(good, 3)[0]
+    bad = good.replace("global_load_dwordx4 v[0:3], v4, s[0:1]\n", "", 1)          # the compiler dropped one
+    ok, detail = gemm_waits_hold(bad, 3)
+    assert not ok and "allows 3" in detail
+    assert not gemm_waits_hold("s_endpgm", 3)[0]                                    # no counted wait at all
+
+
+def test_jit_falls_back_to_a_full_drain_when_the_count_fails(tmp_path, monkeypatch):
+    """A GEMM object whose ISA fails the re-count is rebuilt with vmcnt(0) waits; the object says which it is."""
+    from qfactory.jit.compiler import JITCompiler
+    monkeypatch.setenv("QFACTORY_CACHE_DIR", str(tmp_path))
+    q = _gemm_qfunc(40, 64, 1024, 4, 128)
+
+    copies = iter(range(10))
+
+    def describe(runtime):
+        # a fresh file name per load: dlopen would hand back the object already loaded under the same path
+        copy = tmp_path / f"copy{next(copies)}.so"
+        copy.write_bytes(open(os.path.join(runtime.path, "kernel.so"), "rb").read())
+        lib = ctypes.CDLL(str(copy))
+        lib.qf_describe.restype = ctypes.c_char_p
+        return lib.qf_describe().decode()
+
+    jit = JITCompiler()
+    assert describe(jit.compile(q, force=True)).endswith("waits=counted")
+    jit.check_gemm_waits = staticmethod(lambda isa, pa: (False, "forced by the test"))
+    assert describe(jit.compile(q, force=True)).endswith("waits=drain")
+    assert not [d for d in os.listdir(tmp_path / "tmp") if d.startswith("temps.")]  # the ISA dump is cleaned up

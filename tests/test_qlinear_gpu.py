@@ -143,6 +143,41 @@ def test_closure_rejects_bad_tensors(qf):
         qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), bias=True)
 
 
+def test_forward_fast_path_checks_what_changes_per_call(qf, oracle):
+    """``forward`` validates the layer's packed tensors once and then only the activation and the output; a bad
+    activation still fails the reference's checks, ``out=`` is written in place, and replacing a packed tensor
+    of the layer rebinds the launch."""
+    N, K, nbits, GS = 96, 512, 4, 128
+    A, weight, scale, zero = make_problem(8, 3, N, K, nbits, GS)
+    layer = qf.init(1, K, N, nbits, weight.cuda(), GS, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
+    plain = qf.init(1, K, N, nbits, weight.cuda(), compile_flags={"enable_schedule": False, "enable_lower": False})
+    x = A.cuda()
+    for mod, ref in ((layer, reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS)),
+                     (plain, reference_output(oracle, A, plain.w, None, None, nbits, -1))):
+        first = mod(x)
+        buf = torch.full((3, N), float("nan"), dtype=torch.float16, device="cuda")
+        assert mod(x, out=buf) is buf and torch.equal(buf, first)
+        assert_close(oracle, buf.cpu().numpy(), ref, "out=")
+        assert torch.equal(mod(x), first)                                  # the cached launcher, second call
+        with pytest.raises(AssertionError):
+            mod(x[:, :256])                                                # K mismatch (and not contiguous)
+        with pytest.raises(AssertionError):
+            mod(x.T.contiguous().T)                                        # right shape, wrong strides
+        with pytest.raises(AssertionError):
+            mod(x, out=torch.empty(3, N + 1, dtype=torch.float16, device="cuda"))
+        with pytest.raises(AssertionError):
+            mod(x, out=torch.empty(3, N, dtype=torch.bfloat16, device="cuda"))
+        with pytest.raises(AssertionError):
+            mod(A)                                                         # a host tensor
+    # replacing a packed tensor of the layer: the next call uses the new one
+    before = layer(x).clone()
+    layer.s = (layer.s * 2).contiguous()
+    torch.cuda.synchronize()
+    after = layer(x)
+    assert not torch.equal(after, before)
+    assert_close(oracle, after.cpu().numpy(), reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS), "rebound")
+
+
 @pytest.mark.parametrize("M", [1, 16, 64])
 def test_reference_launch_symbol_through_plain_ctypes(qf, oracle, M):
     """The reference-shaped entry point `launch(act, weight, out, scale, zero, stream, &rc)` (compile-time
@@ -246,3 +281,35 @@ def test_gemv_with_scales_through_lds(oracle, case):
     assert rc == 0
     ref = reference_output(oracle, A, w, s, z, nbits, GS)
     assert_close(oracle, out.cpu().numpy(), ref, _id(case))
+
+
+@pytest.mark.parametrize("case", prebuild.eager_cases(), ids=_id)
+def test_the_other_decode_strategy(oracle, case):
+    """``transform()`` (the reference's decode-strategy dimension, qfactory/core/qfunc.py:85-91): where a kernel family
+    implements both strategies, the non-default one computes the same linear to the bar."""
+    from qfactory.convert import convert_params
+    from qfactory.core import QMatmul
+    from qfactory.jit import jit
+    from qfactory.qlinear import _m_bucket
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
+    print(f"[case] decode=eager {_id(case)}", flush=True)
+    A, weight, scale, zero = make_problem(777 + N + K + M, M, N, K, nbits, GS, sym)
+    w, s, z = convert_params({"K": K, "N": N, "NBITS": nbits, "GS": GS},
+                             (weight.cuda(), scale.cuda(), None if zero is None else zero.cuda()))
+    op = QMatmul(_m_bucket(M), N, K, nbits, sym, torch.float16, torch.int8, GS)
+    op.init_qfuncs()
+    variants = op.qfuncs[0].transform()
+    assert [v.decode_strategy for v in variants] == ["deferred", "eager"]
+    outs = []
+    for qfunc in variants:
+        func = op._wrap(jit.compile(qfunc), qfunc)
+        assert f"decode={qfunc.decode_strategy}" in func.runtime.description
+        out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        rc = func(A.cuda(), w, out, s) if sym else func(A.cuda(), w, out, s, z)
+        torch.cuda.synchronize()
+        assert rc == 0
+        outs.append(out.cpu().numpy())
+    ref = reference_output(oracle, A, w, s, z, nbits, GS)
+    for out, qfunc in zip(outs, variants):
+        assert_close(oracle, out, ref, f"{_id(case)} decode={qfunc.decode_strategy}")
+    assert not np.array_equal(outs[0], outs[1]) or M * N < 64          # two different computations, not one object twice

@@ -118,3 +118,73 @@ def test_prefill_sizes_use_the_many_rows_model_only_for_several_rounds():
     assert tiling.gemm_tiling(512, 10240, 8192, 4, 128) == {"BM": 128, "NT32": 2, "WN": 4, "WK": 1, "PA": 4}
     # one round of 64 x 128 tiles: the K axis is still split over wave groups
     assert tiling.gemm_tiling(512, 4096, 4096, 4, 128)["WK"] == 2
+
+
+def _qfunc(M, N, K, nbits, gs, sym=False):
+    import torch
+    from qfactory.core.qfunc import QMatmulQFunc
+    from qfactory.core.qtile import QTile, AsymQTile, SymQTile
+    tile = SymQTile if sym else AsymQTile
+    return QMatmulQFunc(QTile((M, K), torch.float16, 16), tile((N, K), torch.int8, nbits, (1, gs)), "nt")
+
+
+@pytest.mark.parametrize("M,N,K,nbits,gs,regime,strategies", [
+    (1, 512, 1024, 4, 128, "gemv", ["deferred", "eager"]),
+    (16, 384, 1024, 4, 128, "mgemv", ["deferred", "eager"]),
+    (16, 384, 1024, 4, 64, "mgemv", ["eager"]),                  # a chunk of 128 fields spans two groups
+    (9, 64, 8192, 8, 128, "skinny", ["deferred", "eager"]),
+    (11, 40, 11008, 8, 32, "skinny", ["eager"]),
+    (64, 384, 1024, 4, 128, "gemm", ["eager"]),
+])
+def test_transform_yields_the_decode_strategies_the_kernel_implements(M, N, K, nbits, gs, regime, strategies):
+    """The reference's transform() yields an eager and a deferred candidate (qfactory/core/qfunc.py:85-91)."""
+    q = _qfunc(M, N, K, nbits, gs)
+    assert q.regime == regime and q.decode_strategy == strategies[0]
+    variants = q.transform()
+    assert [v.decode_strategy for v in variants] == strategies
+    codes = [v.emit() for v in variants]
+    assert len(set(codes)) == len(codes)                                            # really different translation units
+    for v, code in zip(variants, codes):
+        assert f"decode={v.decode_strategy}" in code
+        assert ("_EAGER 1" in code) == (v.decode_strategy == "eager" and regime != "gemm")
+
+
+def test_a_strategy_the_kernel_lacks_is_an_error_not_ignored():
+    q = _qfunc(64, 384, 1024, 4, 128)
+    q.decode_strategy = "deferred"
+    with pytest.raises(ValueError, match="decode_strategy 'deferred' is not implemented by the 'gemm' kernel"):
+        q.emit()
+    q = _qfunc(16, 384, 1024, 4, 64)
+    q.decode_strategy = "deferred"
+    with pytest.raises(ValueError, match="available: \\['eager'\\]"):
+        q.emit()
+
+
+def test_config_file_may_only_set_the_search_attributes(tmp_path, monkeypatch):
+    import json
+    import torch
+    from qfactory.core import QMatmul
+    path = tmp_path / "cfg.json"
+    monkeypatch.setenv("QFACTORY_CONFIG", str(path))
+    path.write_text(json.dumps({"4-1-64-512-128": {"decode_strategy": "eager", "l2cache_b": True}}))
+    op = QMatmul(1, 64, 512, 4, False, torch.float16, torch.int8, 128)
+    func = op.compile_profile()
+    assert "decode=eager" in func.runtime.description and "nt_b=0" in func.runtime.description
+    path.write_text(json.dumps({"4-1-64-512-128": {"defines": {"QF_GEMV_EXPERIMENT": 1}}}))
+    with pytest.raises(ValueError, match="config attribute 'defines'"):
+        QMatmul(1, 64, 512, 4, False, torch.float16, torch.int8, 128).compile_profile()
+    path.write_text(json.dumps({"4-64-64-512-128": {"decode_strategy": "deferred"}}))
+    with pytest.raises(ValueError, match="not implemented by the 'gemm' kernel"):
+        QMatmul(64, 64, 512, 4, False, torch.float16, torch.int8, 128).compile_profile()
+    path.write_text(json.dumps({"4-64-64-512-128": {"regime": "gemv"}}))
+    with pytest.raises(ValueError, match="kernel family"):
+        QMatmul(64, 64, 512, 4, False, torch.float16, torch.int8, 128).compile_profile()
+
+
+def test_timing_experiments_cannot_come_from_the_generator():
+    q = _qfunc(1, 64, 512, 4, 128)
+    q.defines = {"QF_GEMV_EXPERIMENT": 1}
+    with pytest.raises(ValueError, match="not a tuning knob"):
+        q.emit()
+    q.defines = {"QF_GEMV_WAVES_PER_EU": 4}
+    assert "#define QF_GEMV_WAVES_PER_EU 4" in q.emit()
