@@ -41,7 +41,7 @@ CONFIG_ATTRIBUTES = ("regime", "parallel_strategy", "tiling_configs", "decode_st
 # names `QFunc.defines` may hold.  (The headers' QF_*_EXPERIMENT timing knobs give wrong results and refuse to
 # compile unless the translation unit itself asks for them; the generator cannot.)
 TUNING_DEFINES = ("QF_FUSED_AND_OR", "QF_SCHED_FENCE_MODE", "QF_WIDE_HOLDERS", "QF_GEMV_A_FIRST",
-                  "QF_GEMV_WAVES_PER_EU", "QF_MGEMV_SB", "QF_GEMM_FULL_DRAIN")
+                  "QF_GEMV_QUANT_DEDUP", "QF_GEMV_WAVES_PER_EU", "QF_MGEMV_SB", "QF_GEMM_FULL_DRAIN")
 
 
 def apply_config(qfunc, entry):
@@ -224,6 +224,15 @@ class QMatmulQFunc(QFunc):
         if self.regime == "gemv" and p["NBITS"] == 2:
             # sixteen fields per word make the 2-bit GEMV decode-bound: measured 7.6 -> 6.9 us at 8192 x 8192
             defines.setdefault("QF_FUSED_AND_OR", 1)
+        if self.regime == "gemv" and p["NBITS"] == 4 and self.decode_strategy == "deferred" and not self.smem_quant \
+                and tiling.gemv_chunks_per_lane(p["K"], p["NBITS"], t) == 1:
+            # one chunk per lane and row (K <= 4096 x waves): the mask-and-merge decode in one instruction with
+            # compiler-scheduled operands, and one scale / zero-point load per lane and stage after the group's
+            # lanes have added their sums.  Measured against the plain form, cold weights: 12288 x 4096
+            # 6.74 -> 6.47 us, 4096 x 4096 4.00 -> 3.74, 22016 x 4096 10.04 -> 9.86, 8192 x 8192 (eight rows per
+            # stage) 8.85 -> 8.26; two chunks per lane (K = 28672) lose 6 %, K = 11008 is level.
+            defines.setdefault("QF_FUSED_AND_OR", 2)
+            defines.setdefault("QF_GEMV_QUANT_DEDUP", 1)
         if self.act_dtype == torch.bfloat16:
             defines["QF_OUT_BF16"] = 1
             if self.converts_activations:

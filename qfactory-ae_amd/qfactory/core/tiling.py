@@ -145,6 +145,12 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
     return {"MT": mt, "WK": wk, "WN": wn, "U": u, "STEPS": steps, "VB": vb}
 
 
+def gemv_chunks_per_lane(K, nbits, cfg):
+    """IT of qf::GemvCfg: chunks of VB bytes a lane owns per row."""
+    nch = K // elements_per_chunk(nbits, cfg["VB"])
+    return -(-nch // (64 * cfg["WK"]))
+
+
 def gemv_candidates(M, N, K, nbits, group_size):
     """Neighbourhood of the default worth timing on the device (deduplicated, default first)."""
     base = gemv_tiling(M, N, K, nbits, group_size)

@@ -136,7 +136,14 @@ template <int NBITS> struct Decode;
 #endif
 template <uint32_t MASK>
 __device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t magic_vgpr) {
-#if QF_FUSED_AND_OR
+#if QF_FUSED_AND_OR == 2
+    // no instruction is spelled out: the mask is made opaque in a scalar register (the magic pair in a vector
+    // register, magic_register()), so the compiler cannot fold either into a literal and selects v_and_or_b32
+    // itself, and stays free to schedule it
+    uint32_t m = MASK;
+    asm("" : "+s"(m));
+    return (w & m) | magic_vgpr;
+#elif QF_FUSED_AND_OR
     uint32_t r;
     asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(MASK), "v"(magic_vgpr));
     return r;

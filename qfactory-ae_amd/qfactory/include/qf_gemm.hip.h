@@ -437,7 +437,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     //   * tile it+PA is requested into the buffer whose tile every wave has finished reading
     //     before the last barrier; past the end of K the last tile is requested again, so that
     //     the count of loads in flight stays what the waits below assume.
-    auto iteration = [&](int it, auto s_tag, int b0, int b1, int b2) {
+    auto iteration = [&](int it, auto s_tag, int b0, int b1, int b2) __attribute__((always_inline)) {
         constexpr int s = decltype(s_tag)::value;
         const int q = s % SUP, pslot = (s / SUP) & 1;
         const int P = it / SUP;                                 // super index inside the group
@@ -520,19 +520,21 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     wait_loads_and_barrier<0>();
     if constexpr (C::PREFETCH_A) read_frags(fcur, 0);
 
+    // The K loop runs whole passes of 2*SUP iterations (the period of the register rings); what is left over is
+    // a straight-line tail behind it.  No iteration is skipped by a branch inside the loop, so every path through
+    // the loop issues the same loads -- which is what the wait counts assume and what the JIT re-counts on the ISA.
+    constexpr int PASS = 2 * SUP, FULL_PASSES = C::ITERS / PASS, REST = C::ITERS % PASS;
     int b0 = 0, b1 = 1, b2 = C::PA - 1;
+    auto step = [&](int it, auto s_tag) __attribute__((always_inline)) {
+        iteration(it, s_tag, b0, b1, b2);
+        b0 = b1;
+        b1 = b1 == C::NBUF - 1 ? 0 : b1 + 1;
+        b2 = b2 == C::NBUF - 1 ? 0 : b2 + 1;
+    };
 #pragma unroll 1
-    for (int it0 = 0; it0 < C::ITERS; it0 += 2 * SUP) {
-        static_for<0, 2 * SUP>([&](auto s_tag) {
-            constexpr int s = decltype(s_tag)::value;
-            if (it0 + s < C::ITERS) {
-                iteration(it0 + s, s_tag, b0, b1, b2);
-                b0 = b1;
-                b1 = b1 == C::NBUF - 1 ? 0 : b1 + 1;
-                b2 = b2 == C::NBUF - 1 ? 0 : b2 + 1;
-            }
-        });
-    }
+    for (int pass = 0; pass < FULL_PASSES; pass++)
+        static_for<0, PASS>([&](auto s_tag) { step(pass * PASS + decltype(s_tag)::value, s_tag); });
+    static_for<0, REST>([&](auto s_tag) { step(FULL_PASSES * PASS + decltype(s_tag)::value, s_tag); });
     // The wait counts above assume that every iteration really issues the loads `loads_since` counts.  What
     // the last iterations load for supers past the end is never used, and a compiler that can see that (a
     // K loop of a single trip) drops those loads or merges them (they all clamp to the last super): fewer

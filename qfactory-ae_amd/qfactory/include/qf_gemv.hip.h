@@ -60,7 +60,8 @@ struct GemvCfg {
 };
 
 // Timing experiments (results are wrong when non-zero): bit 0 replaces the decode + dot products by
-// an xor of the loaded words, bit 1 skips the activation loads, bit 2 the scale / zero-point loads.
+// an xor of the loaded words, bit 1 skips the activation loads, bit 2 reads the scales / zero-points of row 0 for
+// every row, bit 3 drops the cross-lane sums, the LDS exchange and the stores.
 // A translation unit that sets it must also define QF_ALLOW_TIMING_EXPERIMENTS; the code generator never does.
 #ifndef QF_GEMV_EXPERIMENT
 #define QF_GEMV_EXPERIMENT 0
@@ -100,6 +101,16 @@ struct GemvCfg {
 #define QF_GEMV_SMEM_QUANT 0
 #endif
 
+// 1: scales and zero-points are applied after the first steps of the cross-lane sum instead of per lane.  The
+// lanes that share a group (GS / elements-per-chunk consecutive lanes, four at 4 bits and groups of 128) first
+// add their integer-domain chunk sums with the butterfly's own first halving steps; a lane then owns one row
+// (of the stage's U) and one group, loads that one scale and zero-point, applies  s * (T - Z * sum a)  and the
+// butterfly goes on.  Per stage and chunk a lane issues U >> PRE scale loads instead of U (PRE = 2 at best), and
+// the scale arithmetic shrinks alike.  Deferred decode only; not with the scales through LDS.
+#ifndef QF_GEMV_QUANT_DEDUP
+#define QF_GEMV_QUANT_DEDUP 0
+#endif
+
 // Lower bound on resident waves per SIMD the register allocator must leave room for (0: no bound).
 #ifndef QF_GEMV_WAVES_PER_EU
 #define QF_GEMV_WAVES_PER_EU 0
@@ -125,6 +136,10 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     constexpr bool SILU = QF_GEMV_GATE_UP_SILU != 0;
     constexpr bool EAGER = QF_GEMV_EAGER != 0 && C::QPARAM;
     constexpr bool SMEMQ = QF_GEMV_SMEM_QUANT != 0 && C::QPARAM;
+    constexpr int LPG = C::QPARAM ? C::GS / EPC : 1;                              // lanes per group
+    constexpr int PRE = !(QF_GEMV_QUANT_DEDUP && C::QPARAM && !EAGER && !SMEMQ) ? 0
+                        : ((LPG % 4 == 0 && U % 4 == 0) ? 2 : ((LPG % 2 == 0 && U % 2 == 0) ? 1 : 0));
+    constexpr int UP = U >> PRE, VP = V >> PRE;                                   // rows / partial sums a lane keeps after PRE halving steps
     constexpr int SQ_WORDS = SMEMQ ? (C::RPB * C::G * 2 + 3) / 4 : 1;           // 32-bit words of the block's scales
     constexpr int ZQ_WORDS = SMEMQ && !C::SYM ? (C::RPB * C::ZRB + 3) / 4 : 1;  // and of its zero-points
 
@@ -182,9 +197,14 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     struct Stage {
         uint32_t w[U][IT][NW];
         uint32_t h[U][IT][NWH > 0 ? NWH : 1];
-        scale_holder_t s[U][IT];
-        zero_holder_t z[U][IT];
+        scale_holder_t s[UP][IT];
+        zero_holder_t z[UP][IT];
     };
+    // after PRE halving steps a lane keeps rows j + u_lane, j < UP, of a stage (the halving sends the upper half of
+    // the values to the lanes whose distance bit is set)
+    int u_lane = 0;
+    if constexpr (PRE >= 1) u_lane += (lane & kLaneOrder(0)) ? U / 2 : 0;
+    if constexpr (PRE >= 2) u_lane += (lane & kLaneOrder(1)) ? U / 4 : 0;
 
     auto load_stage = [&](Stage& st, int step) {
 #pragma unroll
@@ -199,9 +219,25 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
             for (int it = 0; it < IT; it++) {
                 load_words<NW, C::NT_B>(wrow + (uint32_t)coff[it], st.w[u][it]);
                 if constexpr (NWH > 0) load_words<NWH, C::NT_B>(wrow + (uint32_t)(C::HI_OFF + coff[it] / 2), st.h[u][it]);
-                if constexpr (C::QPARAM && !SMEMQ && !(QF_GEMV_EXPERIMENT & 4)) {
-                    st.s[u][it] = *reinterpret_cast<const uint16_t*>(srow + (uint32_t)(goff[it] * 2));
-                    if constexpr (!C::SYM) st.z[u][it] = zrow[(uint32_t)(goff[it] / P8)];
+                if constexpr (C::QPARAM && !SMEMQ && PRE == 0) {
+                    const uint8_t* sr = (QF_GEMV_EXPERIMENT & 4) ? reinterpret_cast<const uint8_t*>(S) : srow;   // timing: always row 0 (cache hits)
+                    const uint8_t* zr = (QF_GEMV_EXPERIMENT & 4) ? Zp : zrow;
+                    st.s[u][it] = *reinterpret_cast<const uint16_t*>(sr + (uint32_t)(goff[it] * 2));
+                    if constexpr (!C::SYM) st.z[u][it] = zr[(uint32_t)(goff[it] / P8)];
+                }
+            }
+        }
+        if constexpr (PRE > 0) {
+            // one scale and one zero-point per row this lane will own after the first halving steps
+#pragma unroll
+            for (int j = 0; j < UP; j++) {
+                const int lrow = min(row_base + step * U + j + u_lane, C::N - 1);            // per lane
+                const int row = SILU ? (lrow >> 1) + (lrow & 1) * (C::N / 2) : lrow;
+#pragma unroll
+                for (int it = 0; it < IT; it++) {
+                    st.s[j][it] = *reinterpret_cast<const uint16_t*>(
+                        reinterpret_cast<const uint8_t*>(S) + (uint32_t)(row * (C::G * 2) + goff[it] * 2));
+                    if constexpr (!C::SYM) st.z[j][it] = Zp[(uint32_t)(row * C::ZRB + goff[it] / P8)];
                 }
             }
         }
@@ -273,8 +309,21 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         }
     }
 
+    // sum of the activations over a group's share of lanes (the lanes PRE halving steps bring together)
+    float saq[MT][IT];
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int it = 0; it < IT; it++) {
+            float v = sa[m][it];
+            if constexpr (PRE >= 1) v += lane_xor<kLaneOrder(0)>(v);
+            if constexpr (PRE >= 2) v += lane_xor<kLaneOrder(1)>(v);
+            saq[m][it] = v;
+        }
+
     auto compute_stage = [&](const Stage& st, int step) {
         float part[V];
+        float tq[PRE > 0 ? IT : 1][V];        // PRE > 0: integer-domain chunk sums, scaled after the first halving steps
 #pragma unroll
         for (int v = 0; v < V; v++) part[v] = 0.0f;
 #pragma unroll
@@ -287,7 +336,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
 #pragma unroll
                     for (int c2 = 0; c2 < NCLS; c2++) acc[m][c2] = 0.0f;
                 uint32_t sbits = 0x3C00u, zint = 0u;               // scale (fp16 bits) and zero-point of this chunk's group
-                if constexpr (C::QPARAM) {
+                if constexpr (C::QPARAM && PRE == 0) {
                     const int brow = team * C::RPT + step * U + u;            // row inside the block
                     if constexpr (SMEMQ) sbits = reinterpret_cast<const uint16_t*>(sq_s)[brow * C::G + goff[it]];
                     else sbits = (uint16_t)st.s[u][it];
@@ -339,7 +388,9 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                         part[u * MT + m] += t;                   // the weights were dequantised before the dot product
                     } else {
                         t -= c1[m][it];                          // = sum a*q over the chunk
-                        if constexpr (C::QPARAM) {
+                        if constexpr (PRE > 0) {
+                            tq[it][u * MT + m] = t;
+                        } else if constexpr (C::QPARAM) {
                             t = __builtin_fmaf(-zf, sa[m][it], t);   // sum a*(q - Z)
                             part[u * MT + m] = __builtin_fmaf(sc, t, part[u * MT + m]);
                         } else {
@@ -349,7 +400,30 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 }
             }
         }
-        wave_reduce_many<V>(part, lane);
+        if constexpr (PRE > 0) {
+            // the lanes of a group add their chunk sums (the butterfly's first PRE halving steps); the lane then
+            // owns rows j + u_lane of the stage and applies its own row's scale and zero-point
+#pragma unroll
+            for (int it = 0; it < IT; it++) {
+                halve_step<kLaneOrder(0), V, V>(tq[it], lane);
+                if constexpr (PRE >= 2) halve_step<kLaneOrder(1), V / 2, V>(tq[it], lane);
+#pragma unroll
+                for (int i = 0; i < VP; i++) {
+                    const int j = i / MT, m = i % MT;
+                    const float sc = f16_bits_to_f32((uint16_t)st.s[j][it]);
+                    float zf = (float)(1 << (C::NBITS - 1));
+                    if constexpr (!C::SYM) zf = (float)((st.z[j][it] >> ((goff[it] % P8) * C::ZFB)) & ZMASK);
+                    part[i] = __builtin_fmaf(sc, __builtin_fmaf(-zf, saq[m][it], tq[it][i]), part[i]);
+                }
+            }
+            reduce_from<VP, PRE, V>(part, lane);
+        } else if constexpr ((QF_GEMV_EXPERIMENT & 8) != 0) {          // timing: no cross-lane sums, no LDS, no stores
+            float t = 0.f;
+            for (int v = 0; v < V; v++) t += part[v];
+            if (t == 12345.678f) Cout[lane] = 1;
+            return;
+        }
+        if constexpr (PRE == 0) wave_reduce_many<V>(part, lane);
         if (reduce_owner<V>(lane)) {
             const int v = reduce_index<V>(lane);
             if constexpr (WK == 1 && !SILU) { // one wave owns the rows: store straight from the lane
@@ -381,6 +455,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     }
 
     if constexpr (WK == 1 && !SILU) return;
+    if constexpr ((QF_GEMV_EXPERIMENT & 8) != 0) return;
     __syncthreads();
 
     if constexpr (SILU) {

@@ -43,13 +43,22 @@ def test_every_counted_load_is_issued(M, N, K, nbits, gs, tmp_path):
 
 def test_checker_rejects_a_missing_load():
     from qfactory.jit.verify import gemm_waits_hold
-    body = ["global_load_dwordx4 v[0:3], v4, s[0:1]"] * 3 + ["s_waitcnt vmcnt(3) lgkmcnt(0)"]
-    good = "\n".join(["s_waitcnt vmcnt(0) lgkmcnt(0)"] + body * 4)
-    assert gemm_waits_hold(good, 3)[0]
-    bad = good.replace("global_load_dwordx4 v[0:3], v4, s[0:1]\n", "", 1)          # the compiler dropped one
-    ok, detail = gemm_waits_hold(bad, 3)
-    assert not ok and "allows 3" in detail
-    assert not gemm_waits_hold("s_endpgm", 3)[0]                                    # no counted wait at all
+    load = "\tglobal_load_dwordx4 v[0:3], v4, s[0:1]"
+    iteration = [load] * 3 + ["\ts_waitcnt vmcnt(3) lgkmcnt(0)", "\ts_barrier"]
+    def listing(body):
+        return "\n".join(["_Z6kernelv:", "\ts_waitcnt vmcnt(0) lgkmcnt(0)"] + body + ["\ts_endpgm", ".Lfunc_end0:"])
+    assert gemm_waits_hold(listing(iteration * 4), 3) == (True, "3 counted waits hold on every path")
+    dropped = iteration * 2 + iteration[1:] + iteration                           # the compiler dropped one load
+    ok, detail = gemm_waits_hold(listing(dropped), 3)
+    assert not ok and "allows 3 loads in flight but a path issues only 2" in detail
+    # a rotated loop: the latch block (with the wait) is laid out in front of the header; and a branch that
+    # skips a load on one path only
+    rotated = ["\ts_branch .LBB0_2", ".LBB0_1:", "\ts_waitcnt vmcnt(3) lgkmcnt(0)", ".LBB0_2:"] + [load] * 3 + \
+              ["\ts_cbranch_scc1 .LBB0_1"]
+    assert gemm_waits_hold(listing(iteration * 2 + rotated), 3)[0]
+    skipping = iteration * 2 + [load, "\ts_cbranch_vccnz .LBB0_3", load, ".LBB0_3:", load, "\ts_waitcnt vmcnt(3) lgkmcnt(0)"]
+    assert not gemm_waits_hold(listing(skipping), 3)[0]
+    assert not gemm_waits_hold("s_endpgm", 3)[0]                                    # no kernel, no counted wait
 
 
 def test_jit_falls_back_to_a_full_drain_when_the_count_fails(tmp_path, monkeypatch):
