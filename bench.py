@@ -12,8 +12,16 @@ inner loop of a decode step) and replayed once between synchronisations.
 Printed JSON: `value` = algorithmic bytes moved per second over the timed region (the reference's
 own footprint formula, reproduce/fig9/plot_bandwidth_size.py:37-44); `roofline` = the dominant
 kernel (gate+up) against the 8 TB/s HBM peak, its duration measured here with HIP events on the
-launch stream; `cpu_baseline` = the torch CPU dequant+matmul port of the reference's test path on
-the same four shapes, on this machine's host cores.
+launch stream, beside two ceilings measured in the same run (`roofline.empirical`: a pure streaming
+read of the same number of bytes, and a large dense fp16 GEMM of the vendor library);
+`cpu_baseline` = the torch CPU dequant+matmul port of the reference's test path on the same four
+shapes, on this machine's host cores.  Further sections, none of them part of `value`:
+`small_m` (configs[1] at M = 4 / 16, configs[2]: the bit-width sweep at N = K = 8192, and the
+Llama-3-70B shapes at M = 1), `gemm_m256` and `gemm_m32_m64_m128` (configs[3]) and `decode`
+(configs[4]: the Llama-2-7B-shaped decode loop at batch 1 / 16 / 64).
+
+Every per-kernel timing rotates over at least 512 MB of distinct packed weights (twice the 256 MB
+Infinity Cache), so each launch streams its weights from HBM.
 """
 import argparse
 import json
@@ -88,21 +96,42 @@ def check_against_oracle(layer, acts):
     return m
 
 
-def kernel_event_time_us(lins, x, reps=64):
-    """Average duration of one launch of a layer type with cold weights.
+COLD_BYTES = 512 << 20          # distinct packed bytes a per-kernel timing rotates over: 2 x the 256 MB Infinity Cache
 
-    `reps` back-to-back launches (rotating over the layers' distinct weight copies) are captured in
-    a HIP graph on a side stream; the replay is bracketed by HIP events recorded on the stream it is
-    launched on, and the elapsed time is divided by `reps`.  Back-to-back launches on one stream
+
+def cold_copies(bytes_per_copy, minimum=2):
+    """Number of distinct weight copies a timing needs so that a launch never finds its weights in a cache."""
+    return max(minimum, -(-COLD_BYTES // int(bytes_per_copy)))
+
+
+def weight_sets(lin, n, gen):
+    """`n` independent sets of packed tensors (w, s, z) shaped like the layer's, random bytes / scales in range."""
+    import torch
+    sets = []
+    for _ in range(n):
+        w = torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=gen)
+        s = (torch.rand(lin.s.shape, device="cuda", generator=gen) * 0.019 + 0.001).to(torch.float16)
+        z = None if lin.z is None else torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=gen)
+        sets.append((w, s, z))
+    return sets
+
+
+def kernel_event_time_us(func, sets, x, n_out, reps=None):
+    """Average duration of one launch of a compiled closure with cold weights.
+
+    `reps` back-to-back launches (rotating over the distinct weight sets, at least 512 MB of them) are
+    captured in a HIP graph on a side stream; the replay is bracketed by HIP events recorded on the stream
+    it is launched on, and the elapsed time is divided by `reps`.  Back-to-back launches on one stream
     serialise on this GPU, so this is the per-launch duration a kernel trace reports.
     """
     import torch
-    outs = [torch.empty(x.shape[0], lin.w.shape[0], dtype=torch.float16, device="cuda") for lin in lins]
+    reps = reps or max(16, len(sets))
+    out = torch.empty(x.shape[0], n_out, dtype=torch.float16, device="cuda")
 
     def launches():
         for i in range(reps):
-            lin, out = lins[i % len(lins)], outs[i % len(lins)]
-            rc = lin.func(x, lin.w, out, lin.s, lin.z) if lin.z is not None else lin.func(x, lin.w, out, lin.s)
+            w, s, z = sets[i % len(sets)]
+            rc = func(x, w, out, s, z) if z is not None else func(x, w, out, s)
             assert rc == 0
 
     launches()
@@ -128,6 +157,60 @@ def kernel_event_time_us(lins, x, reps=64):
     return best[len(best) // 2]
 
 
+def stream_read_time_us(nbytes):
+    """A pure 128-bit streaming read (qf_stream_read of libqfactory_hip.so) of `nbytes` cold bytes, timed like a
+    kernel above: the ceiling this machine gives a launch that only has to read that many bytes."""
+    import torch
+    from qfactory import native
+    nbytes = int(nbytes) // 4096 * 4096
+    n = cold_copies(nbytes)
+    bufs = [torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device="cuda") for _ in range(n)]
+    sink = torch.zeros(4096, dtype=torch.int32, device="cuda")          # qf_stream_read writes one word per block, index modulo 4096
+    reps = max(16, n)
+
+    def launches():
+        for i in range(reps):
+            native.stream_read(bufs[i % n], sink)
+
+    launches()
+    torch.cuda.synchronize()
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+        launches()
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(5):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(end) * 1e3 / reps)
+    times.sort()
+    return times[len(times) // 2]
+
+
+def dense_square_tflops(n=8192, reps=10):
+    """A large square dense fp16 GEMM of the vendor library (torch.matmul): the matrix-core ceiling this machine
+    gives a well-shaped problem."""
+    import torch
+    a = torch.randn(n, n, device="cuda", dtype=torch.float16)
+    b = torch.randn(n, n, device="cuda", dtype=torch.float16)
+    for _ in range(3):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        torch.matmul(a, b)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2.0 * n ** 3 * reps / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
+
 def module_time_us(lins, x, reps=256):
     """Average time of one eager ``layer(x)`` call -- output allocation, Python checks, ctypes and the launch, as the
     reference's latency harness times it (qfactory/testing.py:31-35) -- rotating over the layers' weight copies;
@@ -144,18 +227,18 @@ def module_time_us(lins, x, reps=256):
     return (time.perf_counter() - t0) / reps * 1e6
 
 
-def dense_fp16_time_us(M, N, K, total_bytes=600e6):
+def dense_fp16_time_us(M, N, K, total_bytes=COLD_BYTES):
     """The vendor library's dense fp16 GEMM of the same shape (torch.matmul on hipBLASLt / rocBLAS), cold
     weights: the comparison the reference's own evaluation makes against cuBLAS
     (qfactory/testing.py:36-41).  A reported yardstick, not part of the path."""
     import torch
-    n = max(2, min(8, int(total_bytes // (N * K * 2))))
+    n = max(2, -(-int(total_bytes) // (N * K * 2)))
     ws = [torch.randn(N, K, device="cuda", dtype=torch.float16) for _ in range(n)]
     x = torch.randn(M, K, device="cuda", dtype=torch.float16)
     for w in ws:
         torch.matmul(x, w.T)
     torch.cuda.synchronize()
-    reps = 4 * n
+    reps = max(8, n)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(reps):
@@ -165,39 +248,34 @@ def dense_fp16_time_us(M, N, K, total_bytes=600e6):
     return e0.elapsed_time(e1) * 1e3 / reps
 
 
-def gemm_report(M=256, copies_bytes=600e6):
-    """BASELINE.json configs[3] at M = 256: W4A16 g128 GEMM on Llama-3-70B-style shapes, per shape
-    microseconds, TFLOP/s and the fraction of the dense fp16 MFMA peak."""
+def gemm_report(M=256):
+    """BASELINE.json configs[3]: W4A16 g128 GEMM on Llama-3-70B-style shapes, per shape microseconds, TFLOP/s,
+    the fraction of the dense fp16 MFMA peak and of the HBM peak (M <= 64 is HBM-bound by arithmetic intensity)."""
     import torch
     from qfactory import QLinear
     flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
     g = torch.Generator(device="cuda").manual_seed(1)
     report = []
     for name, N, K in GEMM_SHAPES:
-        n_copies = max(2, min(8, int(copies_bytes // (N * K // 2))))
-        lins = []
-        for _ in range(n_copies):
-            lin = QLinear.empty(M, K, N, NBITS, GS, sym=False, compile_flags=flags)
-            lin.w.copy_(torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=g))
-            lin.s.copy_((torch.rand(lin.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
-            lin.z.copy_(torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=g))
-            lins.append(lin)
+        lin = QLinear.empty(M, K, N, NBITS, GS, sym=False, compile_flags=flags)
+        sets = weight_sets(lin, cold_copies(N * K // 2), g)
         x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
-        us = kernel_event_time_us(lins, x, reps=2 * n_copies)
-        description = lins[0].func.runtime.description
-        del lins
+        us = kernel_event_time_us(lin.func, sets, x, N, reps=max(8, len(sets)))
+        description = lin.func.runtime.description
+        del lin, sets
         torch.cuda.empty_cache()
         dense_us = dense_fp16_time_us(M, N, K)
         flops = 2.0 * M * N * K
         rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1),
                "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
                "GB/s": round(algorithmic_bytes(M, N, K) / us / 1e3, 1),
+               "hbm_frac": round(algorithmic_bytes(M, N, K) / us / 1e3 / HBM_PEAK_GBPS, 4),
                "dense_fp16_us": round(dense_us, 2), "speedup_over_dense_fp16": round(dense_us / us, 3),
                "kernel": description}
         report.append(rec)
         log(f"[bench] GEMM M={M} {name:11s} N={N:6d} K={K:6d} {us:8.2f} us {rec['TFLOP/s']:7.1f} TFLOP/s "
-            f"{100 * rec['mfma_frac']:5.1f}% of fp16 MFMA peak; dense fp16 torch.matmul {dense_us:8.2f} us "
-            f"(x{rec['speedup_over_dense_fp16']:.2f})")
+            f"{100 * rec['mfma_frac']:5.1f}% of fp16 MFMA peak, {100 * rec['hbm_frac']:5.1f}% of HBM peak; "
+            f"dense fp16 torch.matmul {dense_us:8.2f} us (x{rec['speedup_over_dense_fp16']:.2f})")
     return report
 
 
@@ -205,11 +283,10 @@ COPY_BYTES = 64 << 20
 
 # HBM traffic per launch of the dominant kernel, from hardware counters: rocprofv3 --pmc FETCH_SIZE
 # and --pmc WRITE_SIZE over `bench.py --counter-pass`, each scaled by what the same counter reads
-# for the 64 MiB stream copy of that run (which moves COPY_BYTES each way).  Keyed by the kernel's
-# description so that a different specialisation reports null instead of a stale figure.
+# for the 64 MiB stream copy of that run (which moves COPY_BYTES each way).  A stored measurement:
+# keyed by the description of the specialisation it was taken on, reported with that key, and null
+# for any other specialisation (profiles/gemv_w4g128_llama2_7b_m1_hbm_traffic_pmc.md holds the run).
 MEASURED_TRAFFIC = {
-    # FETCH_SIZE 22938.4 KiB x (65536 / 32807.5, the copy's read of 64 MiB) + WRITE_SIZE 86 KiB x (65536 / 65536)
-    "regime=gemv M=1 N=22016 K=4096 NBITS=4 GS=128 SYM=0 decode=deferred nt_b=1 MT=1 STEPS=1 U=4 VB=16 WK=2 WN=2": 47009000,
 }
 
 
@@ -228,42 +305,36 @@ def counter_pass(layers, acts, reps=5):
     log(f"[bench] counter pass: {reps} launches of each kernel and of a {COPY_BYTES} byte stream copy")
 
 
-def _timed_layers(M, N, K, nbits, sym, total_bytes=600e6):
-    """A few QLinear copies of one problem with random packed tensors (enough bytes to defeat the caches)."""
+def _timed_problem(M, N, K, nbits, sym):
+    """One QLinear of the problem plus enough random packed-tensor sets to defeat the caches (>= 512 MB)."""
     import torch
     from qfactory import QLinear
     flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
     g = torch.Generator(device="cuda").manual_seed(2)
-    n_copies = max(2, min(8, int(total_bytes // (N * K * nbits // 8))))
-    lins = []
-    for _ in range(n_copies):
-        lin = QLinear.empty(M, K, N, nbits, GS, sym=sym, compile_flags=flags)
-        lin.w.copy_(torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=g))
-        lin.s.copy_((torch.rand(lin.s.shape, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16))
-        if not sym:
-            lin.z.copy_(torch.randint(-128, 128, lin.z.shape, dtype=torch.int8, device="cuda", generator=g))
-        lins.append(lin)
+    lin = QLinear.empty(M, K, N, nbits, GS, sym=sym, compile_flags=flags)
+    sets = weight_sets(lin, cold_copies(N * K * nbits // 8), g)
     x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
-    return lins, x
+    return lin, sets, x
 
 
 def small_m_report():
-    """BASELINE.json configs[1] at M in {4, 16} and configs[2] (N = K = 8192, M in {1, 16}, 2/3/4/8-bit,
-    symmetric and asymmetric): per shape microseconds and the fraction of the 8 TB/s HBM roofline."""
+    """BASELINE.json configs[1] at M in {4, 16}, configs[2] (N = K = 8192, M in {1, 16}, 2/3/4/8-bit,
+    symmetric and asymmetric) and the Llama-3-70B shapes at M = 1: per shape microseconds and the fraction
+    of the 8 TB/s HBM roofline."""
     import torch
     report = []
 
     def one(tag, M, N, K, nbits, sym):
-        lins, x = _timed_layers(M, N, K, nbits, sym)
-        us = kernel_event_time_us(lins, x, reps=8 * len(lins))
+        lin, sets, x = _timed_problem(M, N, K, nbits, sym)
+        us = kernel_event_time_us(lin.func, sets, x, N)
         b = algorithmic_bytes(M, N, K, nbits, GS, sym)
         rec = {"config": tag, "M": M, "N": N, "K": K, "bits": nbits, "sym": sym, "us": round(us, 3),
                "GB/s": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
-               "TFLOP/s": round(2.0 * M * N * K / us / 1e6, 2), "kernel": lins[0].func_for(M).runtime.description}
+               "TFLOP/s": round(2.0 * M * N * K / us / 1e6, 2), "kernel": lin.func.runtime.description}
         report.append(rec)
         log(f"[bench] {tag} M={M:3d} N={N:6d} K={K:6d} b={nbits} {'sym ' if sym else 'asym'} {us:8.2f} us "
             f"{rec['GB/s']:7.1f} GB/s {100 * rec['hbm_frac']:5.1f}% of HBM peak")
-        del lins
+        del lin, sets
         torch.cuda.empty_cache()
 
     for M in (4, 16):
@@ -276,6 +347,24 @@ def small_m_report():
     # the 28672-wide end of the "4096 - 28672-wide LLM shapes" the GEMV target names: Llama-3-70B at M = 1
     for name, N, K in GEMM_SHAPES:
         one("70b-gemv", 1, N, K, NBITS, False)
+    return report
+
+
+def decode_report(batches=(1, 16, 64), prompt_len=128, new_tokens=128):
+    """BASELINE.json configs[4]: the Llama-2-7B-shaped greedy decode loop (32 layers, every linear a W4A16 g128
+    QLinear, random weights and prompt ids): tokens/s and the share of a decode step spent in the quantized
+    linears, per batch size (qfactory-ae_amd/decode_llama.py)."""
+    import torch
+    import decode_llama
+    shape = decode_llama.LlamaShape(max_len=prompt_len + new_tokens)
+    report = []
+    for batch in batches:
+        rec = decode_llama.run(shape, batch, prompt_len, new_tokens)
+        report.append(rec)
+        log(f"[bench] decode batch={batch:3d}: {rec['value']:9.1f} tokens/s, step {rec['decode_step_us']:8.1f} us, "
+            f"quantized linears {rec['quantized_linears_us_per_step']:8.1f} us ({100 * rec['quantized_linear_share']:.0f}%), "
+            f"prefill {rec['prefill_tokens_per_s']:9.1f} tokens/s")
+        torch.cuda.empty_cache()
     return report
 
 
@@ -322,8 +411,10 @@ def main():
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=256 GEMM report")
     ap.add_argument("--no-module-time", action="store_true",
                     help="skip the eager layer(x) timing (its launches would mix into a kernel trace's averages)")
-    ap.add_argument("--small-m", action="store_true",
-                    help="also report configs[1] at M = 4, 16 and the configs[2] bit-width sweep (not part of `value`)")
+    ap.add_argument("--small-m", action="store_true", help="accepted for compatibility: the small-M report is on by default")
+    ap.add_argument("--no-small-m", action="store_true",
+                    help="skip configs[1] at M = 4, 16, the configs[2] bit-width sweep and the 70B shapes at M = 1")
+    ap.add_argument("--no-decode", action="store_true", help="skip the configs[4] decode loop")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
     ap.add_argument("--counter-pass", action="store_true",
                     help="only launch each of the four kernels (cold weights) and a 64 MiB stream copy a few times, "
@@ -376,22 +467,34 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     value = step_bytes / (elapsed / args.steps) / 1e9
 
-    # per-kernel durations (HIP events on the launch stream), cold weights
+    # per-kernel durations (HIP events on the launch stream), cold weights: >= 512 MB of distinct packed tensors each
     shapes_report = []
     dominant = None
+    g = torch.Generator(device="cuda").manual_seed(3)
     for name, N, K in SHAPES:
-        us = kernel_event_time_us([layer[name] for layer in layers], acts[K])
+        lin = layers[0][name]
+        sets = weight_sets(lin, cold_copies(N * K // 2), g)
+        us = kernel_event_time_us(lin.func, sets, acts[K], N)
+        del sets
+        torch.cuda.empty_cache()
         b = algorithmic_bytes(M, N, K)
         rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 3), "GB/s": round(b / us / 1e3, 1),
                "TFLOP/s": round(2 * M * N * K / us / 1e6, 3), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
-               "bytes": int(b), "kernel": layers[0][name].func.runtime.description}
+               "bytes": int(b), "kernel": lin.func.runtime.description}
+        stream_us = stream_read_time_us(b)
+        rec["stream_read_us"] = round(stream_us, 3)
+        rec["frac_of_stream_read"] = round(stream_us / us, 4)
         if not args.no_module_time:
             rec["module_us"] = round(module_time_us([layer[name] for layer in layers], acts[K]), 2)
         shapes_report.append(rec)
         log(f"[bench] {name:8s} N={N:6d} K={K:6d}  {us:7.2f} us  {rec['GB/s']:7.1f} GB/s  {100 * rec['hbm_frac']:5.1f}% of HBM peak"
+            f"  (a pure streaming read of the same bytes: {stream_us:.2f} us)"
             + (f"  (eager layer(x): {rec['module_us']:.2f} us per call)" if "module_us" in rec else ""))
         if name == DOMINANT:
             dominant = rec
+    dense_tflops = dense_square_tflops()
+    log(f"[bench] ceilings measured here: streaming read of {dominant['bytes']} bytes {dominant['bytes'] / dominant['stream_read_us'] / 1e3:.1f} GB/s, "
+        f"dense fp16 8192^3 torch.matmul {dense_tflops:.1f} TFLOP/s")
 
     result = {
         "metric": "W4A16 g128 GEMV (M=1) algorithmic HBM throughput over the Llama-2-7B linear shapes",
@@ -406,17 +509,30 @@ def main():
         "roofline": {"bound": "hbm", "achieved": dominant["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(dominant["GB/s"] / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC.get(dominant["kernel"]),
+                     "traffic_source": ("stored rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE measurement of this specialisation"
+                                        if dominant["kernel"] in MEASURED_TRAFFIC else
+                                        "no stored counter measurement for this specialisation"),
                      "kernel": f"qf::gemv_kernel {DOMINANT} N=22016 K=4096 M=1", "avg_launch_us": dominant["us"],
-                     "algorithmic_bytes_per_launch": dominant["bytes"]},
+                     "algorithmic_bytes_per_launch": dominant["bytes"],
+                     "empirical": {"stream_read_GB/s": round(dominant["bytes"] / dominant["stream_read_us"] / 1e3, 1),
+                                   "stream_read_us": dominant["stream_read_us"],
+                                   "frac_of_stream_read": dominant["frac_of_stream_read"],
+                                   "what": "qf_stream_read of the same number of cold bytes, timed like the kernel",
+                                   "dense_fp16_TFLOP/s": round(dense_tflops, 1),
+                                   "dense_fp16_what": "torch.matmul 8192 x 8192 x 8192 (vendor library), hot operands"}},
         "shapes": shapes_report,
         "parity": parity,
     }
     if not args.no_gemm:
-        result["gemm_m256"] = {"peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS, "shapes": gemm_report(256)}
-    if args.small_m:
+        result["gemm_m256"] = {"peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS, "dense_fp16_TFLOP/s_measured": round(dense_tflops, 1),
+                               "shapes": gemm_report(256)}
+        result["gemm_m32_m64_m128"] = [rec for m_rows in (32, 64, 128) for rec in gemm_report(m_rows)]
+    if not args.no_small_m:
         result["small_m"] = small_m_report()
-        if not args.no_gemm:
-            result["gemm_m32_m64_m128"] = [rec for M in (32, 64, 128) for rec in gemm_report(M)]
+    if not args.no_decode:
+        del layers
+        torch.cuda.empty_cache()
+        result["decode"] = decode_report()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
         log(f"[bench] cpu baseline: {result['cpu_baseline']}")

@@ -55,7 +55,8 @@ int qf_bf16_to_f16(const uint16_t* src, uint16_t* dst, int64_t n, void* stream);
 /*
  * Calibration kernels (no reference counterpart; the reference times with triton's do_bench only,
  * qfactory/profile.py:5-10).  qf_stream_read reads `bytes` (multiple of 16) with 128-bit loads and
- * writes one checksum word per block to `sink` (>= 4096 uint32); qf_stream_copy copies `bytes`
+ * writes to `sink` (>= 4096 uint32) only where a thread's folded words equal a fixed constant (practically
+ * never: the stores exist so that the loads cannot be dropped); qf_stream_copy copies `bytes`
  * (multiple of 16) from src to dst.  They give the achievable HBM rate for a given footprint and a
  * known-traffic dispatch against which hardware counters can be scaled.
  */

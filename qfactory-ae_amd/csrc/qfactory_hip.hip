@@ -106,8 +106,13 @@ __global__ __launch_bounds__(256) void transpose_u16_kernel(const uint16_t* __re
 // Calibration kernels
 // ---------------------------------------------------------------------------------------------
 constexpr int kStreamThreads = 256;
-constexpr int kStreamUnroll = 8;
+constexpr int kStreamUnroll = 4;
 
+// Every thread requests kStreamUnroll 16-byte units, all before it touches any, and folds them into one word.  The
+// word is stored only if it equals a fixed constant, which random data practically never does: the loads cannot
+// be dropped and the block ends with its last byte -- no cross-lane sum, no barrier, no store.  (A version that
+// wrote one checksum word per block through a wave shuffle and LDS measured 6 % slower at 47 MB: the read ceiling
+// is what this kernel is for.)
 __global__ __launch_bounds__(kStreamThreads) void stream_read_kernel(const u32x4* __restrict__ src, size_t n16,
                                                                      uint32_t* __restrict__ sink) {
     const size_t per_block = (size_t)kStreamThreads * kStreamUnroll;
@@ -117,20 +122,11 @@ __global__ __launch_bounds__(kStreamThreads) void stream_read_kernel(const u32x4
 #pragma unroll
     for (int u = 0; u < kStreamUnroll; u++) {
         const size_t i = base + (size_t)u * kStreamThreads;
-        v[u] = i < n16 ? __builtin_nontemporal_load(src + i) : u32x4{0, 0, 0, 0};
+        v[u] = __builtin_nontemporal_load(src + (i < n16 ? i : n16 - 1));
     }
 #pragma unroll
     for (int u = 0; u < kStreamUnroll; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
-    // one word per block so that the loads cannot be dropped
-    for (int d = 32; d >= 1; d >>= 1) acc ^= __shfl_xor(acc, d);
-    __shared__ uint32_t part[kStreamThreads / 64];
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t t = 0;
-        for (int w = 0; w < kStreamThreads / 64; w++) t ^= part[w];
-        sink[blockIdx.x & 4095] = t;
-    }
+    if (acc == 0x9E3779B9u) sink[blockIdx.x & 4095] = acc;
 }
 
 __global__ __launch_bounds__(kStreamThreads) void stream_copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src,

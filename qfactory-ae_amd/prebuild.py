@@ -122,6 +122,7 @@ def large_parity_cases():
     build from int32 tensors in a test; the tests fill packed tensors directly (every byte pattern
     is a valid packed weight) and check a seeded subset of output columns."""
     return ([_case(M, N, K) for N, K in LLAMA3_70B for M in (32, 64, 128, 256)]
+            + [_case(64, N, K) for N, K in LLAMA2_7B]              # the batch-64 decode linears
             + [_case(512, 10240, 8192), _case(1024, 12288, 4096), _case(700, 22016, 4096), _case(512, 22016, 4096), _case(1024, 10240, 8192)]
             # the large block tiles at the other bit widths, group sizes and with a partial last window
             + [_case(256, 16384, 4096, 2, 64), _case(256, 16384, 4096, 3, 128, True), _case(256, 16384, 4096, 8, 32),
@@ -188,7 +189,7 @@ TINY_LLAMA = [(768, 256), (256, 256), (1024, 256), (256, 512)]      # the decode
 def decode_cases():
     """decode_llama.py: Llama-2-7B shapes at batch 1 / 16 / 64 (decode) and at prefill row counts,
     plus the tiny model tests/test_decode_gpu.py runs."""
-    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 1024)]
+    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 512, 1024)]
     cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
     return cases + silu_mul_cases()
 

@@ -123,6 +123,7 @@ def bf16_to_f16(src, out=None):
 
 
 def stream_read(src, sink):
+    assert sink.numel() * sink.element_size() >= 4096 * 4, "qf_stream_read writes one checksum word per block into 4096 words"
     _check(load().qf_stream_read(src.data_ptr(), src.numel() * src.element_size(), sink.data_ptr(), _stream()), "qf_stream_read")
 
 
