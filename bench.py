@@ -193,6 +193,52 @@ def stream_read_time_us(nbytes):
     return times[len(times) // 2]
 
 
+def _graph_time_us(launches, reps):
+    """`launches()` enqueues `reps` back-to-back launches; they are captured in a HIP graph, the replay is timed with
+    HIP events on the launch stream (median of five), and the time per launch is returned."""
+    import torch
+    launches()
+    torch.cuda.synchronize()
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+        launches()
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(5):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(end) * 1e3 / reps)
+    times.sort()
+    return times[len(times) // 2]
+
+
+def launch_floor_report():
+    """What a launch costs before it does any work, and what a pure streaming read of a given size reaches, both timed
+    like the kernels (back-to-back launches in a HIP graph): a kernel that does nothing at several grid sizes, and
+    qf_stream_read at the footprints of the benchmark shapes.  The gap between a GEMV and 8 TB/s that is not the
+    kernel's own is read off these."""
+    from qfactory import native
+    report = {"empty_kernel_us": [], "stream_read": []}
+    for blocks, threads in ((1, 64), (256, 64), (256, 256), (1024, 256), (2752, 256), (4096, 256), (11008, 64), (16384, 256)):
+        us = _graph_time_us(lambda: [native.empty_launch(blocks, threads) for _ in range(64)], 64)
+        report["empty_kernel_us"].append({"blocks": blocks, "threads": threads, "us": round(us, 3)})
+        log(f"[bench] empty kernel {blocks:6d} x {threads:4d}: {us:6.2f} us per launch")
+    sizes = [(f"{name} M=1", algorithmic_bytes(1, N, K)) for name, N, K in SHAPES + GEMM_SHAPES]
+    sizes += [("1 MiB", 1 << 20), ("4 MiB", 4 << 20), ("512 MiB", 512 << 20)]
+    for what, nbytes in sizes:
+        us = stream_read_time_us(nbytes)
+        report["stream_read"].append({"what": what, "bytes": int(nbytes), "us": round(us, 3),
+                                      "GB/s": round(nbytes / us / 1e3, 1), "frac_of_8TB/s": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
+        log(f"[bench] stream read {what:18s} {int(nbytes):10d} B: {us:8.2f} us  {nbytes / us / 1e3:7.1f} GB/s")
+    return report
+
+
 def dense_square_tflops(n=8192, reps=10):
     """A large square dense fp16 GEMM of the vendor library (torch.matmul): the matrix-core ceiling this machine
     gives a well-shaped problem."""
@@ -416,6 +462,9 @@ def main():
                     help="skip configs[1] at M = 4, 16, the configs[2] bit-width sweep and the 70B shapes at M = 1")
     ap.add_argument("--no-decode", action="store_true", help="skip the configs[4] decode loop")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the timed steps eagerly from Python")
+    ap.add_argument("--launch-floor", action="store_true",
+                    help="only measure the launch floor (a kernel that does nothing, several grids) and the streaming-read "
+                         "ceiling at the benchmark footprints; prints one JSON object")
     ap.add_argument("--counter-pass", action="store_true",
                     help="only launch each of the four kernels (cold weights) and a 64 MiB stream copy a few times, "
                          "eagerly: the run to put under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
@@ -426,6 +475,9 @@ def main():
     import torch
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     torch.cuda.set_device(0)
+    if args.launch_floor:
+        print(json.dumps({"launch_floor": launch_floor_report()}), flush=True)
+        return
     M = 1
     layers, acts = build_layers(args.layers, M)
     parity = check_against_oracle(layers[0], acts)

@@ -62,6 +62,8 @@ int qf_bf16_to_f16(const uint16_t* src, uint16_t* dst, int64_t n, void* stream);
  */
 int qf_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
 int qf_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
+/* A kernel that does nothing, `blocks` x `threads` (<= 1024): the launch floor of a given grid. */
+int qf_empty_launch(int64_t blocks, int64_t threads, void* stream);
 
 /*
  * Steps of one decode token between the quantized linears of a Llama-style layer, one launch each.

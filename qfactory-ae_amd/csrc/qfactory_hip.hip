@@ -219,6 +219,16 @@ extern "C" int qf_transpose_scale(const uint16_t* scale, uint16_t* out, int64_t 
     return launched("qf_transpose_scale");
 }
 
+__global__ void empty_kernel(uint32_t* sink) {
+    if (sink == nullptr && threadIdx.x == 0xFFFFu) sink[0] = 1;     // never true: the kernel does nothing
+}
+
+extern "C" int qf_empty_launch(int64_t blocks, int64_t threads, void* stream_) {
+    if (blocks <= 0 || blocks > 0x7fffffff || threads <= 0 || threads > 1024) return fail("qf_empty_launch", "blocks positive, threads in 1..1024");
+    hipLaunchKernelGGL(empty_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0, (hipStream_t)stream_, (uint32_t*)nullptr);
+    return launched("qf_empty_launch");
+}
+
 extern "C" int qf_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream_) {
     if (!src || !sink) return fail("qf_stream_read", "null pointer");
     if (bytes == 0 || bytes % 16 != 0) return fail("qf_stream_read", "bytes must be a positive multiple of 16");

@@ -26,8 +26,10 @@ runtime_cache = RuntimeCache()
 DEFAULT_ARCH = "gfx950"
 _PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 INCLUDE_DIR = os.path.join(_PKG_DIR, "include")
-# C-ABI declarations live at <checkout>/include; present in a source checkout, optional otherwise.
-ABI_INCLUDE_DIR = os.path.normpath(os.path.join(_PKG_DIR, "..", "..", "include"))
+# C-ABI declarations: qfactory/abi in a built distribution (setup.py copies them there), <checkout>/include in a
+# source checkout; optional either way (the generated code includes them under __has_include).
+ABI_INCLUDE_DIR = (os.path.join(_PKG_DIR, "abi") if os.path.isdir(os.path.join(_PKG_DIR, "abi"))
+                   else os.path.normpath(os.path.join(_PKG_DIR, "..", "..", "include")))
 
 _lock = threading.Lock()
 _memo = {}

@@ -10,8 +10,11 @@ import subprocess
 import threading
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-CSRC_DIR = os.path.join(os.path.dirname(PKG_DIR), "csrc")
-REPO_INCLUDE = os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include")
+# sources and C-ABI headers: copies inside the package in a built distribution (setup.py), else the checkout's
+# csrc/ beside the package and include/ at the repository root
+CSRC_DIR = os.path.join(PKG_DIR, "csrc") if os.path.isdir(os.path.join(PKG_DIR, "csrc")) else os.path.join(os.path.dirname(PKG_DIR), "csrc")
+REPO_INCLUDE = (os.path.join(PKG_DIR, "abi") if os.path.isdir(os.path.join(PKG_DIR, "abi"))
+                else os.path.join(os.path.dirname(os.path.dirname(PKG_DIR)), "include"))
 SOURCES = [os.path.join(CSRC_DIR, "qfactory_hip.hip"), os.path.join(CSRC_DIR, "qfactory_decode.hip")]
 LIBRARY = os.path.join(CSRC_DIR, "libqfactory_hip.so")
 
@@ -28,6 +31,7 @@ SIGNATURES = {
     "qf_bf16_to_f16": (_INT, [_P, _P, _I64, _P]),
     "qf_stream_read": (_INT, [_P, _SZ, _P, _P]),
     "qf_stream_copy": (_INT, [_P, _P, _SZ, _P]),
+    "qf_empty_launch": (_INT, [_I64, _I64, _P]),
     "qf_add_rmsnorm": (_INT, [_P, _P, _P, _P, _I64, _I64, _F, _P]),
     "qf_rope_kv_store": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_decode_attention": (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
@@ -125,6 +129,11 @@ def bf16_to_f16(src, out=None):
 def stream_read(src, sink):
     assert sink.numel() * sink.element_size() >= 4096 * 4, "qf_stream_read writes one checksum word per block into 4096 words"
     _check(load().qf_stream_read(src.data_ptr(), src.numel() * src.element_size(), sink.data_ptr(), _stream()), "qf_stream_read")
+
+
+def empty_launch(blocks, threads):
+    """A kernel that does nothing: what a launch of that grid costs."""
+    _check(load().qf_empty_launch(blocks, threads, _stream()), "qf_empty_launch")
 
 
 def stream_copy(dst, src):

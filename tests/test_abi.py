@@ -28,7 +28,7 @@ def _declared_functions(header, guard=None):
 
 def test_header_parsers_see_the_expected_prototypes():
     assert _declared_functions("qfactory_hip.h") == sorted(
-        ["qf_version", "qf_pack_weight", "qf_pack_zero", "qf_transpose_scale", "qf_bf16_to_f16", "qf_stream_read", "qf_stream_copy",
+        ["qf_version", "qf_pack_weight", "qf_pack_zero", "qf_transpose_scale", "qf_bf16_to_f16", "qf_stream_read", "qf_stream_copy", "qf_empty_launch",
          "qf_add_rmsnorm", "qf_rope_kv_store", "qf_decode_attention", "qf_rope_decode_attention", "qf_silu_mul"])
     assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_GROUPED") == ["launch", "launch_m", "qf_describe"]
     assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_PLAIN") == ["launch", "qf_describe"]
@@ -73,3 +73,26 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(native, "LIBRARY", str(tmp_path / "absent.so"))
     with pytest.raises(RuntimeError, match="missing"):
         native.load()
+
+
+def test_built_distribution_carries_headers_and_native_sources(tmp_path):
+    """setup.py (the reference ships include/**/* as package data, setup.py:11-23): a built copy of the package holds
+    the kernel headers, the sources of libqfactory_hip.so and the C-ABI headers, where the package looks for them."""
+    import subprocess
+    import sys
+    pkg_parent = os.path.join(ROOT, "qfactory-ae_amd")
+    build = tmp_path / "build"
+    subprocess.run([sys.executable, "setup.py", "-q", "build", "--build-base", str(build)], cwd=pkg_parent, check=True,
+                   capture_output=True)
+    lib = build / "lib" / "qfactory"
+    for rel in ("include/qf_gemv.hip.h", "include/qf_gemm.hip.h", "include/qf_common.hip.h", "csrc/qfactory_hip.hip",
+                "csrc/qfactory_decode.hip", "abi/qfactory_launch.h", "abi/qfactory_hip.h", "jit/compiler.py", "core/tiling.py",
+                "integrations/vllm_qfactory.py"):
+        assert (lib / rel).exists(), rel
+    probe = ("import qfactory.native as n, qfactory.jit.compiler as c; "
+             "print(n.CSRC_DIR); print(n.REPO_INCLUDE); print(c.ABI_INCLUDE_DIR)")
+    out = subprocess.run([sys.executable, "-c", probe], cwd=str(tmp_path), check=True, capture_output=True, text=True,
+                         env=dict(os.environ, PYTHONPATH=str(build / "lib"))).stdout.split()
+    assert out == [str(lib / "csrc"), str(lib / "abi"), str(lib / "abi")]
+    import shutil
+    shutil.rmtree(os.path.join(pkg_parent, "qfactory.egg-info"), ignore_errors=True)
