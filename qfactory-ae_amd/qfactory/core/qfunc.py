@@ -148,8 +148,6 @@ class QMatmulQFunc(QFunc):
             return tiling.gemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "mgemv":
             return tiling.mgemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
-        if regime == "panel":
-            return tiling.panel_tiling(p["M"], p["N"], p["K"], nbits, gs, self.qtile_b.quant_method == "sym")
         if regime == "skinny":
             return tiling.skinny_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "gemm":
@@ -171,7 +169,6 @@ class QMatmulQFunc(QFunc):
         * dot2 GEMV: deferred (default) and eager in packed fp16.
         * A-stationary and streaming matrix-core kernels: deferred where a chunk of 512/b fields lies inside one
           group (the group sum is formed on the matrix core and scaled once in fp32), eager always.
-        * activation-panel kernel: deferred where groups are whole chunks, eager where they are narrower.
         * GEMM and the generic matrix-core kernel: eager only (dequantised fp16 fragments feed the MFMA)."""
         nbits, gs = self.qtile_b.nbits, self._gs
         chunk = 4 * (128 // tiling.plane_bits(nbits))
@@ -181,8 +178,6 @@ class QMatmulQFunc(QFunc):
             return ["deferred", "eager"] if gs % chunk == 0 else ["eager"]
         if self.regime == "skinny":
             return ["deferred", "eager"] if (gs >= 2 * chunk or gs == chunk) else ["eager"]
-        if self.regime == "panel":
-            return ["deferred"] if gs % chunk == 0 else ["eager"]
         return ["eager"]
 
     def transform(self) -> List[QFunc]:
@@ -198,8 +193,6 @@ class QMatmulQFunc(QFunc):
             cands = tiling.gemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         elif self.regime == "mgemv":
             cands = tiling.mgemv_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
-        elif self.regime == "panel":
-            cands = tiling.panel_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"], p["SYM"])
         elif self.regime == "skinny":
             cands = tiling.skinny_candidates(p["M"], p["N"], p["K"], p["NBITS"], p["GS"])
         elif self.regime == "gemm":
@@ -223,7 +216,7 @@ class QMatmulQFunc(QFunc):
                              f"for {p['NBITS']}-bit weights in groups of {p['GS']} (available: {self.decode_strategies()})")
         if self.decode_strategy == "eager" and self.regime in ("gemv", "mgemv", "skinny"):
             defines[{"gemv": "QF_GEMV_EAGER", "mgemv": "QF_MGEMV_EAGER", "skinny": "QF_SKINNY_EAGER"}[self.regime]] = 1
-        if self.regime in ("gemm", "mgemv", "skinny", "panel"):
+        if self.regime in ("gemm", "mgemv", "skinny"):
             # the matrix-core kernels expose their dequantisation's vector-instruction issue and have
             # registers to spare: the one-instruction mask-and-merge decode pays there (2 - 7 %
             # measured); it does not in the 4-bit GEMV kernel, where it costs a resident wave
@@ -261,10 +254,6 @@ class QMatmulQFunc(QFunc):
             code += '#include "qf_mgemv.hip.h"\n'
             cfg = tiling.mgemv_cfg_string(p, t, not self.l2cache_b)
             call = "qf::mgemv_launch<Cfg>"
-        elif self.regime == "panel":
-            code += '#include "qf_panel.hip.h"\n'
-            cfg = tiling.panel_cfg_string(p, t, not self.l2cache_b)
-            call = "qf::panel_launch<Cfg>"
         elif self.regime == "skinny":
             code += '#include "qf_skinny.hip.h"\n'
             cfg = tiling.skinny_cfg_string(p, t, not self.l2cache_b)

@@ -44,8 +44,6 @@ def regime_for(M, K=None, nbits=None, group_size=None, N=None):
     if not mfma_supported(K, nbits, group_size):
         # K is not a whole number of 16-byte lane loads: only the GEMM (64-element iterations) and the dot2 GEMV remain
         return "gemm" if M > GEMV_MAX_M and gemm_supported(K, nbits, group_size) else "gemv"
-    if N is not None and M <= PANEL_MAX_M and panel_tiling(M, N, K, nbits, group_size) is not None:
-        return "panel"
     if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
         return "mgemv"
     if skinny_preferred(M, K, nbits, group_size, N):
@@ -264,101 +262,6 @@ def mfma_cfg_string(problem, t, decode_strategy, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::MfmaCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
             f"{t['AT']}, {t['BT']}, {t['WM']}, {t['WN']}, {t['WK']}, {b(nt_b)}>")
-
-
-# --------------------------------------------------------------------------------------------
-# Activation-panel regime (3 <= M <= 16): activations in LDS, all waves of a block split K
-# --------------------------------------------------------------------------------------------
-
-PANEL_MAX_M = 16
-PANEL_MAX_KP = 4096            # 16 rows x 4096 fp16 columns = 128 KB of the 160 KB of LDS
-PANEL_MAX_STAGES = 40          # (panel, tile) pairs per block the kernel unrolls
-PANEL_ENABLED = False         # switched on once measured against the kernels it would replace
-
-
-def panel_supported(K, nbits, group_size, sym=False):
-    if nbits not in (2, 4, 8) or not group_size or group_size <= 0:
-        return False
-    epl = 128 // nbits
-    chunk = 4 * epl
-    if K % chunk or K % group_size or group_size % epl:
-        return False
-    if group_size % chunk and chunk % group_size:
-        return False
-    return sym or (K // group_size) % (8 // nbits) == 0
-
-
-def panel_lds_bytes(cfg, N, K, nbits, group_size, sym=False):
-    """LDS of qf::panel_kernel (PanelCfg::LDS_BYTES): the activation panel, the partial-tile slots (two sets when
-    they fit, else one), the partial tiles kept between panels and the two quantisation buffers."""
-    chunk = 4 * (128 // nbits)
-    kp, wv, d = cfg["KP"], cfg["WV"], cfg["D"]
-    npanel = -(-(K // chunk) // (kp // chunk))
-    nt = -(-N // 16)
-    slots = -(-nt // min(nt, cfg["PB"]))
-    lds_a = 16 * kp * 2
-    lds_ct = slots * 1024 if npanel > 1 else 0
-    pg = kp // group_size if kp % group_size == 0 else 0
-    g = K // group_size
-    sw, zb = pg // 2, pg * nbits // 8
-    qt = 16 * (sw + (0 if sym else zb))
-    qstage = pg > 0 and pg % 2 == 0 and g % 2 == 0 and (pg * nbits) % 8 == 0 and qt <= 64 * wv and d >= 2
-    lds_q = 2 * 4 * (16 * sw + (16 * zb + 3) // 4) if qstage else 0
-    sets = 2 if lds_a + lds_ct + lds_q + 2 * wv * 1024 <= 160 * 1024 else 1
-    return lds_a + lds_ct + lds_q + sets * wv * 1024
-
-
-def panel_tiling(M, N, K, nbits, group_size, sym=False, **pins):
-    """Default tiling of qf::panel_kernel, or None where the kernel does not apply: sixteen waves per block, the
-    widest activation panel that fits (fewest panels; among those the one with the least padding), the loads of
-    up to four tiles in flight per wave."""
-    if not PANEL_ENABLED or not panel_supported(K, nbits, group_size, sym) or M > PANEL_MAX_M:
-        return None
-    chunk = 4 * (128 // nbits)
-    unit = chunk if chunk % 128 == 0 else 128                      # a panel is whole chunks and a multiple of 128 columns
-    if group_size > unit and group_size % unit == 0:
-        unit = group_size                                          # whole groups per panel: scales go through LDS
-    if K % unit:
-        unit = chunk if chunk % 128 == 0 else 128
-    kp_cap = min(PANEL_MAX_KP, K) // unit * unit
-    if kp_cap < unit:
-        return None
-    npanel = -(-K // kp_cap)
-    kp = -(-K // npanel)                                           # evenest split into that many panels ...
-    kp = -(-kp // unit) * unit                                     # ... in whole units
-    nt = -(-N // 16)
-    slots = -(-nt // min(nt, NUM_CUS))
-    nstage = -(-K // kp) * slots
-    if nstage > PANEL_MAX_STAGES:
-        return None
-    for wv in (16, 8):                                             # eight waves where sixteen partial-tile slots do not fit
-        cfg = {"WV": wv, "D": max(2, min(4, nstage)), "KP": kp, "PB": NUM_CUS}
-        cfg.update(pins)
-        if panel_lds_bytes(cfg, N, K, nbits, group_size, sym) <= 160 * 1024:
-            return cfg
-    return None
-
-
-def panel_candidates(M, N, K, nbits, group_size, sym=False):
-    base = panel_tiling(M, N, K, nbits, group_size, sym)
-    if base is None:
-        return []
-    seen, out = set(), []
-    for wv in (16, 8):
-        for d in (2, 3, 4, 6):
-            cfg = dict(base, WV=wv, D=d)
-            key = tuple(sorted(cfg.items()))
-            if key not in seen and panel_lds_bytes(cfg, N, K, nbits, group_size, sym) <= 160 * 1024:
-                seen.add(key)
-                out.append(cfg)
-    out.sort(key=lambda c: c != base)
-    return out
-
-
-def panel_cfg_string(problem, t, nt_b):
-    b = lambda x: "true" if x else "false"
-    return (f"qf::PanelCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
-            f"{t['WV']}, {t['D']}, {t['KP']}, {t['PB']}, {b(nt_b)}>")
 
 
 # --------------------------------------------------------------------------------------------
