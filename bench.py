@@ -333,6 +333,8 @@ COPY_BYTES = 64 << 20
 # keyed by the description of the specialisation it was taken on, reported with that key, and null
 # for any other specialisation (profiles/gemv_w4g128_llama2_7b_m1_hbm_traffic_pmc.md holds the run).
 MEASURED_TRAFFIC = {
+    "regime=gemv M=1 N=22016 K=4096 NBITS=4 GS=128 SYM=0 decode=deferred nt_b=1 MT=1 STEPS=1 U=4 VB=16 WK=2 WN=2 "
+    "QF_FUSED_AND_OR=2 QF_GEMV_QUANT_DEDUP=1": 47041000,
 }
 
 

@@ -280,7 +280,10 @@ class QMatmulQFunc(QFunc):
                 + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
                 + ("epilogue=silu_mul " if self.output_epilogue == "silu_mul" else "")
                 + ("smem_quant=1 " if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none" else "")
-                + " ".join(f"{k}={v}" for k, v in sorted(t.items())))
+                + " ".join(f"{k}={v}" for k, v in sorted(t.items()))
+                # the header knobs that change the generated code and are not named above
+                + "".join(f" {k}={v}" for k, v in sorted(defines.items())
+                          if k in TUNING_DEFINES and k != "QF_GEMM_FULL_DRAIN"))
         wait_desc = " QF_GEMM_WAIT_DESC" if self.regime == "gemm" else ""    # string literal from the header: counted / drain
         code += f'extern "C" const char* qf_describe() {{ return "{desc}"{wait_desc}; }}\n'
         return code
