@@ -257,18 +257,20 @@ def dense_square_tflops(n=8192, reps=10):
     return 2.0 * n ** 3 * reps / (e0.elapsed_time(e1) * 1e-3) / 1e12
 
 
-def module_time_us(lins, x, reps=256):
+def module_time_us(lins, x, reps=256, out=None):
     """Average time of one eager ``layer(x)`` call -- output allocation, Python checks, ctypes and the launch, as the
     reference's latency harness times it (qfactory/testing.py:31-35) -- rotating over the layers' weight copies;
     wall clock around `reps` calls with a synchronisation on both sides.  At small M this is bound by the host
-    (the kernel is shorter than its enqueue), which is why the decode loop replays HIP graphs."""
+    (the kernel is shorter than its enqueue), which is why the decode loop replays HIP graphs.  With ``out``: the
+    same through ``layer.forward(x, out=out)``, i.e. without the allocator."""
     import torch
+    call = (lambda lin: lin(x)) if out is None else (lambda lin: lin.forward(x, out=out))
     for i in range(16):
-        lins[i % len(lins)](x)
+        call(lins[i % len(lins)])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(reps):
-        lins[i % len(lins)](x)
+        call(lins[i % len(lins)])
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / reps * 1e6
 
@@ -540,10 +542,12 @@ def main():
         rec["frac_of_stream_read"] = round(stream_us / us, 4)
         if not args.no_module_time:
             rec["module_us"] = round(module_time_us([layer[name] for layer in layers], acts[K]), 2)
+            rec["module_out_us"] = round(module_time_us([layer[name] for layer in layers], acts[K],
+                                                        out=torch.empty(M, N, dtype=torch.float16, device="cuda")), 2)
         shapes_report.append(rec)
         log(f"[bench] {name:8s} N={N:6d} K={K:6d}  {us:7.2f} us  {rec['GB/s']:7.1f} GB/s  {100 * rec['hbm_frac']:5.1f}% of HBM peak"
             f"  (a pure streaming read of the same bytes: {stream_us:.2f} us)"
-            + (f"  (eager layer(x): {rec['module_us']:.2f} us per call)" if "module_us" in rec else ""))
+            + (f"  (eager layer(x): {rec['module_us']:.2f} us per call, forward(x, out=...): {rec['module_out_us']:.2f})" if "module_us" in rec else ""))
         if name == DOMINANT:
             dominant = rec
     dense_tflops = dense_square_tflops()
