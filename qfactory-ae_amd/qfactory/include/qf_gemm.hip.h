@@ -18,7 +18,7 @@
 //     agree: lane (row, kb) takes the 32 consecutive k of half kb of a 64-wide K-iteration, k-step
 //     ks its eight fields 8*ks .. 8*ks+7, and the activation fragment is read to match.
 //   * Packed weights travel global -> registers -> LDS in supers of 128 bytes per row (eight lanes
-//     share a row: fully coalesced), two supers ahead of use, into a buffer private to the wave
+//     share a row: fully coalesced), one to two supers ahead of use, into a buffer private to the wave
 //     (no block barrier on that path); a lane then picks its 4*NBITS bytes per K-iteration with
 //     one LDS read.  The scales and zero-points of a super are loaded with it and stay in registers.
 //   * Activations go from global memory straight into LDS (global_load_lds_dwordx4: no register
@@ -59,6 +59,17 @@
 #define QF_GEMM_WAIT_DESC " waits=counted"
 #endif
 
+// When are the packed words of a super requested?  0: all of them in the last iteration of the super three before
+// it, into the register slot that has just gone to LDS.  n > 0: in n instalments (16-byte unit p in instalment
+// p % n), in the first n iterations of the super two before it.  Every wave of a block requesting a whole super in
+// the same iteration, next to that iteration's LDS hand-over and scale loads, was measured (clock stamps per
+// iteration) as ~1000 clocks every SUP iterations in which the waves queue behind each other's load instructions
+// and no MFMA runs; two instalments take 3 - 13 % off the 4-bit launches.  Supers of fewer than four iterations
+// (8 bits) keep the early whole-super request: they need its longer lead (12.4 against 14.2 us on 2048 x 2048 at M = 100).
+#ifndef QF_GEMM_SPREAD
+#define QF_GEMM_SPREAD 2
+#endif
+
 // 1: block -> tile map that keeps the slabs of one column of tiles together on one XCD (see the
 // kernel), 0: plain blockIdx order.  Measured no faster (358 vs 365 us on 57344 x 8192 at M = 256, slower
 // with two 32-row tiles per wave): the Infinity Cache already serves the second fetch.  Off.
@@ -92,6 +103,7 @@ struct GemmCfg {
     static constexpr bool HI = NBITS == 3;
     static constexpr int SUPK = 1024 / PB;                     // elements of K in 128 bytes of the main plane
     static constexpr int SUP = SUPK / BK;                      // K-iterations per super
+    static constexpr int SPREAD = (SUP < 4 || QF_GEMM_SPREAD < 1) ? 0 : (QF_GEMM_SPREAD < SUP ? QF_GEMM_SPREAD : SUP);   // instalments of a super's loads (0: one early request)
     // K need not be a whole number of supers: the last one may hold only TAIL_IT of its SUP iterations.  Its
     // 128-byte window (and those of the 1-bit plane, the scales and the zero-points) is then moved back to end
     // at the end of the row -- every load stays inside the row -- and iteration q of it reads position
@@ -167,13 +179,25 @@ __device__ __forceinline__ void load_to_lds_16(const void* global, void* lds) {
     __builtin_amdgcn_global_load_lds(global, (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
 }
 
+// Vector-memory loads of one super that a wave issues in iteration q of a super: its instalment of packed words
+// (and of the 1-bit plane), and in the last iteration the scales and zero-points.
+template <class C>
+constexpr int super_loads_at(int q) {
+    if (C::SPREAD == 0) return q == C::SUP - 1 ? C::SUPER_LOADS : 0;
+    int n = 0;
+    for (int p = 0; p < C::UPS; p++) n += (p % C::SPREAD == q) ? 1 : 0;
+    if (C::HI)
+        for (int p = 0; p < C::UPH; p++) n += (p % C::SPREAD == q) ? 1 : 0;
+    if (q == C::SUP - 1) n += C::NT32 * (C::SYM ? 1 : 2);
+    return n;
+}
 // Vector-memory loads a wave issues in the `back` iterations that end with iteration s (s counted
-// modulo the super): UA activation loads each, plus a whole super in the last iteration of a super.
+// modulo the super): UA activation loads each, plus that iteration's share of a super.
 template <class C>
 constexpr int loads_since(int s, int back) {
     int n = 0;
     for (int d = 0; d < back; d++)
-        n += C::UA + ((((s - d) % C::SUP + C::SUP) % C::SUP == C::SUP - 1) ? C::SUPER_LOADS : 0);
+        n += C::UA + super_loads_at<C>(((s - d) % C::SUP + C::SUP) % C::SUP);
     return n;
 }
 
@@ -279,7 +303,8 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     const uint8_t* w_rows = W + (size_t)n_base * C::RB;
     const uint8_t* s_rows = reinterpret_cast<const uint8_t*>(S + (size_t)n_base * C::G);
     const uint8_t* z_rows = Zp + (size_t)n_base * C::ZRB;
-    auto load_super = [&](WStage& st, int sup_local) {
+    // instalment `part` of the super (part < 0: all of it)
+    auto load_super = [&](WStage& st, int sup_local, int part) {
         if (QF_GEMM_EXPERIMENT & 32) return;
         const int sup = min(sup_local * WK + grp, C::NSUP - 1);
         // byte offset of the super's window in the main plane (half of it in the 1-bit plane); wave-uniform, and
@@ -289,6 +314,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         const uint8_t* wb = w_rows + woff;
 #pragma unroll
         for (int p = 0; p < UPS; p++) {
+            if (part >= 0 && p % (C::SPREAD ? C::SPREAD : 1) != part) continue;
             const uint8_t* src = wb + w_off[p];
             st.w[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
         }
@@ -296,6 +322,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
             const uint8_t* hb = w_rows + woff / 2;
 #pragma unroll
             for (int p = 0; p < C::UPH; p++) {
+                if (part >= 0 && p % (C::SPREAD ? C::SPREAD : 1) != part) continue;
                 const uint8_t* src = hb + h_off[p];
                 st.h[p] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)src) : *(const u32x4*)src;
             }
@@ -492,13 +519,16 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         if constexpr (C::PREFETCH_A) load_a(b0, min(it + C::PA, C::ITERS - 1));
         cur = nxt;
         if constexpr (C::PREFETCH_A) fcur = fnxt;
-        if (q == SUP - 1) {
-            // its register slot goes to the super two after it; the quantisation slot of the super
-            // that ends here goes to the one after next (no register is copied: a copy of a loaded
-            // value at the loop's back-edge would wait for every load in flight)
-            load_super(ringW[pslot ^ 1], P + 3);
-            load_quant(ringQ[pslot], P + 2);
+        // The register slot whose super went to LDS when this super began (slot pslot) takes the super two after
+        // this one, an instalment per iteration; the quantisation slot of the super that ends here goes to the
+        // one after next (no register is copied: a copy of a loaded value at the loop's back-edge would wait
+        // for every load in flight).
+        if constexpr (C::SPREAD > 0) {
+            if (q < C::SPREAD) load_super(ringW[pslot], P + 2, q);
+        } else {
+            if (q == SUP - 1) load_super(ringW[pslot ^ 1], P + 3, -1);          // the slot that went to LDS in this iteration
         }
+        if (q == SUP - 1) load_quant(ringQ[pslot], P + 2);
         // Publish the tile the next iteration reads (tile it+2 with fragment prefetch, else it+1).
         // Either way its request is PA - 2 whole iterations old, and every vector-memory load the
         // wave has issued in those iterations (activation tiles and whole supers) may stay in
@@ -507,15 +537,15 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
         wait_loads_and_barrier<QF_GEMM_FULL_DRAIN ? 0 : ((QF_GEMM_EXPERIMENT & (8 | 64)) ? 63 : loads_since<C>(s, C::PA - 2)), !(QF_GEMM_EXPERIMENT & 16)>();
     };
 
-    // ---- prologue: supers 0, 1 (then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----
-    load_super(ringW[0], 0);
+    // ---- prologue: supers 0, 1 (with the early request: then 2) and activation tiles 0 .. PA-1 requested, all complete at the barrier ----
+    load_super(ringW[0], 0, -1);
     load_quant(ringQ[0], 0);
-    load_super(ringW[1], 1);
+    load_super(ringW[1], 1, -1);
     load_quant(ringQ[1], 1);
 #pragma unroll
     for (int p = 0; p < (C::PREFETCH_A ? C::PA : C::PA - 1); p++) load_a(p, min(p, C::ITERS - 1));
     store_super(ringW[0]);
-    load_super(ringW[0], 2);
+    if constexpr (C::SPREAD == 0) load_super(ringW[0], 2, -1);
     read_packed(cur, is_tail(0) ? C::TAIL_SHIFT : 0);
     wait_loads_and_barrier<0>();
     if constexpr (C::PREFETCH_A) read_frags(fcur, 0);
