@@ -558,13 +558,40 @@ def gemm_supported(K, nbits, group_size):
     return gemm_valid(probe, K, nbits, group_size)
 
 
+_GEMM_TUNED = None
+
+
+def gemm_tuned(M, N, K, nbits, group_size):
+    """The winner of the on-device sweep over ``gemm_candidates`` for this exact problem, where the sweep was run
+    and beat the model below by 3 % or more (``gemm_tuned_gfx950.json`` beside this file: the reference times its
+    candidates at every first construction, qfunc.py:110-131; here that was done once for the reference's own
+    shape list at M = 32 .. 256, W4 g128).  None for any other problem."""
+    global _GEMM_TUNED
+    if _GEMM_TUNED is None:
+        import json
+        import os
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_tuned_gfx950.json")
+        try:
+            with open(path) as f:
+                _GEMM_TUNED = json.load(f)
+        except FileNotFoundError:
+            _GEMM_TUNED = {}
+    cfg = _GEMM_TUNED.get(f"{nbits}-{M}-{N}-{K}-{group_size}")
+    return dict(cfg) if cfg is not None and gemm_valid(cfg, K, nbits, group_size) else None
+
+
 def gemm_tiling(M, N, K, nbits, group_size, **pins):
-    """Default GEMM tiling from a small cost model fitted to on-device sweeps: a launch takes
+    """Default GEMM tiling: the swept winner where there is one (``gemm_tuned``), else a small cost model fitted to
+    on-device sweeps: a launch takes
     ceil(blocks / CUs) rounds of one tile's work, and a tile costs its area plus a fixed overhead
     (pipeline fill, reduction, barriers) worth about 2048 outputs.  It reproduces the measured
     winners: 64 x 128 tiles on 8192-wide, 128 x 128 on 10240-wide (160 tiles in one round beat 320
     in two) and 256 x 256 on 57344-wide layers at M = 256; 32 x 32 ... 64 x 64 tiles for M <= 128."""
     import math
+    cfg = gemm_tuned(M, N, K, nbits, group_size)
+    if cfg is not None:
+        cfg.update(pins)
+        return cfg
     if M >= 512:
         cfg = _gemm_tiling_many_rows(M, N, K, nbits, group_size)
         if cfg is not None:
@@ -588,28 +615,38 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     _, bm, wn, nt32, blocks = best
     # with at most one block per CU the K axis is split over wave groups inside the block, so
     # that every SIMD still holds two waves (one dequantises while the other multiplies)
-    wk = max(1, 8 // wn) if blocks <= NUM_CUS else 1
+    # (no more than four groups: eight groups of one wave leave LDS for three activation tiles per group only and
+    # measured slower than four groups with four tiles, 20.6 against 18.3 us on 8192 x 8192 at M = 32, 23.0 against
+    # 21.0 on 4096 x 11008 at M = 64)
+    wk = max(1, min(4, 8 // wn)) if blocks <= NUM_CUS else 1
     if bm == 256:
         wk = 1
-    if M >= 256 and (bm, wn, nt32) == (64, 4, 1) and wk == 2:
-        # one round of 64 x 128 tiles with two groups: a 64 x 64 wave tile (two 32-row weight tiles
-        # per wave) reuses every activation fragment twice; measured 59.7 against 62.6 us on
-        # 8192 x 8192 and 172 against 183 us on 8192 x 28672 at M = 256 (slower than four 64 x 32
-        # waves when blocks come in several rounds and there is only one group)
-        wn, nt32 = 2, 2
     nsup = -(-K // (1024 // plane_bits(nbits)))
     wk = max(1, min(wk, nsup))
-    pa = 4
+    # 128 x 256 block tiles of four 128 x 64 waves: three activation tiles in flight measured 128.7 against 156.7 us
+    # for four on 57344 x 8192 at M = 128 and the same on 22016 x 4096 at M = 256
+    pa_first = 3 if (bm, nt32, wn) == (128, 2, 4) else 4
+    pa = pa_first
     while not gemm_valid({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}, K, nbits, group_size):
         if pa == 4:
             pa = 3                                    # one activation tile less in LDS
         elif wk > 1:
-            wk, pa = wk // 2, 4
+            wk, pa = wk // 2, pa_first
         else:
             break
     cfg = {"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}
     cfg.update(pins)
     return cfg
+
+
+def gemm_tiling_model(M, N, K, nbits, group_size):
+    """The cost model's choice alone (what ``gemm_tiling`` returns for a problem that was never swept)."""
+    global _GEMM_TUNED
+    saved, _GEMM_TUNED = _GEMM_TUNED, {}
+    try:
+        return gemm_tiling(M, N, K, nbits, group_size)
+    finally:
+        _GEMM_TUNED = saved
 
 
 def _gemm_tiling_many_rows(M, N, K, nbits, group_size):

@@ -43,7 +43,7 @@ if __name__ == "__main__":
         description="QFactory quantized linear layers on MI355X (gfx950): hipcc JIT of hand-written HIP kernels",
         packages=["qfactory", "qfactory.core", "qfactory.jit", "qfactory.integrations"],
         package_dir={"": "."},
-        package_data={"qfactory": ["include/*.h"]},
+        package_data={"qfactory": ["include/*.h"], "qfactory.core": ["*.json"]},
         python_requires=">=3.9",
         cmdclass={"build_py": build_py_with_native_sources},
     )

@@ -1,6 +1,7 @@
 """Host-side tiling logic (no GPU): regime routing, and that every default tiling the package would
 compile satisfies the static limits its kernel checks at launch (registers, LDS, divisibility)."""
 import math
+import os
 
 import pytest
 
@@ -188,3 +189,20 @@ def test_timing_experiments_cannot_come_from_the_generator():
         q.emit()
     q.defines = {"QF_GEMV_WAVES_PER_EU": 4}
     assert "#define QF_GEMV_WAVES_PER_EU 4" in q.emit()
+
+
+def test_swept_gemm_tilings_are_valid_and_override_the_model():
+    """core/gemm_tuned_gfx950.json: every entry is a tiling the kernel accepts for its problem, differs from what the
+    cost model alone picks (or it would not be there), and is what ``gemm_tiling`` returns; any other problem gets
+    the model's choice."""
+    import json
+    path = os.path.join(os.path.dirname(tiling.__file__), "gemm_tuned_gfx950.json")
+    table = json.load(open(path))
+    assert table, "the shipped table is empty"
+    for key, cfg in table.items():
+        nbits, m, n, k, gs = (int(x) for x in key.split("-"))
+        assert set(cfg) == {"BM", "NT32", "WN", "WK", "PA"}, key
+        assert tiling.gemm_valid(cfg, k, nbits, gs), key
+        assert tiling.gemm_tiling(m, n, k, nbits, gs) == cfg, key
+        assert tiling.gemm_tiling_model(m, n, k, nbits, gs) != cfg, key
+    assert tiling.gemm_tiling(256, 8192 + 128, 8192, 4, 128) == tiling.gemm_tiling_model(256, 8192 + 128, 8192, 4, 128)
