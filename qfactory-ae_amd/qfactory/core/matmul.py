@@ -25,6 +25,7 @@ from .qtile import QTile, SymQTile, AsymQTile
 from .qfunc import QMatmulQFunc, MatmulQFunc, apply_config
 from ..convert import weight_row_bytes, zero_row_bytes
 from ..jit import jit
+from .. import fastpath
 
 logger = logging.getLogger(__name__)
 
@@ -216,6 +217,22 @@ class QMatmul:
             wp, sp, zp = weight.data_ptr(), scale.data_ptr(), zero.data_ptr()
             get_stream = _get_raw_stream
 
+            # With the native extension both forms of the call are one C++ call each: launch(activation, output)
+            # -> rc into the caller's tensor, launch.alloc(activation) -> a new output tensor.  Either hands an
+            # activation (or output) it was not bound for back to the checks of `inner`, which name the problem.
+            bound = None
+            if not convert_first and get_stream is not None and runtime._launch_m is not None:
+                bound = fastpath.bound_launch(runtime._launch_m, weight, scale, zero, True, n_out, k, dtype_a, device_index)
+            if bound is not None:
+                into = bound.into
+
+                def launch(activation, output):
+                    rc = into(activation, output, get_stream(device_index))
+                    return inner(activation, weight, output, scale, zero) if rc is None else rc
+
+                launch.alloc = lambda activation: bound(activation, get_stream(device_index))
+                return launch
+
             def launch(activation, output):
                 m = activation.shape[0]
                 if (activation.dim() != 2 or activation.shape[1] != k or output.shape != (m, n_out)
@@ -229,6 +246,7 @@ class QMatmul:
                 fn(m, activation.data_ptr(), wp, output.data_ptr(), sp, zp, stream, rc_ref)
                 return rc.value
 
+            launch.alloc = None
             return launch
 
         func = inner_sym if self.sym else inner
@@ -315,6 +333,19 @@ class Matmul:
             wp = weight.data_ptr()
             get_stream = _get_raw_stream
 
+            bound = None
+            if get_stream is not None:
+                bound = fastpath.bound_launch(fn, weight, None, None, False, n, k, dtype_a, device_index)
+            if bound is not None:
+                into = bound.into
+
+                def launch(activation, output):
+                    rc_native = into(activation, output, get_stream(device_index))
+                    return inner(activation, weight, output) if rc_native is None else rc_native
+
+                launch.alloc = lambda activation: bound(activation, get_stream(device_index))
+                return launch
+
             def launch(activation, output):
                 m = activation.shape[0]
                 if (activation.dim() != 2 or activation.shape[1] != k or output.shape != (m, n)
@@ -326,6 +357,7 @@ class Matmul:
                 fn(m, activation.data_ptr(), wp, output.data_ptr(), stream, rc_ref)
                 return rc.value
 
+            launch.alloc = None
             return launch
 
         inner.runtime = runtime

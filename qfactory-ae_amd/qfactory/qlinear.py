@@ -111,14 +111,20 @@ class GPTQLinear(torch.nn.Module):
         allocates, qlinear.py:53): a preallocated contiguous ``(M, N)`` tensor to write into, e.g. under HIP-graph
         capture or in a loop that reuses its buffers."""
         m, dtype = x.shape[0], x.dtype
+        launch = None
+        if m > 0:
+            launch = self._launchers.get((m, dtype))
+            if launch is None:
+                launch = self._launcher(m, dtype)
         if out is None:
+            if launch is not None and launch.alloc is not None:
+                out = launch.alloc(x)                      # allocation and launch in one native call
+                if out is not None:
+                    return out
             out = torch.empty((m, self.out_features), dtype=dtype, device=x.device)
         if m == 0:
             assert out.shape == (0, self.out_features)
             return out                                     # no rows: nothing to launch
-        launch = self._launchers.get((m, dtype))
-        if launch is None:
-            launch = self._launcher(m, dtype)
         rc = launch(x, out)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")
@@ -207,14 +213,18 @@ class GEMVLinear(torch.nn.Module):
 
     def forward(self, x: torch.Tensor, out: torch.Tensor = None):
         m, dtype = x.shape[0], x.dtype
+        launch = self._launchers.get(dtype)
+        if launch is None:
+            launch = self._launchers[dtype] = self.func_for(dtype).bind(self.w)
         if out is None:
+            if launch.alloc is not None:
+                out = launch.alloc(x)                      # allocation and launch in one native call
+                if out is not None:
+                    return out
             out = torch.empty((m, self.out_features), dtype=dtype, device=x.device)
         if m == 0:
             assert out.shape == (0, self.out_features)
             return out
-        launch = self._launchers.get(dtype)
-        if launch is None:
-            launch = self._launchers[dtype] = self.func_for(dtype).bind(self.w)
         rc = launch(x, out)
         if rc != 0:
             raise RuntimeError(f"quantized linear launch failed with return code {rc}")

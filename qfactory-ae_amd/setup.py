@@ -2,7 +2,8 @@
 
 Counterpart of the reference's setup.py (setup.py:11-23: packages qfactory, qfactory/core, qfactory/jit with
 ``include/**/*`` as package data).  Besides the kernel headers the package needs, at run time, the sources of
-libqfactory_hip.so (``csrc/*.hip``, compiled by ``qfactory.native.build()`` with hipcc) and the C-ABI headers the
+libqfactory_hip.so (``csrc/*.hip``, compiled by ``qfactory.native.build()`` with hipcc), the source of the
+allocate-and-launch extension (``csrc/qf_fastpath.cpp``, ``qfactory.fastpath.build()``) and the C-ABI headers the
 generated translation units include (``<checkout>/include/*.h``).  In a checkout both live outside the package
 directory; a built distribution carries copies inside it (``qfactory/csrc``, ``qfactory/abi``), which is where
 ``qfactory.native`` and ``qfactory.jit.compiler`` look first.
@@ -26,6 +27,7 @@ class build_py_with_native_sources(build_py):
         super().run()
         pkg = os.path.join(self.build_lib, "qfactory")
         for sub, pattern in (("csrc", os.path.join(HERE, "csrc", "*.hip")),
+                             ("csrc", os.path.join(HERE, "csrc", "*.cpp")),
                              ("abi", os.path.join(HERE, "..", "include", "*.h"))):
             os.makedirs(os.path.join(pkg, sub), exist_ok=True)
             for path in glob.glob(pattern):
