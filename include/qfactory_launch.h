@@ -55,6 +55,18 @@ typedef void (*qf_launch_grouped_m_fn)(int m, void* activation, void* weight, vo
 typedef void (*qf_launch_plain_fn)(int m, void* activation, void* weight, void* output, void* stream,
                                    int* return_code);
 
+/*
+ * Grouped-scale kernel with the decoder layer's residual add and RMSNorm in front of its dot products (few rows;
+ * fp16):  h = fp16(activation + delta)  (delta may be null),  a = fp16(fp16(h * rsqrt(mean(h^2) + eps)) * gamma),
+ * output = a x dequant(weight)^T;  x_out (may be null; must not alias activation or delta) receives h.
+ * gamma is the (K) fp16 RMSNorm weight.  Exported, besides launch / launch_m (which return 1: no norm operands),
+ * by objects generated with the "add_rmsnorm" input prologue.  No counterpart in the reference, whose end-to-end
+ * runs leave the step to vLLM's fused_add_rms_norm (third_party/vllm-qfactory.patch:205-214 calls the linear alone).
+ */
+typedef void (*qf_launch_grouped_norm_fn)(int m, void* activation, void* delta, void* gamma, void* x_out, float eps,
+                                          void* weight, void* output, void* scale, void* zero, void* stream,
+                                          int* return_code);
+
 /* Static string naming the specialisation ("regime=gemv M=1 N=4096 K=4096 NBITS=4 ..."). */
 typedef const char* (*qf_describe_fn)(void);
 
@@ -67,6 +79,11 @@ const char* qf_describe(void);
 #elif defined(QF_LAUNCH_PLAIN)
 void launch(int m, void* _activation, void* _weight, void* _output, void* _stream, QF_RC_ARG __return_code);
 const char* qf_describe(void);
+#endif
+
+#if defined(QF_LAUNCH_NORM)
+void launch_norm(int m, void* _activation, void* _delta, void* _gamma, void* _x_out, float eps, void* _weight,
+                 void* _output, void* _scale, void* _zero, void* _stream, QF_RC_ARG __return_code);
 #endif
 
 #ifdef __cplusplus

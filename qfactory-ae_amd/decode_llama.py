@@ -13,7 +13,8 @@ RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plai
 replaces its norm and SiLU steps by single launches.  A decode
 step runs the steps between the linears as one HIP launch each (residual add + RMSNorm, RoPE + cache
 append + attention of the new position, SiLU * up: libqfactory_hip.so) -- eight launches per layer
-instead of about fifty; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
+instead of about fifty -- and, for one or two sequences, five: the dot2 GEMV kernel then runs the residual add and
+RMSNorm in front of its dot products and SiLU * up behind them; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
 Prints one JSON line per batch size: tokens/s over the decode phase, prefill time, and the share of
@@ -88,9 +89,14 @@ class QuantLlama:
         ang = torch.arange(shape.max_len, device="cuda", dtype=torch.float32)[:, None] * inv[None, :]
         self.cos, self.sin = ang.cos(), ang.sin()                                   # (max_len, hd/2) fp32
         self.linear = lambda lin, x: lin(x)                 # hook: tests swap in a dense fp32 evaluation
+        self._own_linear = self.linear
+        # residual add + RMSNorm inside the projection that follows them, where its kernel can (few rows); False
+        # keeps them a launch of their own
+        self.fuse_norm = True
         # buffers of the fused decode step (one new position per sequence)
         f16 = dict(dtype=torch.float16, device="cuda")
         self._hdn, self._att = (torch.empty(batch, h, **f16) for _ in range(2))
+        self._res = [torch.empty(batch, h, **f16) for _ in range(2)]      # the residual stream alternates between the two
 
     def _norm(self, x, w):
         xf = x.float()
@@ -163,6 +169,26 @@ class QuantLlama:
         shape = self.shape
         x = self.embed[tok[:, 0]]                                # (B, h): the residual stream, updated in place
         delta = None
+        first = self.layers[0]
+        if (self.fuse_norm and self.linear is self._own_linear and first["qkv"].fuses_add_rmsnorm(x.shape[0])
+                and first["gate_up"].fuses_add_rmsnorm(x.shape[0], silu_mul=True)):
+            # five launches per layer: the two residual adds and norms run inside the projections behind them, each
+            # writing the new residual stream to the buffer the old one is not in
+            turn = 0
+            for li, layer in enumerate(self.layers):
+                if delta is None:
+                    qkv = layer["qkv"].forward_add_rmsnorm(x, None, layer["norm1"], shape.eps)
+                else:
+                    qkv = layer["qkv"].forward_add_rmsnorm(x, delta, layer["norm1"], shape.eps, x_out=self._res[turn])
+                    x, turn = self._res[turn], turn ^ 1
+                native.rope_decode_attention(qkv, pos, self.cos, self.sin, self.k_cache[li], self.v_cache[li], self._att)
+                delta = layer["o"](self._att)
+                act = layer["gate_up"].forward_add_rmsnorm(x, delta, layer["norm2"], shape.eps, x_out=self._res[turn],
+                                                           silu_mul=True)
+                x, turn = self._res[turn], turn ^ 1
+                delta = layer["down"](act)
+            native.add_rmsnorm(x, delta, self.final_norm, self._hdn, shape.eps)
+            return self._hdn @ self.lm_head.T
         for li, layer in enumerate(self.layers):
             native.add_rmsnorm(x, delta, layer["norm1"], self._hdn, shape.eps)
             qkv = self.linear(layer["qkv"], self._hdn)
@@ -258,7 +284,10 @@ def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
             "prefill_tokens_per_s": round(batch * prompt_len / prefill_s, 1),
             "quantized_linears_us_per_step": round(lin_us, 1), "quantized_linear_share": round(lin_us / step_us, 3),
             "layers": shape.layers, "hidden": shape.hidden, "data": "random weights, random prompt ids",
-            "between_linears": "torch ops" if torch_glue else "one HIP launch per step (libqfactory_hip.so)"}
+            "between_linears": "torch ops" if torch_glue else (
+                "attention one HIP launch (libqfactory_hip.so); residual add + RMSNorm and SiLU * up inside the projections"
+                if model.layers[0]["gate_up"].fuses_add_rmsnorm(batch, silu_mul=True) and model.fuse_norm
+                else "one HIP launch per step (libqfactory_hip.so)")}
 
 
 def main():

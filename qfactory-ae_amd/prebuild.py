@@ -208,6 +208,25 @@ def silu_mul_cases():
     return [dict(c, epilogue="silu_mul") for c in cases]
 
 
+def norm_prologue_cases():
+    """Projections that run the residual add and RMSNorm in front of their dot products
+    (GPTQLinear.forward_add_rmsnorm, dot2 GEMV rows): the decode loop's qkv and gate+up at batch 1 and 2, the tiny
+    test model's, and the shapes of tests/test_norm_prologue_gpu.py (every bit width, symmetric and not, a team
+    whose last lanes own no chunk, two chunks per lane, one wave per team and several; with and without the SwiGLU
+    epilogue)."""
+    cases = [dict(_case(M, 12288, 4096), prologue="add_rmsnorm") for M in (1, 2)]
+    cases += [dict(_case(M, 22016, 4096), prologue="add_rmsnorm", epilogue="silu_mul") for M in (1, 2)]
+    cases += [dict(_case(2, 768, 256, 4, 64), prologue="add_rmsnorm"),
+              dict(_case(2, 1024, 256, 4, 64), prologue="add_rmsnorm", epilogue="silu_mul")]
+    for c in (_case(1, 100, 1024), _case(2, 77, 512, 3, 64, True), _case(1, 130, 2048, 8, 128, True),
+              _case(1, 48, 4096, 2, 128), _case(2, 96, 2816, 4, 128), _case(1, 64, 11008, 4, 128),
+              _case(1, 40, 28672, 4, 128), _case(2, 50, 512, 4, 16)):
+        cases.append(dict(c, prologue="add_rmsnorm"))
+    for c in (_case(1, 100, 1024), _case(2, 154, 512, 3, 64), _case(1, 260, 2048, 8, 128), _case(2, 96, 2816, 2, 128, True)):
+        cases.append(dict(c, prologue="add_rmsnorm", epilogue="silu_mul"))
+    return cases
+
+
 def search_cases():
     """Problems whose whole tiling search space is compiled (tests/test_tune.py searches on the device)."""
     return [_case(1, 64, 256, 4, 128)]
@@ -233,7 +252,7 @@ def drain_cases(base=None):
 def all_cases(with_drain=True):
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases()):
+              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
@@ -272,9 +291,10 @@ def qfuncs_of(case):
         qfuncs += eager
     if case.get("drain"):
         qfuncs += [q.clone(defines={"QF_GEMM_FULL_DRAIN": 1}) for q in list(qfuncs) if q.regime == "gemm"]
-    if case.get("epilogue") == "silu_mul":
+    if case.get("epilogue") == "silu_mul" or case.get("prologue"):
         op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
-                     torch.float16, torch.int8, case["GS"], output_epilogue="silu_mul")
+                     torch.float16, torch.int8, case["GS"], output_epilogue=case.get("epilogue", "none"),
+                     input_prologue=case.get("prologue", "none"))
         op.init_qfuncs()
         qfuncs += op.qfuncs
     return qfuncs

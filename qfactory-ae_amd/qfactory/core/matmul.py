@@ -13,6 +13,7 @@ same argument lists and checks.  Differences that matter to callers:
   are then bf16, scales stay fp16.  The kernels compute on fp16 pairs either way; bf16 activations are
   converted as they are loaded, or, for the GEMM kernel, by one ``qf_bf16_to_f16`` launch before it.
 """
+import ctypes
 import json
 import logging
 import os
@@ -88,8 +89,13 @@ def _pick_best(runtimes, qfuncs, dummy_inputs, what):
 class QMatmul:
     def __init__(self, m: int, n: int, k: int, nbits: int, sym: bool, dtype_a, dtype_b,
                  group_size: int = -1, layout: str = "nt", base_impl: bool = False,
-                 output_epilogue: str = "none"):
+                 output_epilogue: str = "none", input_prologue: str = "none"):
         self.m, self.n, self.k = m, n, k
+        # "add_rmsnorm" (beyond the reference): the closure takes the residual stream, the previous block's output and
+        # the RMSNorm weight instead of ready activations -- closure(activation, delta, gamma, x_out, eps, weight,
+        # output, scale, zero=None); rows of the dot2 GEMV kernel only (M < 3), fp16 only
+        self.input_prologue = input_prologue
+        assert input_prologue in ("none", "add_rmsnorm")
         # "silu_mul" (beyond the reference): the weight is a fused gate+up projection and the closure's output is
         # the (M, N/2) SwiGLU activation fp16(silu(gate)) * up; M <= 32 only (dot2 GEMV and A-stationary kernels), fp16 only
         self.output_epilogue = output_epilogue
@@ -125,6 +131,7 @@ class QMatmul:
             tile_b((self.n, self.k), self.dtype_b, self.nbits, (1, self.group_size)),
             "nt", self.base_impl)]
         self.qfuncs[0].output_epilogue = self.output_epilogue
+        self.qfuncs[0].input_prologue = self.input_prologue
 
     def get_dummy_inputs(self):
         require_gpu()
@@ -138,6 +145,9 @@ class QMatmul:
     def compile_profile(self, enable_transform: bool = False, enable_schedule: bool = False,
                         enable_lower: bool = False):
         self.init_qfuncs()
+        if self.input_prologue != "none":
+            # the candidates are timed through `launch`, which these objects answer with 1: no search, the default tiling
+            enable_transform = enable_schedule = enable_lower = False
         shape = f"{self.nbits}-{self.m}-{self.n}-{self.k}-{self.group_size}"
         predefined = _load_predefined(shape)
         if predefined is not None:
@@ -202,6 +212,35 @@ class QMatmul:
 
         def inner_sym(activation, weight, output, scale):
             return inner(activation, weight, output, scale, zero_empty)
+
+        def inner_norm(activation, delta, gamma, x_out, eps, weight, output, scale, zero=None):
+            """Objects with the residual-add + RMSNorm prologue: ``activation`` is the residual stream, ``delta`` what
+            is added to it first (or None), ``x_out`` receives the sum (or None)."""
+            if zero is None:
+                zero = zero_empty
+            assert activation.shape[1] == k and output.shape[1] == n_out and activation.shape[0] == output.shape[0]
+            assert activation.dtype == torch.float16 and output.dtype == torch.float16
+            assert activation.is_contiguous() and output.is_contiguous() and activation.is_cuda and output.is_cuda
+            assert gamma.shape == (k,) and gamma.dtype == torch.float16 and gamma.is_contiguous() and gamma.is_cuda
+            for other in (delta, x_out):
+                if other is not None:
+                    assert other.shape == activation.shape and other.dtype == torch.float16
+                    assert other.is_contiguous() and other.is_cuda
+            if x_out is not None:
+                assert x_out.data_ptr() != activation.data_ptr(), "x_out must not alias the residual stream it is computed from"
+                assert delta is None or x_out.data_ptr() != delta.data_ptr(), "x_out must not alias delta"
+            check_packed(weight, scale, zero)
+            rc = ctypes.c_int(0)
+            runtime._launch_norm(activation.shape[0], activation.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                 gamma.data_ptr(), x_out.data_ptr() if x_out is not None else None, float(eps),
+                                 weight.data_ptr(), output.data_ptr(), scale.data_ptr(), zero.data_ptr(),
+                                 _raw_stream(activation), ctypes.byref(rc))
+            return rc.value
+
+        if self.input_prologue == "add_rmsnorm":
+            assert runtime._launch_norm is not None, "the compiled object does not export launch_norm"
+            inner_norm.runtime = runtime
+            return inner_norm
 
         def bind(weight, scale, zero=None):
             """The packed tensors of a layer never change between calls: validate them once and return

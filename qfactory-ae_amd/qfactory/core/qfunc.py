@@ -122,6 +122,9 @@ class QMatmulQFunc(QFunc):
         # "silu_mul": the weight is a fused gate+up projection and the kernel writes the (M, N/2) SwiGLU activation
         # fp16(silu(gate)) * up instead of the (M, N) projection (the kernels for M <= 32; not in the reference)
         self.output_epilogue = "none"
+        # "add_rmsnorm": the kernel makes its activations itself -- residual add and RMSNorm of a decoder layer run in
+        # front of the dot products -- and the object exports launch_norm (dot2 GEMV kernel, fp16; not in the reference)
+        self.input_prologue = "none"
         assert qtile_a.dtype in (torch.float16, torch.bfloat16), f"Data type {qtile_a.dtype} is not supported for A"
 
     @property
@@ -241,6 +244,10 @@ class QMatmulQFunc(QFunc):
             assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
                 "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, write silu(gate) * up"
             defines["QF_GEMV_GATE_UP_SILU" if self.regime == "gemv" else "QF_MGEMV_GATE_UP_SILU"] = 1
+        if self.input_prologue != "none":
+            assert self.input_prologue == "add_rmsnorm" and self.regime == "gemv" and self.act_dtype == torch.float16, \
+                "only the dot2 GEMV kernel, on fp16, runs the residual add and RMSNorm in front of its dot products"
+            defines["QF_GEMV_NORM_PROLOGUE"] = 1
         if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none":
             defines["QF_GEMV_SMEM_QUANT"] = 1
         for name, value in sorted(defines.items()):
@@ -268,16 +275,26 @@ class QMatmulQFunc(QFunc):
             call = "qf::mfma_launch<Cfg>"
         else:
             raise ValueError(f"unknown regime {self.regime}")
-        code += '#if __has_include("qfactory_launch.h")\n#define QF_LAUNCH_GROUPED 1\n#include "qfactory_launch.h"\n#endif\n\n'
+        norm_abi = "#define QF_LAUNCH_NORM 1\n" if self.input_prologue == "add_rmsnorm" else ""
+        code += f'#if __has_include("qfactory_launch.h")\n#define QF_LAUNCH_GROUPED 1\n{norm_abi}#include "qfactory_launch.h"\n#endif\n\n'
         code += f"using Cfg = {cfg};\nconstexpr int M = {p['M']};\n\n"
         args = "_activation, _weight, _output, _scale, _zero"
         code += self._signature("launch", leading_m=False)
         code += f"\t__return_code = {call}({args}, M, (hipStream_t)_stream);\n}}\n\n"
         code += self._signature("launch_m", leading_m=True)
         code += f"\t__return_code = {call}({args}, m, (hipStream_t)_stream);\n}}\n\n"
+        if self.input_prologue == "add_rmsnorm":
+            # the entry point of this object (launch / launch_m return 1: they carry no norm operands)
+            code += ('extern "C" void launch_norm (\n\tint m,\n\tvoid* _activation,\n\tvoid* _delta,\n\tvoid* _gamma,\n'
+                     '\tvoid* _x_out,\n\tfloat eps,\n\tvoid* _weight,\n\tvoid* _output,\n\tvoid* _scale,\n\tvoid* _zero,\n'
+                     '\tvoid* _stream,\n\tint& __return_code\n) {\n'
+                     '\tqf::GemvNormArgs norm;\n\tnorm.delta = (const uint16_t*)_delta;\n\tnorm.gamma = (const uint16_t*)_gamma;\n'
+                     '\tnorm.x_out = (uint16_t*)_x_out;\n\tnorm.eps = eps;\n'
+                     f'\t__return_code = _gamma == nullptr ? 1 : {call}({args}, m, (hipStream_t)_stream, norm);\n}}\n\n')
         desc = (f"regime={self.regime} M={p['M']} N={p['N']} K={p['K']} NBITS={p['NBITS']} GS={p['GS']} "
                 f"SYM={int(p['SYM'])} decode={self.decode_strategy} nt_b={int(not self.l2cache_b)} "
                 + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
+                + ("prologue=add_rmsnorm " if self.input_prologue == "add_rmsnorm" else "")
                 + ("epilogue=silu_mul " if self.output_epilogue == "silu_mul" else "")
                 + ("smem_quant=1 " if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none" else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items()))

@@ -93,6 +93,17 @@ struct GemvCfg {
 #define QF_GEMV_GATE_UP_SILU 0
 #endif
 
+// 1: the kernel's activations are not read but made: residual add and RMSNorm of the decoder layer run in front of
+// the dot products,  h = fp16(x + delta),  a = fp16(fp16(h * rsqrt(mean(h^2) + eps)) * gamma)  -- the roundings of
+// qf_add_rmsnorm in libqfactory_hip.so, which this replaces for few rows.  Every team holds a whole activation row
+// in its lanes (that is the kernel's mapping), so the sum of squares is one butterfly and one exchange through LDS,
+// done by every block for itself while its first weights are in flight; the first team of block (0, y) also
+// writes h to x_out, the next residual stream (a buffer of its own: other blocks still read x and delta).
+// fp16 only.  Not in the reference, whose end-to-end runs leave the norm to vLLM's fused_add_rms_norm.
+#ifndef QF_GEMV_NORM_PROLOGUE
+#define QF_GEMV_NORM_PROLOGUE 0
+#endif
+
 // 1: the scales and zero-points of the block's rows go through LDS (the reference's SMEM_QUANT choice,
 // qfactory/include/gptq_gemv.h:62-82): the rows of a block are contiguous in both tensors, so the block fetches
 // them with coalesced loads issued ahead of everything else, and a lane reads its group's pair from LDS instead
@@ -121,10 +132,18 @@ struct GemvCfg {
 #define QF_GEMV_OCCUPANCY
 #endif
 
+// Operands of the norm prologue (ignored by kernels compiled without it).
+struct GemvNormArgs {
+    const uint16_t* delta = nullptr;   // (M, K) fp16 added to the activation rows first, or null
+    const uint16_t* gamma = nullptr;   // (K) fp16 RMSNorm weight
+    uint16_t* x_out = nullptr;         // (M, K) fp16: receives x + delta, or null
+    float eps = 0.0f;
+};
+
 template <class C>
 __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
-    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
+    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total, GemvNormArgs norm) {
     using D = Decode<C::NBITS>;
     constexpr int NW = C::NW, EPC = C::EPC, NCH = C::NCH, T = C::T, IT = C::IT;
     constexpr int MT = C::MT, U = C::U, STEPS = C::STEPS, V = C::V, WK = C::WK;
@@ -134,6 +153,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
     constexpr int NWH = C::NWH;
     constexpr bool SILU = QF_GEMV_GATE_UP_SILU != 0;
+    constexpr bool NORM = QF_GEMV_NORM_PROLOGUE != 0;
     constexpr bool EAGER = QF_GEMV_EAGER != 0 && C::QPARAM;
     constexpr bool SMEMQ = QF_GEMV_SMEM_QUANT != 0 && C::QPARAM;
     constexpr int LPG = C::QPARAM ? C::GS / EPC : 1;                              // lanes per group
@@ -145,6 +165,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
 
     __shared__ uint32_t sq_s[SQ_WORDS], sq_z[ZQ_WORDS];
     __shared__ float red[C::WN][WK][STEPS * V];
+    __shared__ float norm_ss[NORM ? C::WN : 1][NORM ? WK : 1][MT];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -271,6 +292,79 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         }
     }
     if constexpr (QF_GEMV_A_FIRST) load_stage(st0, 0);
+    if constexpr (NORM) {
+        static_assert(!QF_IN_BF16, "the norm prologue is fp16 only");
+        // ---- residual add, sum of squares, normalisation: a[][][] becomes the normalised row ----
+        uint32_t gam[IT][AR];
+#pragma unroll
+        for (int it = 0; it < IT; it++) {
+            const uint16_t* gp = norm.gamma + (size_t)(coff[it] / C::VB) * EPC;
+#pragma unroll
+            for (int r = 0; r < AR; r += (AR >= 4 ? 4 : AR)) {
+                constexpr int LW = AR >= 4 ? 4 : AR;
+                uint32_t tmp[LW];
+                load_words<LW, false>(gp + 2 * r, tmp);
+#pragma unroll
+                for (int j = 0; j < LW; j++) gam[it][r + j] = tmp[j];
+            }
+        }
+        float ss[MT];
+        const bool writer = norm.x_out != nullptr && blockIdx.x == 0 && team == 0;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            ss[m] = 0.0f;
+            const int mm = min(m0 + m, m_total - 1);
+#pragma unroll
+            for (int it = 0; it < IT; it++) {
+                const size_t eoff = (size_t)mm * C::K + (size_t)(coff[it] / C::VB) * EPC;
+                if (norm.delta != nullptr) {
+#pragma unroll
+                    for (int r = 0; r < AR; r += (AR >= 4 ? 4 : AR)) {
+                        constexpr int LW = AR >= 4 ? 4 : AR;
+                        uint32_t tmp[LW];
+                        load_words<LW, false>(norm.delta + eoff + 2 * r, tmp);
+#pragma unroll
+                        for (int j = 0; j < LW; j++)
+                            a[m][it][r + j] = __builtin_bit_cast(uint32_t, as_f16x2(a[m][it][r + j]) + as_f16x2(tmp[j]));
+                    }
+                }
+                if (writer && cvalid[it] && m0 + m < m_total) {
+#pragma unroll
+                    for (int r = 0; r < AR; r++) reinterpret_cast<uint32_t*>(norm.x_out + eoff)[r] = a[m][it][r];
+                }
+#pragma unroll
+                for (int r = 0; r < AR; r++) {
+                    if (!cvalid[it]) a[m][it][r] = 0u;
+                    ss[m] = __builtin_amdgcn_fdot2(as_f16x2(a[m][it][r]), as_f16x2(a[m][it][r]), ss[m], false);
+                }
+            }
+            ss[m] += lane_xor<1>(ss[m]);
+            ss[m] += lane_xor<2>(ss[m]);
+            ss[m] += lane_xor<4>(ss[m]);
+            ss[m] += lane_xor<8>(ss[m]);
+            ss[m] += lane_xor<16>(ss[m]);
+            ss[m] += lane_xor<32>(ss[m]);
+            if (lane == 0) norm_ss[team][wk][m] = ss[m];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            float total = 0.0f;
+#pragma unroll
+            for (int w2 = 0; w2 < WK; w2++) total += norm_ss[team][w2][m];
+            const float rn = rsqrtf(total / (float)C::K + norm.eps);
+#pragma unroll
+            for (int it = 0; it < IT; it++)
+#pragma unroll
+                for (int r = 0; r < AR; r++) {
+                    const f16x2 h = as_f16x2(a[m][it][r]);
+                    f16x2 n;
+                    n.x = (_Float16)((float)h.x * rn);
+                    n.y = (_Float16)((float)h.y * rn);
+                    a[m][it][r] = __builtin_bit_cast(uint32_t, n * as_f16x2(gam[it][r]));
+                }
+        }
+    }
     if constexpr (SMEMQ) {
 #pragma unroll
         for (int i = 0; i < SQ_PER; i++)
@@ -490,7 +584,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
 // Host launcher: static validity checks (return 1 and say why on stderr), then the launch.
 template <class C>
 int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m,
-                hipStream_t stream) {
+                hipStream_t stream, GemvNormArgs norm = GemvNormArgs{}) {
     const char* why = nullptr;
     if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8";
     else if (C::VB != 4 && C::VB != 8 && C::VB != 16) why = "VB must be 4, 8 or 16";
@@ -508,6 +602,10 @@ int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const v
         why = "scales through LDS: a block's scales and zero-points must be whole 32-bit words";
     else if (QF_GEMV_SMEM_QUANT && C::QPARAM && (size_t)C::RPB * C::G * 2 + (size_t)C::RPB * C::ZRB + sizeof(float) * C::WN * C::WK * C::STEPS * C::V > 64 * 1024) why = "scales through LDS exceed LDS";
     else if (C::WN * C::WK * C::STEPS * C::V * 4 > 64 * 1024) why = "reduction scratch exceeds LDS";
+    else if (QF_GEMV_NORM_PROLOGUE && (QF_IN_BF16 || QF_OUT_BF16)) why = "the norm prologue is fp16 only";
+    else if (QF_GEMV_NORM_PROLOGUE && norm.gamma == nullptr) why = "an object with the norm prologue is called through launch_norm (RMSNorm weight missing)";
+    else if (!QF_GEMV_NORM_PROLOGUE && norm.gamma != nullptr) why = "this object was compiled without the norm prologue";
+    else if (QF_GEMV_NORM_PROLOGUE && (norm.x_out == A || (norm.x_out != nullptr && norm.x_out == norm.delta))) why = "x_out must be a buffer of its own: other blocks still read x and delta";
     if (why) {
         fprintf(stderr, "qfactory gemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT=%d WK=%d WN=%d U=%d STEPS=%d VB=%d)\n",
                 why, C::NBITS, C::GS, C::N, C::K, C::MT, C::WK, C::WN, C::U, C::STEPS, C::VB);
@@ -516,7 +614,7 @@ int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const v
     if (m <= 0) return 0;
     dim3 grid(C::GRID_X, (m + C::MT - 1) / C::MT);
     hipLaunchKernelGGL(gemv_kernel<C>, grid, dim3(C::THREADS), 0, stream, (const uint16_t*)A, (const uint8_t*)W,
-                       (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m);
+                       (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m, norm);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
         fprintf(stderr, "qfactory gemv: launch failed: %s\n", hipGetErrorString(err));

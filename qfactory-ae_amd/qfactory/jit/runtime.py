@@ -66,6 +66,11 @@ class Runtime:
         if self._launch_m is not None:
             self._launch_m.restype = None
             self._launch_m.argtypes = [ctypes.c_int] + sig + [rc_type]
+        self._launch_norm = getattr(self.lib, "launch_norm", None)      # objects with the residual-add + RMSNorm prologue
+        if self._launch_norm is not None:
+            self._launch_norm.restype = None
+            ptr = ctypes.c_void_p
+            self._launch_norm.argtypes = [ctypes.c_int, ptr, ptr, ptr, ptr, ctypes.c_float, ptr, ptr, ptr, ptr, ptr, rc_type]
         describe = getattr(self.lib, "qf_describe", None)
         if describe is not None:
             describe.restype = ctypes.c_char_p

@@ -78,16 +78,21 @@ class GPTQLinear(torch.nn.Module):
             self._launchers.clear()     # bound launchers hold the addresses of the tensors they were made for
         super().__setattr__(name, value)
 
-    def _compile(self, m, compile_flags, dtype=torch.float16, epilogue="none"):
+    def _compile(self, m, compile_flags, dtype=torch.float16, epilogue="none", prologue="none"):
         matmul = QMatmul(m, self.out_features, self.in_features, self.n_bits, self.z is None,
-                         dtype, torch.int8, self.group_size, base_impl=self.base_impl, output_epilogue=epilogue)
+                         dtype, torch.int8, self.group_size, base_impl=self.base_impl, output_epilogue=epilogue,
+                         input_prologue=prologue)
         func = matmul.compile_profile(**compile_flags)
         # One launch now: the first call of a specialisation loads its code object and may raise its
         # LDS limit (hipFuncSetAttribute), neither of which should happen inside a HIP-graph capture.
         if self.w.is_cuda:
             x = torch.zeros(m, self.in_features, dtype=dtype, device=self.w.device)
             out = torch.empty(m, self.out_features // (2 if epilogue == "silu_mul" else 1), dtype=dtype, device=self.w.device)
-            rc = func(x, self.w, out, self.s, self.z) if self.z is not None else func(x, self.w, out, self.s)
+            if prologue == "add_rmsnorm":
+                rc = func(x, None, torch.ones(self.in_features, dtype=dtype, device=self.w.device), None, 1e-6,
+                          self.w, out, self.s, self.z)
+            else:
+                rc = func(x, self.w, out, self.s, self.z) if self.z is not None else func(x, self.w, out, self.s)
             if rc != 0:
                 raise RuntimeError(f"quantized linear launch failed with return code {rc}")
         return func
@@ -143,6 +148,47 @@ class GPTQLinear(torch.nn.Module):
         if regime != "gemv":
             return False
         return tiling.gemv_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)["U"] % 2 == 0
+
+    def fuses_add_rmsnorm(self, m, dtype=torch.float16, silu_mul=False):
+        """Does ``forward_add_rmsnorm`` on ``m`` rows run as one launch?  Where the dot2 GEMV kernel serves (fp16)."""
+        if dtype != torch.float16 or (silu_mul and not self.fuses_silu_mul(m, dtype)):
+            return False
+        return tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features) == "gemv"
+
+    def forward_add_rmsnorm(self, x: torch.Tensor, delta, gamma: torch.Tensor, eps: float, x_out=None, silu_mul=False):
+        """The step of a decoder layer that ends in this projection: ``h = x + delta`` (fp16 add; ``delta`` may be
+        None), ``a = fp16(fp16(h * rsqrt(mean(h^2) + eps)) * gamma)``, then ``self(a)`` -- or, with ``silu_mul``,
+        ``self.forward_silu_mul(a)``.  ``x_out`` (required with ``delta``; a buffer of its own) receives ``h``, the
+        next residual stream.  One launch where the dot2 GEMV kernel serves (M < 3): every block normalises the row
+        for itself while its first weights are in flight.  Otherwise ``qf_add_rmsnorm`` followed by the projection,
+        which is also what the one launch is checked against: its sum of squares is added in another order, so a
+        normalised element may differ by one fp16 ulp.  Not in the reference, whose end-to-end runs leave residual
+        add and norm to vLLM's ``fused_add_rms_norm``."""
+        from . import native
+        m = x.shape[0]
+        assert delta is None or x_out is not None, "with delta, the sum needs a buffer to go to"
+        if m == 0 or not self.fuses_add_rmsnorm(m, x.dtype, silu_mul):
+            h = x
+            if delta is not None:
+                h = torch.add(x, delta, out=x_out)
+            elif x_out is not None:
+                x_out.copy_(x)
+            a = torch.empty_like(x)
+            if m > 0:
+                native.add_rmsnorm(h, None, gamma, a, eps)
+            return self.forward_silu_mul(a) if silu_mul else self.forward(a)
+        key = (_m_bucket(m), x.dtype, "add_rmsnorm+silu_mul" if silu_mul else "add_rmsnorm")
+        func = self._funcs.get(key)
+        if func is None:
+            func = self._funcs[key] = self._compile(key[0], self.compile_flags, x.dtype,
+                                                    "silu_mul" if silu_mul else "none", "add_rmsnorm")
+        output = torch.empty(m, self.out_features // (2 if silu_mul else 1), dtype=x.dtype, device=x.device)
+        rc = func(x, delta, gamma, x_out, eps, self.w, output, self.s, self.z)
+        if rc != 0:
+            raise RuntimeError(f"quantized linear launch failed with return code {rc}")
+        if delta is None and x_out is not None:
+            x_out.copy_(x)
+        return output
 
     def forward_silu_mul(self, x: torch.Tensor):
         """For a fused gate+up projection (rows 0 .. N/2-1 gate, the rest up): the SwiGLU activation

@@ -67,6 +67,27 @@ def test_jit_object_exports_the_launch_abi(gs, guard):
     assert f"#define {guard}" in src and '#include "qfactory_launch.h"' in src
 
 
+def test_jit_object_with_the_norm_prologue_exports_launch_norm():
+    from qfactory.core.qfunc import QMatmulQFunc
+    from qfactory.core.qtile import AsymQTile, QTile
+    from qfactory.jit import jit
+    assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_NORM") == ["launch_norm"]
+    qfunc = QMatmulQFunc(QTile((1, 512), torch.float16, 16), AsymQTile((64, 512), torch.int8, 4, (1, 128)), "nt")
+    qfunc.input_prologue = "add_rmsnorm"
+    runtime = jit.compile(qfunc)
+    lib = ctypes.CDLL(os.path.join(runtime.path, "kernel.so"))
+    for name in _declared_functions("qfactory_launch.h", "QF_LAUNCH_GROUPED") + ["launch_norm"]:
+        assert hasattr(lib, name), f"{name} missing from {runtime.path}"
+    assert runtime._launch_norm is not None and "prologue=add_rmsnorm" in runtime.description
+    src = open(os.path.join(runtime.path, "kernel.hip")).read()
+    assert "#define QF_LAUNCH_NORM" in src and "#define QF_GEMV_NORM_PROLOGUE 1" in src
+    # the prologue is the dot2 GEMV kernel's: a matrix-core problem refuses it
+    wide = QMatmulQFunc(QTile((64, 512), torch.float16, 16), AsymQTile((64, 512), torch.int8, 4, (1, 128)), "nt")
+    wide.input_prologue = "add_rmsnorm"
+    with pytest.raises(AssertionError):
+        wide.emit()
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from qfactory import native
     monkeypatch.setattr(native, "_lib", None)

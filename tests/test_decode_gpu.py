@@ -172,3 +172,11 @@ def test_decode_step_matches_the_torch_evaluation_of_the_same_model():
     assert torch.equal(got.argmax(-1), want.argmax(-1))
     assert ((got_k.float() - want_k.float()).norm() / want_k.float().norm()).item() <= 3e-3
     assert ((got_v.float() - want_v.float()).norm() / want_v.float().norm()).item() <= 3e-3
+    # two rows: the residual adds and norms ran inside the qkv and gate+up projections (five launches per layer);
+    # as launches of their own (eight per layer) the step gives the same tokens and logits to the same bar
+    keys = [k for layer in model.layers for name in ("qkv", "gate_up") for k in layer[name]._funcs]
+    assert (2, torch.float16, "add_rmsnorm") in keys and (2, torch.float16, "add_rmsnorm+silu_mul") in keys
+    model.fuse_norm = False
+    apart, apart_k, _ = run(model.decode_step)
+    assert ((apart - got).norm() / got.norm()).item() <= 1e-3 and torch.equal(apart.argmax(-1), got.argmax(-1))
+    assert ((apart_k.float() - got_k.float()).norm() / got_k.float().norm()).item() <= 1e-3
