@@ -22,6 +22,7 @@ from itertools import chain
 
 import torch
 
+from . import tiling
 from .qtile import QTile, SymQTile, AsymQTile
 from .qfunc import QMatmulQFunc, MatmulQFunc, apply_config
 from ..convert import weight_row_bytes, zero_row_bytes
@@ -132,6 +133,15 @@ class QMatmul:
             "nt", self.base_impl)]
         self.qfuncs[0].output_epilogue = self.output_epilogue
         self.qfuncs[0].input_prologue = self.input_prologue
+        q = self.qfuncs[0]
+        if self.input_prologue != "none" and q.regime == "gemv" and tiling.gemv_chunks_per_lane(self.k, self.nbits, q.tiling_configs) == 1:
+            # every block normalises the row before its first dot product (loads from L2, a sum across the team, a
+            # barrier): four stages per block spread that over four times the rows.  Measured at M = 1, cold
+            # weights, against qf_add_rmsnorm + the plain kernel: 12288 x 4096 8.6 -> 7.4 us (one team per block),
+            # 22016 x 4096 with the SwiGLU epilogue 11.9 -> 11.0 (two teams); with the plain kernel's one-stage
+            # tiling the fused form is slower than the two launches (9.6 and 16.5 us)
+            q.tiling_configs = tiling.gemv_tiling(self.m, self.n, self.k, self.nbits, self.group_size, u=4, steps=4,
+                                                  wn=2 if self.n >= 16384 else 1)
 
     def get_dummy_inputs(self):
         require_gpu()
