@@ -224,6 +224,13 @@ class QMatmulQFunc(QFunc):
             # registers to spare: the one-instruction mask-and-merge decode pays there (2 - 7 %
             # measured); it does not in the 4-bit GEMV kernel, where it costs a resident wave
             defines.setdefault("QF_FUSED_AND_OR", 1)
+        if self.regime == "gemv" and p["NBITS"] in (2, 3) and t["VB"] == 8 and t["MT"] == 1 \
+                and self.decode_strategy == "deferred" and not self.smem_quant \
+                and tiling.gemv_chunks_per_lane(p["K"], p["NBITS"], t) == 1:
+            # 32 fields per lane and row: the compiler-scheduled one-instruction decode and one scale / zero-point
+            # load per lane and stage, as for 4 bits below (part of the 8-byte tiling's measured gain)
+            defines.setdefault("QF_FUSED_AND_OR", 2)
+            defines.setdefault("QF_GEMV_QUANT_DEDUP", 1)
         if self.regime == "gemv" and p["NBITS"] == 2:
             # sixteen fields per word make the 2-bit GEMV decode-bound: measured 7.6 -> 6.9 us at 8192 x 8192
             defines.setdefault("QF_FUSED_AND_OR", 1)

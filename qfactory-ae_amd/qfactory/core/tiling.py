@@ -66,11 +66,23 @@ def elements_per_chunk(nbits, vb):
     return vb * 8 // plane_bits(nbits)
 
 
-def gemv_vec_bytes(K, nbits, group_size):
+def gemv_vec_bytes(K, nbits, group_size, mt=None, N=None):
     """Widest per-lane load (16/8/4 bytes of the main plane) that divides a packed row and stays
-    inside one group; 3-bit rows need at least 8 (one whole word of the 1-bit plane per chunk)."""
+    inside one group; 3-bit rows need at least 8 (one whole word of the 1-bit plane per chunk).
+    One activation row against a 2-bit main plane (2- and 3-bit weights, ``mt == 1``): 8 bytes -- 32 fields --
+    per lane where the row then still fits one pass of eight waves.  Sixteen bytes are 64 fields and 32 activation
+    registers per lane and half as many waves; measured at M = 1, cold weights, sixteen against eight bytes:
+    2 bits 3.80 -> 3.02 us on 4096 x 4096, 8.86 -> 7.05 on 22016 x 4096, 6.10 -> 5.63 on 8192 x 8192, 29.6 -> 28.2 on
+    57344 x 8192; 3 bits 4.93 -> 3.64, 12.9 -> 10.9, 8.55 -> 8.17, but 43.5 -> 48.4 on 57344 x 8192 (its 1-bit plane
+    then comes in 4-byte loads), so 3-bit launches of many rounds of waves keep sixteen."""
     row_bytes = K * plane_bits(nbits) // 8
-    for vb in ((16, 8) if nbits == 3 else (16, 8, 4)):
+    widths = (16, 8) if nbits == 3 else (16, 8, 4)
+    waves8 = -(-(K // elements_per_chunk(nbits, 8)) // 64)
+    if mt == 1 and plane_bits(nbits) == 2 and waves8 <= 8:
+        many_rounds = N is not None and (N * waves8) // 4 > 2 * 8 * 4 * NUM_CUS
+        if not (nbits == 3 and many_rounds):
+            widths = (8, 16) if nbits == 3 else (8, 16, 4)
+    for vb in widths:
         epc = elements_per_chunk(nbits, vb)
         if row_bytes % vb:
             continue
@@ -110,11 +122,11 @@ def gemv_wave_split(K, nbits, vb, mt, max_waves=8, a_reg_budget=128):
 
 def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None, mt=None):
     """Default GEMV tiling; keyword arguments pin individual parameters."""
-    vb = gemv_vec_bytes(K, nbits, group_size)
     if mt is None:
         mt = min(_pow2_floor(max(M, 1)), GEMV_MAX_M)
         if mt < M <= GEMV_MAX_M:
             mt *= 2                                   # 3 -> 4: one pass, one predicated row
+    vb = gemv_vec_bytes(K, nbits, group_size, mt, N)
     if wk is None:
         wk, it = gemv_wave_split(K, nbits, vb, mt)[0]
     else:
@@ -130,6 +142,8 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
     big = it >= 2 or (N * wk) // 4 > 2 * 8 * 4 * NUM_CUS
     if u is None:
         in_flight = 8 if (big or nbits <= 3) else 4
+        if nbits == 3 and vb == 8 and mt == 1:
+            in_flight = 4                             # two planes per row: four rows are eight loads (8192 x 8192: 7.94 us against 8.36)
         if nbits == 4 and it == 1 and wk == 4 and mt == 1:
             # K = 8192 at 4 bits (four waves per row): eight rows per stage with one scale / zero-point load per lane
             # and stage measured 8.26 us on 8192 x 8192 against 8.85 for four (cold weights)
