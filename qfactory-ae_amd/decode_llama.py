@@ -13,8 +13,8 @@ RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plai
 replaces its norm and SiLU steps by single launches.  A decode
 step runs the steps between the linears as one HIP launch each (residual add + RMSNorm, RoPE + cache
 append + attention of the new position, SiLU * up: libqfactory_hip.so) -- eight launches per layer
-instead of about fifty -- and, for one or two sequences, five: the dot2 GEMV kernel then runs the residual add and
-RMSNorm in front of its dot products and SiLU * up behind them; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
+instead of about fifty -- and, up to 32 sequences, five: the kernels for few rows run the residual add and
+RMSNorm in front of their dot products and SiLU * up behind them; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
 Prints one JSON line per batch size: tokens/s over the decode phase, prefill time, and the share of
@@ -96,7 +96,6 @@ class QuantLlama:
         # buffers of the fused decode step (one new position per sequence)
         f16 = dict(dtype=torch.float16, device="cuda")
         self._hdn, self._att = (torch.empty(batch, h, **f16) for _ in range(2))
-        self._res = [torch.empty(batch, h, **f16) for _ in range(2)]      # the residual stream alternates between the two
 
     def _norm(self, x, w):
         xf = x.float()
@@ -170,24 +169,19 @@ class QuantLlama:
         x = self.embed[tok[:, 0]]                                # (B, h): the residual stream, updated in place
         delta = None
         first = self.layers[0]
-        if (self.fuse_norm and self.linear is self._own_linear and first["qkv"].fuses_add_rmsnorm(x.shape[0])
-                and first["gate_up"].fuses_add_rmsnorm(x.shape[0], silu_mul=True)):
-            # five launches per layer: the two residual adds and norms run inside the projections behind them, each
-            # writing the new residual stream to the buffer the old one is not in
-            turn = 0
+        rows = x.shape[0]
+        if (self.fuse_norm and self.linear is self._own_linear and first["qkv"].fuses_add_rmsnorm(rows)
+                and first["gate_up"].fuses_add_rmsnorm(rows, silu_mul=True) and first["o"].fuses_accumulate(rows)
+                and first["down"].fuses_accumulate(rows)):
+            # five launches per layer: the o and down projections add their result to the residual stream themselves,
+            # and the qkv and gate+up projections normalise it in front of their dot products
             for li, layer in enumerate(self.layers):
-                if delta is None:
-                    qkv = layer["qkv"].forward_add_rmsnorm(x, None, layer["norm1"], shape.eps)
-                else:
-                    qkv = layer["qkv"].forward_add_rmsnorm(x, delta, layer["norm1"], shape.eps, x_out=self._res[turn])
-                    x, turn = self._res[turn], turn ^ 1
+                qkv = layer["qkv"].forward_add_rmsnorm(x, None, layer["norm1"], shape.eps)
                 native.rope_decode_attention(qkv, pos, self.cos, self.sin, self.k_cache[li], self.v_cache[li], self._att)
-                delta = layer["o"](self._att)
-                act = layer["gate_up"].forward_add_rmsnorm(x, delta, layer["norm2"], shape.eps, x_out=self._res[turn],
-                                                           silu_mul=True)
-                x, turn = self._res[turn], turn ^ 1
-                delta = layer["down"](act)
-            native.add_rmsnorm(x, delta, self.final_norm, self._hdn, shape.eps)
+                layer["o"].forward_accumulate(self._att, x)
+                act = layer["gate_up"].forward_add_rmsnorm(x, None, layer["norm2"], shape.eps, silu_mul=True)
+                layer["down"].forward_accumulate(act, x)
+            native.add_rmsnorm(x, None, self.final_norm, self._hdn, shape.eps)
             return self._hdn @ self.lm_head.T
         for li, layer in enumerate(self.layers):
             native.add_rmsnorm(x, delta, layer["norm1"], self._hdn, shape.eps)

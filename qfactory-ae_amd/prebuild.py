@@ -224,7 +224,32 @@ def norm_prologue_cases():
         cases.append(dict(c, prologue="add_rmsnorm"))
     for c in (_case(1, 100, 1024), _case(2, 154, 512, 3, 64), _case(1, 260, 2048, 8, 128), _case(2, 96, 2816, 2, 128, True)):
         cases.append(dict(c, prologue="add_rmsnorm", epilogue="silu_mul"))
+    # the A-stationary kernel (3 .. 32 rows): the decode loop's at batch 16, the tiny model's, ragged M and N, every
+    # bit width, a last wave that owns fewer chunks, two 16-row activation tiles
+    cases += [dict(_case(16, 12288, 4096), prologue="add_rmsnorm"),
+              dict(_case(16, 22016, 4096), prologue="add_rmsnorm", epilogue="silu_mul"),
+              dict(_case(16, 768, 256, 4, 64), prologue="add_rmsnorm"),
+              dict(_case(16, 1024, 256, 4, 64), prologue="add_rmsnorm", epilogue="silu_mul")]
+    for c in (_case(5, 96, 1024, 4, 128), _case(12, 100, 2048, 3, 64), _case(16, 48, 8192, 3, 256, True),
+              _case(7, 1000, 2048, 8, 128), _case(16, 100, 4096, 2, 128), _case(16, 272, 4864, 3, 128),
+              _case(32, 40, 1024, 3, 128), _case(20, 130, 4096, 4, 128)):
+        cases.append(dict(c, prologue="add_rmsnorm"))
+    for c in (_case(5, 96, 1024, 4, 128), _case(12, 4128, 2048, 3, 64), _case(32, 160, 4096, 2, 128, True)):
+        cases.append(dict(c, prologue="add_rmsnorm", epilogue="silu_mul"))
     return cases
+
+
+def accumulate_cases():
+    """Projections that add their result to the output (GPTQLinear.forward_accumulate, up to 32 rows): the decode
+    loop's o and down at batch 1 / 2 / 16, the tiny test model's, and the shapes of tests/test_norm_prologue_gpu.py
+    (dot2 GEMV with one wave per team -- stored from the lane -- and several; A-stationary and streaming kernels;
+    every bit width; ragged M and N)."""
+    cases = [_case(M, N, K) for N, K in ((4096, 4096), (4096, 11008)) for M in (1, 2, 16)]
+    cases += [_case(M, N, K, 4, 64) for N, K in ((256, 256), (256, 512)) for M in (2, 16)]
+    cases += [_case(1, 100, 256), _case(2, 77, 1024, 3, 128, True), _case(1, 130, 2048, 8, 128, True), _case(1, 48, 4096, 2, 128),
+              _case(5, 96, 1024), _case(12, 100, 2048, 3, 64), _case(32, 40, 1024, 8, 128),
+              _case(5, 100, 11008), _case(16, 64, 14336, 2, 512, True), _case(9, 64, 8192, 8, 128)]
+    return [dict(c, epilogue="accumulate") for c in cases]
 
 
 def search_cases():
@@ -252,7 +277,7 @@ def drain_cases(base=None):
 def all_cases(with_drain=True):
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases()):
+              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases() + accumulate_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
@@ -291,7 +316,7 @@ def qfuncs_of(case):
         qfuncs += eager
     if case.get("drain"):
         qfuncs += [q.clone(defines={"QF_GEMM_FULL_DRAIN": 1}) for q in list(qfuncs) if q.regime == "gemm"]
-    if case.get("epilogue") == "silu_mul" or case.get("prologue"):
+    if case.get("epilogue") or case.get("prologue"):
         op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
                      torch.float16, torch.int8, case["GS"], output_epilogue=case.get("epilogue", "none"),
                      input_prologue=case.get("prologue", "none"))

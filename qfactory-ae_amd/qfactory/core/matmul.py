@@ -100,7 +100,9 @@ class QMatmul:
         # "silu_mul" (beyond the reference): the weight is a fused gate+up projection and the closure's output is
         # the (M, N/2) SwiGLU activation fp16(silu(gate)) * up; M <= 32 only (dot2 GEMV and A-stationary kernels), fp16 only
         self.output_epilogue = output_epilogue
-        assert output_epilogue in ("none", "silu_mul")
+        # "accumulate" (beyond the reference): the closure adds the projection to what ``output`` holds,
+        # output = fp16(output + fp16(projection)); M <= 32 (dot2 GEMV, A-stationary and streaming kernels), fp16 only
+        assert output_epilogue in ("none", "silu_mul", "accumulate")
         self.nbits, self.sym = nbits, sym
         self.dtype_a, self.dtype_b = dtype_a, dtype_b
         self.group_size = k if group_size == -1 else group_size

@@ -120,7 +120,9 @@ class QMatmulQFunc(QFunc):
         #                                         measured slower at M = 1 (a barrier in a one-shot block), 3 % faster at M = 2
         self.base_impl = base_impl
         # "silu_mul": the weight is a fused gate+up projection and the kernel writes the (M, N/2) SwiGLU activation
-        # fp16(silu(gate)) * up instead of the (M, N) projection (the kernels for M <= 32; not in the reference)
+        # fp16(silu(gate)) * up instead of the (M, N) projection (the kernels for M <= 32; not in the reference).
+        # "accumulate": the kernel adds its projection to what the output holds, out = fp16(out + fp16(projection))
+        # (the kernels for M <= 32, fp16; a projection that writes into the residual stream; not in the reference)
         self.output_epilogue = "none"
         # "add_rmsnorm": the kernel makes its activations itself -- residual add and RMSNorm of a decoder layer run in
         # front of the dot products -- and the object exports launch_norm (dot2 GEMV kernel, fp16; not in the reference)
@@ -247,14 +249,18 @@ class QMatmulQFunc(QFunc):
             defines["QF_OUT_BF16"] = 1
             if self.converts_activations:
                 defines["QF_IN_BF16"] = 1
-        if self.output_epilogue != "none":
+        if self.output_epilogue == "accumulate":
+            assert self.regime in ("gemv", "mgemv", "skinny") and self.act_dtype == torch.float16, \
+                "only the kernels for up to 32 rows, on fp16, add their result to the output"
+            defines["QF_OUT_ACCUMULATE"] = 1
+        elif self.output_epilogue != "none":
             assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
                 "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, write silu(gate) * up"
             defines["QF_GEMV_GATE_UP_SILU" if self.regime == "gemv" else "QF_MGEMV_GATE_UP_SILU"] = 1
         if self.input_prologue != "none":
-            assert self.input_prologue == "add_rmsnorm" and self.regime == "gemv" and self.act_dtype == torch.float16, \
-                "only the dot2 GEMV kernel, on fp16, runs the residual add and RMSNorm in front of its dot products"
-            defines["QF_GEMV_NORM_PROLOGUE"] = 1
+            assert self.input_prologue == "add_rmsnorm" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
+                "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, run the residual add and RMSNorm themselves"
+            defines["QF_GEMV_NORM_PROLOGUE" if self.regime == "gemv" else "QF_MGEMV_NORM_PROLOGUE"] = 1
         if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none":
             defines["QF_GEMV_SMEM_QUANT"] = 1
         for name, value in sorted(defines.items()):
@@ -295,14 +301,14 @@ class QMatmulQFunc(QFunc):
             code += ('extern "C" void launch_norm (\n\tint m,\n\tvoid* _activation,\n\tvoid* _delta,\n\tvoid* _gamma,\n'
                      '\tvoid* _x_out,\n\tfloat eps,\n\tvoid* _weight,\n\tvoid* _output,\n\tvoid* _scale,\n\tvoid* _zero,\n'
                      '\tvoid* _stream,\n\tint& __return_code\n) {\n'
-                     '\tqf::GemvNormArgs norm;\n\tnorm.delta = (const uint16_t*)_delta;\n\tnorm.gamma = (const uint16_t*)_gamma;\n'
+                     '\tqf::NormArgs norm;\n\tnorm.delta = (const uint16_t*)_delta;\n\tnorm.gamma = (const uint16_t*)_gamma;\n'
                      '\tnorm.x_out = (uint16_t*)_x_out;\n\tnorm.eps = eps;\n'
                      f'\t__return_code = _gamma == nullptr ? 1 : {call}({args}, m, (hipStream_t)_stream, norm);\n}}\n\n')
         desc = (f"regime={self.regime} M={p['M']} N={p['N']} K={p['K']} NBITS={p['NBITS']} GS={p['GS']} "
                 f"SYM={int(p['SYM'])} decode={self.decode_strategy} nt_b={int(not self.l2cache_b)} "
                 + ("act=bf16 " if self.act_dtype == torch.bfloat16 else "")
                 + ("prologue=add_rmsnorm " if self.input_prologue == "add_rmsnorm" else "")
-                + ("epilogue=silu_mul " if self.output_epilogue == "silu_mul" else "")
+                + (f"epilogue={self.output_epilogue} " if self.output_epilogue != "none" else "")
                 + ("smem_quant=1 " if self.smem_quant and self.regime == "gemv" and self.output_epilogue == "none" else "")
                 + " ".join(f"{k}={v}" for k, v in sorted(t.items()))
                 # the header knobs that change the generated code and are not named above

@@ -90,6 +90,23 @@ __device__ __forceinline__ uint16_t f32_to_out_bits(float f) {
 #endif
 }
 
+// 1: the kernel adds its result to what the output already holds -- out = fp16(out + fp16(result)), the two roundings
+// of a projection followed by a residual add -- instead of overwriting it: the o and down projections of a decoder
+// layer writing straight into the residual stream.  Every element is still touched by exactly one lane (read, then
+// written).  fp16 only; the kernels for up to 32 rows.  Not in the reference.
+#ifndef QF_OUT_ACCUMULATE
+#define QF_OUT_ACCUMULATE 0
+#endif
+__device__ __forceinline__ void store_out(uint16_t* p, float f) {
+#if QF_OUT_ACCUMULATE
+    const _Float16 add = (_Float16)f;
+    const _Float16 old = __builtin_bit_cast(_Float16, *p);
+    *p = __builtin_bit_cast(uint16_t, (_Float16)(old + add));
+#else
+    *p = f32_to_out_bits(f);
+#endif
+}
+
 // SwiGLU on two fp32 sums of a fused gate+up projection: both are rounded to fp16 as the projection's output
 // would be, then fp16(silu(gate)) * up with silu(x) = x * rcp(1 + exp2(-x * log2(e))) on the hardware's exp2 and
 // reciprocal -- the expression of qf_silu_mul in libqfactory_hip.so, so that a kernel's fused epilogue and the
@@ -243,6 +260,15 @@ template <> struct Decode<8> {
         x[0] = __builtin_amdgcn_perm(0x64646464u, w, 0x04010400u);
         x[1] = __builtin_amdgcn_perm(0x64646464u, w, 0x04030402u);
     }
+};
+
+// Operands of the residual-add + RMSNorm prologue of the kernels for few rows (ignored by kernels compiled
+// without it):  h = fp16(x + delta),  a = fp16(fp16(h * rsqrt(mean(h^2) + eps)) * gamma).
+struct NormArgs {
+    const uint16_t* delta = nullptr;   // (M, K) fp16 added to the activation rows first, or null
+    const uint16_t* gamma = nullptr;   // (K) fp16 RMSNorm weight
+    uint16_t* x_out = nullptr;         // (M, K) fp16: receives x + delta, or null
+    float eps = 0.0f;
 };
 
 // ---- wave64 lane exchange: value held by lane (l ^ D) ----

@@ -132,18 +132,10 @@ struct GemvCfg {
 #define QF_GEMV_OCCUPANCY
 #endif
 
-// Operands of the norm prologue (ignored by kernels compiled without it).
-struct GemvNormArgs {
-    const uint16_t* delta = nullptr;   // (M, K) fp16 added to the activation rows first, or null
-    const uint16_t* gamma = nullptr;   // (K) fp16 RMSNorm weight
-    uint16_t* x_out = nullptr;         // (M, K) fp16: receives x + delta, or null
-    float eps = 0.0f;
-};
-
 template <class C>
 __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
     const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
-    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total, GemvNormArgs norm) {
+    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total, NormArgs norm) {
     using D = Decode<C::NBITS>;
     constexpr int NW = C::NW, EPC = C::EPC, NCH = C::NCH, T = C::T, IT = C::IT;
     constexpr int MT = C::MT, U = C::U, STEPS = C::STEPS, V = C::V, WK = C::WK;
@@ -524,7 +516,7 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
                 const int u = v / MT, m = v % MT;
                 const int row = row_base + step * U + u;
                 if (row < C::N && m0 + m < m_total)
-                    Cout[(size_t)(m0 + m) * C::N + row] = f32_to_out_bits(part[0]);
+                    store_out(Cout + (size_t)(m0 + m) * C::N + row, part[0]);
             } else {
                 red[team][wk][step * V + v] = part[0];
             }
@@ -577,14 +569,14 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         const int step = j / V, v = j % V;
         const int u = v / MT, m = v % MT;
         const int row = row_base + step * U + u;
-        if (row < C::N && m0 + m < m_total) Cout[(size_t)(m0 + m) * C::N + row] = f32_to_out_bits(total);
+        if (row < C::N && m0 + m < m_total) store_out(Cout + (size_t)(m0 + m) * C::N + row, total);
     }
 }
 
 // Host launcher: static validity checks (return 1 and say why on stderr), then the launch.
 template <class C>
 int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m,
-                hipStream_t stream, GemvNormArgs norm = GemvNormArgs{}) {
+                hipStream_t stream, NormArgs norm = NormArgs{}) {
     const char* why = nullptr;
     if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8";
     else if (C::VB != 4 && C::VB != 8 && C::VB != 16) why = "VB must be 4, 8 or 16";
@@ -603,6 +595,7 @@ int gemv_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (QF_GEMV_SMEM_QUANT && C::QPARAM && (size_t)C::RPB * C::G * 2 + (size_t)C::RPB * C::ZRB + sizeof(float) * C::WN * C::WK * C::STEPS * C::V > 64 * 1024) why = "scales through LDS exceed LDS";
     else if (C::WN * C::WK * C::STEPS * C::V * 4 > 64 * 1024) why = "reduction scratch exceeds LDS";
     else if (QF_GEMV_NORM_PROLOGUE && (QF_IN_BF16 || QF_OUT_BF16)) why = "the norm prologue is fp16 only";
+    else if (QF_OUT_ACCUMULATE && (QF_OUT_BF16 || QF_GEMV_GATE_UP_SILU)) why = "adding to the output is fp16 only and not combined with the SwiGLU epilogue";
     else if (QF_GEMV_NORM_PROLOGUE && norm.gamma == nullptr) why = "an object with the norm prologue is called through launch_norm (RMSNorm weight missing)";
     else if (!QF_GEMV_NORM_PROLOGUE && norm.gamma != nullptr) why = "this object was compiled without the norm prologue";
     else if (QF_GEMV_NORM_PROLOGUE && (norm.x_out == A || (norm.x_out != nullptr && norm.x_out == norm.delta))) why = "x_out must be a buffer of its own: other blocks still read x and delta";

@@ -37,6 +37,15 @@
 #define QF_MGEMV_GATE_UP_SILU 0
 #endif
 
+// 1: the activations are made, not read: residual add and RMSNorm of the decoder layer run while a block brings
+// its activation slices into registers (the roundings of qf_add_rmsnorm in libqfactory_hip.so, which this replaces
+// up to 32 rows; same contract as QF_GEMV_NORM_PROLOGUE in qf_gemv.hip.h).  A wave adds the squares of its own K-slice
+// per row, the WK waves meet once through LDS; the persistent block does this once for all the tiles it sweeps.
+// Block (0, y) also writes x + delta to x_out.  fp16 only.  Not in the reference.
+#ifndef QF_MGEMV_NORM_PROLOGUE
+#define QF_MGEMV_NORM_PROLOGUE 0
+#endif
+
 // Timing experiments (results are wrong when non-zero): bit 0 skips the activation loads, bit 1 the
 // dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores, bit 3 the weight loads.
 #ifndef QF_MGEMV_EXPERIMENT
@@ -119,8 +128,9 @@ struct MGemvCfg {
 template <class C>
 __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
-    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total) {
+    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total, NormArgs norm) {
     constexpr int MT16 = C::MT16, WK = C::WK, CH = C::CH, SLOTS = C::SLOTS, PF = C::PF, SB = C::SB;
+    constexpr bool NORM = QF_MGEMV_NORM_PROLOGUE != 0;
     constexpr int EPL = C::EPL, KSTEPS = C::KSTEPS, CHUNK = C::CHUNK;
     constexpr int P8 = 8 / C::ZFB;                      // zero-point fields per byte
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
@@ -226,6 +236,89 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     if (QF_MGEMV_EXPERIMENT & 1) raw[mt][c][i] = u32x4{(uint32_t)lane, 1u, 2u, 3u};
                     else raw[mt][c][i] = *reinterpret_cast<const u32x4*>(ap);
                 }
+        if constexpr (NORM) {
+            static_assert(!QF_IN_BF16, "the norm prologue is fp16 only");
+            // raw[][][] holds the wave's slices of x in load order: lane -> (row i*RPIA + lane/LPRA, 8 elements at
+            // (lane%LPRA)*8 of chunk c).  Add delta, keep the sum for x_out, add up the squares per row, normalise.
+            u32x4 gam[CH];
+#pragma unroll
+            for (int c = 0; c < CH; c++)
+                gam[c] = *reinterpret_cast<const u32x4*>(norm.gamma + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8);
+            float ss[MT16][LPC];
+            float* nrm = reinterpret_cast<float*>(smem);             // [WK][BM]: before the partial tiles need the space
+            const bool writer = norm.x_out != nullptr && blockIdx.x == 0;
+#pragma unroll
+            for (int mt = 0; mt < MT16; mt++)
+#pragma unroll
+                for (int i = 0; i < LPC; i++) {
+                    const int row = i * RPIA + lane / LPRA;
+                    const int m = m0 + 16 * mt + row;
+                    float acc2 = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < CH; c++) {
+                        const bool own = (lo + c >= own_from) && (lo + c < own_from + CH);
+                        const size_t eoff = (size_t)min(m, m_total - 1) * C::K + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8;
+                        u32x4 v = raw[mt][c][i];
+                        if (norm.delta != nullptr) {
+                            const u32x4 d = *reinterpret_cast<const u32x4*>(norm.delta + eoff);
+                            v.x = __builtin_bit_cast(uint32_t, as_f16x2(v.x) + as_f16x2(d.x));
+                            v.y = __builtin_bit_cast(uint32_t, as_f16x2(v.y) + as_f16x2(d.y));
+                            v.z = __builtin_bit_cast(uint32_t, as_f16x2(v.z) + as_f16x2(d.z));
+                            v.w = __builtin_bit_cast(uint32_t, as_f16x2(v.w) + as_f16x2(d.w));
+                        }
+                        const bool live = own && m < m_total;
+                        if (writer && live) *reinterpret_cast<u32x4*>(norm.x_out + eoff) = v;
+                        if (!live) v = u32x4{0, 0, 0, 0};
+                        raw[mt][c][i] = v;
+                        acc2 = __builtin_amdgcn_fdot2(as_f16x2(v.x), as_f16x2(v.x), acc2, false);
+                        acc2 = __builtin_amdgcn_fdot2(as_f16x2(v.y), as_f16x2(v.y), acc2, false);
+                        acc2 = __builtin_amdgcn_fdot2(as_f16x2(v.z), as_f16x2(v.z), acc2, false);
+                        acc2 = __builtin_amdgcn_fdot2(as_f16x2(v.w), as_f16x2(v.w), acc2, false);
+                    }
+                    // the LPRA lanes of a row sit side by side
+                    if constexpr (LPRA > 1) acc2 += lane_xor<1>(acc2);
+                    if constexpr (LPRA > 2) acc2 += lane_xor<2>(acc2);
+                    if constexpr (LPRA > 4) acc2 += lane_xor<4>(acc2);
+                    if constexpr (LPRA > 8) acc2 += lane_xor<8>(acc2);
+                    if constexpr (LPRA > 16) acc2 += lane_xor<16>(acc2);
+                    if constexpr (LPRA > 32) acc2 += lane_xor<32>(acc2);
+                    ss[mt][i] = acc2;
+                    if (lane % LPRA == 0) nrm[wk * C::BM + 16 * mt + row] = acc2;
+                }
+            __syncthreads();
+#pragma unroll
+            for (int mt = 0; mt < MT16; mt++)
+#pragma unroll
+                for (int i = 0; i < LPC; i++) {
+                    const int row = i * RPIA + lane / LPRA;
+                    float total = 0.0f;
+#pragma unroll
+                    for (int w2 = 0; w2 < WK; w2++) total += nrm[w2 * C::BM + 16 * mt + row];
+                    ss[mt][i] = rsqrtf(total / (float)C::K + norm.eps);
+                }
+            __syncthreads();                                         // the sums are read: the space may be written again
+#pragma unroll
+            for (int mt = 0; mt < MT16; mt++)
+#pragma unroll
+                for (int c = 0; c < CH; c++)
+#pragma unroll
+                    for (int i = 0; i < LPC; i++) {
+                        const float rn = ss[mt][i];
+                        auto scale2 = [&](uint32_t hw, uint32_t gw) {
+                            const f16x2 h = as_f16x2(hw);
+                            f16x2 n;
+                            n.x = (_Float16)((float)h.x * rn);
+                            n.y = (_Float16)((float)h.y * rn);
+                            return __builtin_bit_cast(uint32_t, n * as_f16x2(gw));
+                        };
+                        u32x4 v = raw[mt][c][i];
+                        v.x = scale2(v.x, gam[c].x);
+                        v.y = scale2(v.y, gam[c].y);
+                        v.z = scale2(v.z, gam[c].z);
+                        v.w = scale2(v.w, gam[c].w);
+                        raw[mt][c][i] = v;
+                    }
+        }
 #pragma unroll
         for (int mt = 0; mt < MT16; mt++) {
 #pragma unroll
@@ -422,7 +515,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
             const int m = m0 + 16 * mt + ml;
             const int n = tile * 16 + nl;
-            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_out_bits(total);
+            if (m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, total);
         }
         if (batch + 1 < C::NBATCH) __syncthreads();           // LDS slots are reused by the next batch
     };
@@ -435,7 +528,8 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 }
 
 template <class C>
-int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m, hipStream_t stream) {
+int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m, hipStream_t stream,
+                 NormArgs norm = NormArgs{}) {
     const char* why = nullptr;
     if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8 for this kernel";
     else if (C::K % C::CHUNK != 0) why = "K must be a multiple of 4*128 / (bits of the main plane)";
@@ -452,6 +546,12 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
     else if (C::LDS_BYTES > 160 * 1024) why = "partial tiles exceed the 160 KB of LDS";
     else if (C::SILU && (C::N % 32 != 0 || C::SB % 2 != 0)) why = "gate+up: N/2 must be whole 16-row tiles and a batch whole pairs";
     else if (C::SILU && (QF_IN_BF16 || QF_OUT_BF16)) why = "the SwiGLU epilogue is fp16 only";
+    else if (QF_MGEMV_NORM_PROLOGUE && (QF_IN_BF16 || QF_OUT_BF16)) why = "the norm prologue is fp16 only";
+    else if (QF_OUT_ACCUMULATE && (QF_OUT_BF16 || QF_MGEMV_GATE_UP_SILU)) why = "adding to the output is fp16 only and not combined with the SwiGLU epilogue";
+    else if (QF_MGEMV_NORM_PROLOGUE && norm.gamma == nullptr) why = "an object with the norm prologue is called through launch_norm (RMSNorm weight missing)";
+    else if (!QF_MGEMV_NORM_PROLOGUE && norm.gamma != nullptr) why = "this object was compiled without the norm prologue";
+    else if (QF_MGEMV_NORM_PROLOGUE && (norm.x_out == A || (norm.x_out != nullptr && norm.x_out == norm.delta))) why = "x_out must be a buffer of its own: other blocks still read x and delta";
+    else if (QF_MGEMV_NORM_PROLOGUE && (size_t)C::WK * C::BM * 4 > (size_t)C::WK * C::SB * C::MT16 * 1024) why = "norm sums exceed the reduction space";
     if (why) {
         fprintf(stderr, "qfactory mgemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT16=%d WK=%d CH=%d PB=%d PF=%d)\n",
                 why, C::NBITS, C::GS, C::N, C::K, C::MT16, C::WK, C::CH, C::PB, C::PF);
@@ -470,7 +570,7 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
     }
     dim3 grid(C::GRID_X, (m + C::BM - 1) / C::BM);
     hipLaunchKernelGGL(mgemv_kernel<C>, grid, dim3(C::THREADS), C::LDS_BYTES, stream, (const uint16_t*)A,
-                       (const uint8_t*)W, (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m);
+                       (const uint8_t*)W, (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m, norm);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
         fprintf(stderr, "qfactory mgemv: launch failed: %s\n", hipGetErrorString(err));

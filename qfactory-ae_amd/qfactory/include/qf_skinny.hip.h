@@ -360,7 +360,7 @@ __global__ __launch_bounds__(C::THREADS) void skinny_kernel(
             for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
             const int m = m0 + 16 * mt + ml;
             const int n = tile * 16 + nl;
-            if (m < m_total && n < C::N) Cout[(size_t)m * C::N + n] = f32_to_out_bits(total);
+            if (m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, total);
         }
     };
 
@@ -423,6 +423,7 @@ int skinny_launch(const void* A, const void* W, void* Cout, const void* S, const
     else if (C::D < 1 || C::D > 4) why = "D must be 1 .. 4";
     else if (C::P > 32) why = "unrolled period too long (choose D dividing the steps per wave)";
     else if (C::LDS_BYTES > 160 * 1024) why = "partial tiles exceed the 160 KB of LDS";
+    else if (QF_OUT_ACCUMULATE && QF_OUT_BF16) why = "adding to the output is fp16 only";
     if (why) {
         fprintf(stderr, "qfactory skinny: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT16=%d WK=%d SB=%d D=%d AST=%d PB=%d)\n",
                 why, C::NBITS, C::GS, C::N, C::K, C::MT16, C::WK, C::SB, C::D, (int)C::AST, C::PB);

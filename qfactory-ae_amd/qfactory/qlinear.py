@@ -87,7 +87,7 @@ class GPTQLinear(torch.nn.Module):
         # LDS limit (hipFuncSetAttribute), neither of which should happen inside a HIP-graph capture.
         if self.w.is_cuda:
             x = torch.zeros(m, self.in_features, dtype=dtype, device=self.w.device)
-            out = torch.empty(m, self.out_features // (2 if epilogue == "silu_mul" else 1), dtype=dtype, device=self.w.device)
+            out = torch.zeros(m, self.out_features // (2 if epilogue == "silu_mul" else 1), dtype=dtype, device=self.w.device)
             if prologue == "add_rmsnorm":
                 rc = func(x, None, torch.ones(self.in_features, dtype=dtype, device=self.w.device), None, 1e-6,
                           self.w, out, self.s, self.z)
@@ -149,18 +149,44 @@ class GPTQLinear(torch.nn.Module):
             return False
         return tiling.gemv_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)["U"] % 2 == 0
 
+    def fuses_accumulate(self, m, dtype=torch.float16):
+        """Does ``forward_accumulate`` on ``m`` rows run as one launch?  Up to 32 rows, fp16."""
+        regime = tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features)
+        return dtype == torch.float16 and regime in ("gemv", "mgemv", "skinny")
+
+    def forward_accumulate(self, x: torch.Tensor, out: torch.Tensor):
+        """``out += self(x)`` in place: ``out = fp16(out + fp16(projection))``, the two roundings of the projection
+        followed by a residual add -- the o and down projections of a decoder layer writing into the residual stream.
+        One launch up to 32 rows (the kernel's final sum reads the output element it is about to write); otherwise
+        ``forward`` and an in-place add, which give the same bits.  Not in the reference."""
+        m = x.shape[0]
+        assert out.shape == (m, self.out_features) and out.dtype == x.dtype and out.is_contiguous()
+        if m == 0:
+            return out
+        if not self.fuses_accumulate(m, x.dtype):
+            return out.add_(self.forward(x))
+        key = (_m_bucket(m), x.dtype, "accumulate")
+        func = self._funcs.get(key)
+        if func is None:
+            func = self._funcs[key] = self._compile(key[0], self.compile_flags, x.dtype, "accumulate")
+        rc = func(x, self.w, out, self.s, self.z) if self.z is not None else func(x, self.w, out, self.s)
+        if rc != 0:
+            raise RuntimeError(f"quantized linear launch failed with return code {rc}")
+        return out
+
     def fuses_add_rmsnorm(self, m, dtype=torch.float16, silu_mul=False):
-        """Does ``forward_add_rmsnorm`` on ``m`` rows run as one launch?  Where the dot2 GEMV kernel serves (fp16)."""
+        """Does ``forward_add_rmsnorm`` on ``m`` rows run as one launch?  Where the dot2 GEMV kernel or the A-stationary
+        kernel serves (up to 32 rows, fp16)."""
         if dtype != torch.float16 or (silu_mul and not self.fuses_silu_mul(m, dtype)):
             return False
-        return tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features) == "gemv"
+        return tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features) in ("gemv", "mgemv")
 
     def forward_add_rmsnorm(self, x: torch.Tensor, delta, gamma: torch.Tensor, eps: float, x_out=None, silu_mul=False):
         """The step of a decoder layer that ends in this projection: ``h = x + delta`` (fp16 add; ``delta`` may be
         None), ``a = fp16(fp16(h * rsqrt(mean(h^2) + eps)) * gamma)``, then ``self(a)`` -- or, with ``silu_mul``,
         ``self.forward_silu_mul(a)``.  ``x_out`` (required with ``delta``; a buffer of its own) receives ``h``, the
-        next residual stream.  One launch where the dot2 GEMV kernel serves (M < 3): every block normalises the row
-        for itself while its first weights are in flight.  Otherwise ``qf_add_rmsnorm`` followed by the projection,
+        next residual stream.  One launch where the dot2 GEMV kernel (M < 3) or the A-stationary kernel (up to 32 rows)
+        serves: every block normalises the rows for itself while its first weights are in flight.  Otherwise ``qf_add_rmsnorm`` followed by the projection,
         which is also what the one launch is checked against: its sum of squares is added in another order, so a
         normalised element may differ by one fp16 ulp.  Not in the reference, whose end-to-end runs leave residual
         add and norm to vLLM's ``fused_add_rms_norm``."""

@@ -1,5 +1,5 @@
 """``GPTQLinear.forward_add_rmsnorm``: the residual add and RMSNorm of a decoder layer inside the projection that
-follows them (dot2 GEMV kernel, M < 3; the reference's end-to-end runs leave the step to vLLM's fused_add_rms_norm
+follows them (dot2 GEMV kernel for M < 3, A-stationary kernel up to 32 rows; the reference's end-to-end runs leave the step to vLLM's fused_add_rms_norm
 in front of third_party/vllm-qfactory.patch:205-214).
 
 Checked three ways: the new residual stream equals ``x + delta`` bit for bit; the output is within the acceptance
@@ -56,7 +56,8 @@ def test_projection_with_residual_add_and_rmsnorm_in_front(oracle, case, with_de
     out = layer.forward_add_rmsnorm(x, delta, gamma, EPS, x_out=x_out, silu_mul=silu)
     torch.cuda.synchronize()
     desc = layer._funcs[(_m_bucket(M), torch.float16, "add_rmsnorm+silu_mul" if silu else "add_rmsnorm")].runtime.description
-    assert "prologue=add_rmsnorm" in desc and "regime=gemv" in desc and (("epilogue=silu_mul" in desc) == silu)
+    assert "prologue=add_rmsnorm" in desc and ("regime=gemv" if M < 3 else "regime=mgemv") in desc
+    assert ("epilogue=silu_mul" in desc) == silu
     assert out.shape == (M, N // 2 if silu else N) and out.dtype == torch.float16
     assert torch.equal(x, x_before), "the residual stream it reads must stay as it was"
     h, a = _normalised(x, delta, gamma)
@@ -82,10 +83,36 @@ def test_projection_with_residual_add_and_rmsnorm_in_front(oracle, case, with_de
     assert int(ulp.max()) <= 2 and float((ulp > 0).float().mean()) < 0.02
 
 
+@pytest.mark.parametrize("case", prebuild.accumulate_cases() + [dict(prebuild._case(40, 96, 1024), epilogue="accumulate")], ids=_id)
+def test_projection_added_to_the_output_in_place(case):
+    """``forward_accumulate``: out = fp16(out + fp16(projection)) -- the kernel's own projection (checked against the
+    oracle in tests/test_qlinear_gpu.py) and one fp16 add, so the result equals ``out + layer(x)`` bit for bit."""
+    from qfactory import QLinear
+    from qfactory.qlinear import _m_bucket
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
+    print(f"[case] accumulate {_id(case)}", flush=True)
+    A, weight, scale, zero = make_problem(9 + N + K + M, M, N, K, nbits, GS, sym)
+    layer = QLinear.init(M, K, N, nbits, weight.cuda(), GS, scale.cuda(), None if zero is None else zero.cuda(),
+                         compile_flags=NO_SEARCH)
+    x = A.cuda()
+    before = (torch.randn(M, N, generator=torch.Generator().manual_seed(N)) * 4).to(torch.float16).cuda()
+    out = before.clone()
+    assert layer.forward_accumulate(x, out) is out
+    want = before + layer(x)
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    if layer.fuses_accumulate(M):
+        desc = layer._funcs[(_m_bucket(M), torch.float16, "accumulate")].runtime.description
+        assert "epilogue=accumulate" in desc
+    else:
+        assert M > 32
+    assert layer.forward_accumulate(x[:0], out[:0]).shape == (0, N)
+
+
 def test_rows_the_kernel_does_not_take_go_through_two_launches(oracle):
-    """More rows than the dot2 GEMV kernel serves: ``qf_add_rmsnorm`` and the projection, same contract."""
+    """More rows than the kernels with the prologue serve: ``qf_add_rmsnorm`` and the projection, same contract."""
     from qfactory import QLinear, native
-    M, N, K = 5, 96, 1024
+    M, N, K = 40, 96, 1024
     A, weight, scale, zero = make_problem(11, M, N, K, 4, 128, False)
     layer = QLinear.init(M, K, N, 4, weight.cuda(), 128, scale.cuda(), zero.cuda(), compile_flags=NO_SEARCH)
     x, delta = A.cuda(), (A * 0.5).cuda().flip(0).contiguous()
