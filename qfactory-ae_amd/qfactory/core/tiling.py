@@ -21,6 +21,8 @@ Five kernel families (``regime_for`` picks one):
   ``WK`` wave groups along K, ``PA`` activation tiles in flight.
 * ``mfma``  -- generic fallback, ``qf::MfmaCfg`` (include/qf_mfma.hip.h).
 """
+import json
+import os
 
 NUM_CUS = 256
 GEMV_MAX_M = 4          # largest M served by the dot2 GEMV before the MFMA kernel takes over
@@ -120,15 +122,45 @@ def gemv_wave_split(K, nbits, vb, mt, max_waves=8, a_reg_budget=128):
     return [(wk, it) for _, _, _, wk, it in out]
 
 
+_GEMV_TUNED = None
+
+
+def gemv_tuned(M, N, K, nbits, group_size):
+    """Winner of an on-device sweep over dot2 GEMV tilings for exactly this problem, or None
+    (``gemv_tuned_gfx950.json`` beside this file, keyed like ``$QFACTORY_CONFIG``: "bits-M-N-K-group")."""
+    global _GEMV_TUNED
+    if _GEMV_TUNED is None:
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemv_tuned_gfx950.json")
+        try:
+            with open(path) as f:
+                _GEMV_TUNED = json.load(f)
+        except FileNotFoundError:
+            _GEMV_TUNED = {}
+    entry = _GEMV_TUNED.get(f"{nbits}-{M}-{N}-{K}-{group_size}")
+    return dict(entry) if entry else None
+
+
 def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None, mt=None):
-    """Default GEMV tiling; keyword arguments pin individual parameters."""
+    """Default GEMV tiling: the swept winner where one is stored for the exact problem, else the model below;
+    keyword arguments pin individual parameters (and skip the table)."""
+    if wk is None and u is None and steps is None and wn is None and mt is None:
+        tuned = gemv_tuned(M, N, K, nbits, group_size)
+        if tuned is not None:
+            return tuned
+    return gemv_tiling_model(M, N, K, nbits, group_size, wk, u, steps, wn, mt)
+
+
+def gemv_tiling_model(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None, mt=None):
+    """The analytic default alone."""
     if mt is None:
         mt = min(_pow2_floor(max(M, 1)), GEMV_MAX_M)
         if mt < M <= GEMV_MAX_M:
             mt *= 2                                   # 3 -> 4: one pass, one predicated row
     vb = gemv_vec_bytes(K, nbits, group_size, mt, N)
     if wk is None:
-        wk, it = gemv_wave_split(K, nbits, vb, mt)[0]
+        # one activation row: up to sixteen waves per row when that makes one chunk per lane (8192 x 28672 at 4 bits:
+        # fourteen waves x one chunk 21.8 us against seven x two 24.1, cold weights)
+        wk, it = gemv_wave_split(K, nbits, vb, mt, max_waves=16 if mt == 1 else 8)[0]
     else:
         it = -(-(K // elements_per_chunk(nbits, vb)) // (64 * wk))
     # Loads in flight per lane (rows x chunks per row), measured on MI355X once the kernel's address
@@ -140,6 +172,7 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
     #     (46.6 -> 40.5 us and 37.6 -> 25.5 us);
     #   * 2- and 3-bit rows are short in bytes and heavy in decode work: 8 loads.
     big = it >= 2 or (N * wk) // 4 > 2 * 8 * 4 * NUM_CUS
+    u_free, wn_free, steps_free = u is None, wn is None, steps is None
     if u is None:
         in_flight = 8 if (big or nbits <= 3) else 4
         if nbits == 3 and vb == 8 and mt == 1:
@@ -160,6 +193,14 @@ def gemv_tiling(M, N, K, nbits, group_size, wk=None, u=None, steps=None, wn=None
         # 11.2 -> 10.1 on 8192 x 8192) as long as every CU still gets a block
         if mt >= 2 and it == 1 and N // (wn * u * 4) >= NUM_CUS:
             steps = 4
+    blocks16 = -(-N // 16)
+    whole_rounds = blocks16 <= NUM_CUS or blocks16 % NUM_CUS == 0 or blocks16 >= 4 * NUM_CUS
+    if mt == 1 and it == 1 and wk >= 6 and nbits == 4 and whole_rounds and u_free and wn_free and steps_free:
+        # long rows, one chunk per lane: a team's activations are 22 KB and more, so four stages of four rows per
+        # team and one team per block (cold weights: 4096 x 11008 5.97 us against 6.59 for two teams of one stage,
+        # 3584 x 18944 8.30 against 9.48) -- where sixteen-row blocks fill the CUs evenly (5120 x 13824, 320 blocks:
+        # 10.4 against 8.85 us for one stage)
+        u, wn, steps = 4, 1, 4
     return {"MT": mt, "WK": wk, "WN": wn, "U": u, "STEPS": steps, "VB": vb}
 
 

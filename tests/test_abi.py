@@ -108,7 +108,7 @@ def test_built_distribution_carries_headers_and_native_sources(tmp_path):
     lib = build / "lib" / "qfactory"
     for rel in ("include/qf_gemv.hip.h", "include/qf_gemm.hip.h", "include/qf_common.hip.h", "csrc/qfactory_hip.hip",
                 "csrc/qfactory_decode.hip", "csrc/qf_fastpath.cpp", "abi/qfactory_launch.h", "abi/qfactory_hip.h", "jit/compiler.py", "core/tiling.py",
-                "core/gemm_tuned_gfx950.json", "integrations/vllm_qfactory.py"):
+                "core/gemm_tuned_gfx950.json", "core/gemv_tuned_gfx950.json", "integrations/vllm_qfactory.py"):
         assert (lib / rel).exists(), rel
     probe = ("import qfactory.native as n, qfactory.jit.compiler as c; "
              "print(n.CSRC_DIR); print(n.REPO_INCLUDE); print(c.ABI_INCLUDE_DIR)")

@@ -59,7 +59,8 @@ def test_full_size_decode_step_matches_the_torch_evaluation(llama, batch):
     a, b = got.argmax(-1), want.argmax(-1)
     margin = want.gather(-1, b[..., None])[..., 0] - want.gather(-1, a[..., None])[..., 0]
     assert bool(((a == b) | (margin <= bound)).all()), (a != b).sum().item()
-    assert (a == b).float().mean().item() >= 0.9
+    # ... and such ties are rare: at most a tenth of the choices (one, at batch 1, of the five there are)
+    assert int((a != b).sum()) <= max(1, a.numel() // 10)
 
     # ---- the decode step as a HIP graph (static token / position buffers): same bits as the eager step ----
     tok = tokens[STEPS - 2].clone()

@@ -206,3 +206,34 @@ def test_swept_gemm_tilings_are_valid_and_override_the_model():
         assert tiling.gemm_tiling(m, n, k, nbits, gs) == cfg, key
         assert tiling.gemm_tiling_model(m, n, k, nbits, gs) != cfg, key
     assert tiling.gemm_tiling(256, 8192 + 128, 8192, 4, 128) == tiling.gemm_tiling_model(256, 8192 + 128, 8192, 4, 128)
+
+
+def test_swept_gemv_tilings_are_valid_and_override_the_model():
+    """core/gemv_tuned_gfx950.json: every entry satisfies the dot2 GEMV kernel's static limits (whole chunks inside a
+    group, a power of two of partial sums, a block of at most 1024 threads, the team covering the row), differs from
+    the analytic default (or it would not be there) and is what ``gemv_tiling`` returns; pinned parameters and other
+    problems get the model."""
+    import json
+    path = os.path.join(os.path.dirname(tiling.__file__), "gemv_tuned_gfx950.json")
+    table = json.load(open(path))
+    assert table, "the shipped table is empty"
+    for key, cfg in table.items():
+        nbits, m, n, k, gs = (int(x) for x in key.split("-"))
+        assert set(cfg) == {"MT", "WK", "WN", "U", "STEPS", "VB"}, key
+        assert tiling.regime_for(m, k, nbits, gs, n) == "gemv", key
+        epc = tiling.elements_per_chunk(nbits, cfg["VB"])
+        assert cfg["VB"] in (4, 8, 16) and gs % epc == 0 and (k * tiling.plane_bits(nbits)) % (8 * cfg["VB"]) == 0, key
+        v = cfg["U"] * cfg["MT"]
+        assert v & (v - 1) == 0 and v <= 64 and 64 * cfg["WK"] * cfg["WN"] <= 1024, key
+        assert tiling.gemv_chunks_per_lane(k, nbits, cfg) * 64 * cfg["WK"] >= k // epc, key
+        assert tiling.gemv_tiling(m, n, k, nbits, gs) == cfg, key
+        assert tiling.gemv_tiling_model(m, n, k, nbits, gs) != cfg, key
+        assert tiling.gemv_tiling(m, n, k, nbits, gs, steps=1) == tiling.gemv_tiling_model(m, n, k, nbits, gs, steps=1), key
+    assert tiling.gemv_tiling(1, 4096 + 16, 4096, 4, 128) == tiling.gemv_tiling_model(1, 4096 + 16, 4096, 4, 128)
+
+
+def test_long_rows_take_up_to_sixteen_waves_and_four_stages():
+    assert tiling.gemv_tiling_model(1, 8192, 28672, 4, 128) == {"MT": 1, "WK": 14, "WN": 1, "U": 4, "STEPS": 4, "VB": 16}
+    assert tiling.gemv_tiling_model(1, 4096, 11008, 4, 128) == {"MT": 1, "WK": 6, "WN": 1, "U": 4, "STEPS": 4, "VB": 16}
+    assert tiling.gemv_tiling_model(1, 5120, 13824, 4, 128)["STEPS"] == 1          # 320 sixteen-row blocks: uneven rounds
+    assert tiling.gemv_tiling_model(2, 8192, 28672, 4, 128)["WK"] <= 8             # two activation rows: eight waves at most
