@@ -10,11 +10,12 @@ The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear 
 (M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
 regimes through the layers' own row-count dispatch.  ``forward`` runs everything else (embedding,
 RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch; ``prefill``
-replaces its norm and SiLU steps by single launches.  A decode
-step runs the steps between the linears as one HIP launch each (residual add + RMSNorm, RoPE + cache
-append + attention of the new position, SiLU * up: libqfactory_hip.so) -- eight launches per layer
-instead of about fifty -- and, up to 32 sequences, five: the kernels for few rows run the residual add and
-RMSNorm in front of their dot products and SiLU * up behind them; ``--torch-glue`` keeps PyTorch ops there for comparison.  One decode step --
+replaces its norm and SiLU steps by single launches.  A decode step has no PyTorch op between the linears:
+up to 32 sequences a layer is five launches -- qkv with the RMSNorm in front of its dot products, RoPE + cache
+append + attention of the new position (libqfactory_hip.so), o adding its result to the residual stream, gate+up
+with the RMSNorm in front and SiLU * up behind, down adding to the residual stream; for more sequences eight
+(residual add + RMSNorm and SiLU * up as launches of their own) -- instead of about fifty; ``--torch-glue`` keeps
+PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
 Prints one JSON line per batch size: tokens/s over the decode phase, prefill time, and the share of
