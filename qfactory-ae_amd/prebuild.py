@@ -252,6 +252,17 @@ def accumulate_cases():
     return [dict(c, epilogue="accumulate") for c in cases]
 
 
+def odd_wave_cases():
+    """GEMM tilings whose wave count along N does not divide the activation tile's 1 KB blocks (3, 5, 6, 7 waves: the
+    waves past the last block fetch it again), pinned explicitly (tests/test_qlinear_gpu.py): ragged M and N, one and two
+    wave groups along K, one and two weight tiles per wave, a tile of four blocks on three waves, 2 and 8 bits."""
+    def tile(bm, nt32, wn, wk, pa):
+        return tuple(sorted({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa}.items()))
+    return [dict(_case(70, 250, 1024), tiling=tile(64, 1, 3, 2, 4)), dict(_case(256, 500, 2048), tiling=tile(256, 1, 7, 1, 3)),
+            dict(_case(100, 960, 1024, 4, 64), tiling=tile(128, 2, 5, 1, 4)), dict(_case(40, 200, 512, 8, 32), tiling=tile(32, 1, 3, 1, 3)),
+            dict(_case(64, 400, 2048, 2, 128, True), tiling=tile(64, 1, 6, 1, 4)), dict(_case(33, 100, 4096, 4, 128), tiling=tile(64, 2, 3, 2, 3))]
+
+
 def search_cases():
     """Problems whose whole tiling search space is compiled (tests/test_tune.py searches on the device)."""
     return [_case(1, 64, 256, 4, 128)]
@@ -277,7 +288,7 @@ def drain_cases(base=None):
 def all_cases(with_drain=True):
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases() + accumulate_cases()):
+              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases() + accumulate_cases() + odd_wave_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
@@ -304,6 +315,8 @@ def qfuncs_of(case):
                          dtype, torch.int8, case["GS"])
         op.init_qfuncs()
         qfuncs += op.qfuncs
+    if case.get("tiling"):
+        qfuncs = [q.clone(tiling_configs=dict(case["tiling"])) for q in qfuncs]
     if case.get("smem_quant"):
         op = QMatmul(_m_bucket(case["M"]), case["N"], case["K"], case["NBITS"], case["sym"],
                      torch.float16, torch.int8, case["GS"])

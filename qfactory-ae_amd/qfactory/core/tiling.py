@@ -599,7 +599,7 @@ def gemm_valid(cfg, K, nbits, group_size):
         return False
     # (asymmetric weights also need K/GS to fill whole zero-point bytes: a property of the packed tensors,
     # checked where they are built and again by the launcher, not a tiling matter -- symmetric ones do not)
-    if (bm * 8) % (64 * wn) or not 3 <= pa <= 12:
+    if not 3 <= pa <= 12:
         return False
     if (bm // 32) * nt32 * 16 > 256:
         return False
@@ -658,7 +658,12 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
             continue
         # 256-row tiles: eight waves side by side (a 256 x 256 block tile, every weight dequantised
         # once); measured 250 against 300 us on 57344 x 8192 at M = 256
-        for wn in ((8,) if bm == 256 else (4, 2, 1)):
+        # any number of waves along N: the count that deals the columns to the 256 CUs in whole rounds wins (57344
+        # columns are 256 tiles of 7 x 32: 230 against 269 us for 224 tiles of 8 x 32 at M = 256; 22016 x 4096 at
+        # M = 256: 58.6 us for six waves against 67.1 for 128 x 256 tiles)
+        # (32-row tiles keep 4 / 2 / 1: with the odd counts the model over-picked them -- mean regret over the 124
+        # swept cells 1.032 against 1.017, worst 1.36 against 1.23)
+        for wn in ((8, 7, 6, 5) if bm == 256 else ((4, 7, 6, 5, 3, 2, 1) if bm >= 64 else (4, 2, 1))):
             for nt32 in ((1, 2) if (bm, wn) == (128, 4) else (1,)):
                 bn = 32 * wn * nt32
                 blocks = -(-N // bn) * -(-M // bm)
@@ -674,8 +679,8 @@ def gemm_tiling(M, N, K, nbits, group_size, **pins):
     # measured slower than four groups with four tiles, 20.6 against 18.3 us on 8192 x 8192 at M = 32, 23.0 against
     # 21.0 on 4096 x 11008 at M = 64)
     wk = max(1, min(4, 8 // wn)) if blocks <= NUM_CUS else 1
-    if bm == 256:
-        wk = 1
+    if bm >= 128:
+        wk = 1                                        # 128-row tiles in two wave groups spill (six waves of 128 x 32: 85 against 38 us)
     nsup = -(-K // (1024 // plane_bits(nbits)))
     wk = max(1, min(wk, nsup))
     # 128 x 256 block tiles of four 128 x 64 waves: three activation tiles in flight measured 128.7 against 156.7 us
@@ -744,7 +749,7 @@ def gemm_candidates(M, N, K, nbits, group_size):
         if bm >= 2 * M and bm > 32:
             continue
         for nt32 in (1, 2):
-            for wn in (1, 2, 4, 8):
+            for wn in (1, 2, 3, 4, 5, 6, 7, 8):          # any count: 57344 columns are 256 tiles of 7 x 32, one per CU
                 for wk in (1, 2, 4, 8):
                     for pa in (3, 4, 6):
                         add({"BM": bm, "NT32": nt32, "WN": wn, "WK": wk, "PA": pa})

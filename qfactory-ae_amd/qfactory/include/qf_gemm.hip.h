@@ -115,7 +115,8 @@ struct GemmCfg {
     static constexpr int SUP_PER_GROUP = (NSUP + WK - 1) / WK;
     static constexpr int ITERS = SUP_PER_GROUP * SUP;          // K-iterations of every group
     static constexpr int UPS = TN * 8 / 64;                    // 16-byte units per lane and super
-    static constexpr int UA = BM * (BK / 8) / TG;              // activation units per thread and iteration
+    static constexpr int AB = BM * (BK / 8) / 64;              // 1 KB blocks (64 16-byte units, 8 rows) of an activation tile
+    static constexpr int UA = (AB + WN - 1) / WN;              // activation units per thread and iteration
     static constexpr int LW = PB;                              // main-plane words per lane, tile and iteration
     static constexpr int NGS = SUPK / GS > 0 ? SUPK / GS : 1;  // groups per row and super
     static constexpr int SREGS = (NGS + 1) / 2;                // registers of fp16 scales per tile and super
@@ -255,7 +256,10 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 
     // ---- activations: UA 16-byte units per lane and iteration, global memory -> LDS ----
     // Instruction p of wave wn fills the 1 KB of 16-byte slots (p*WN + wn)*64 .. +63 of the tile
-    // (the hardware writes the 64 lanes' 16 bytes back to back); slot 8*row + (c ^ (row/2 % 8))
+    // (the hardware writes the 64 lanes' 16 bytes back to back); where WN does not divide the tile's
+    // AB blocks, the instructions past the last block fetch the last block once more -- same bytes to
+    // the same place -- so that every wave issues the same number of loads (the waits count them);
+    // slot 8*row + (c ^ (row/2 % 8))
     // holds columns 8c .. 8c+7 of a row: an XOR swizzle instead of row padding.  A 16-byte fragment
     // read is served 16 lanes (= 16 rows, one column slot) at a time; rows 2a and 2a+1 start 32
     // banks apart and the eight values of a move the slot to eight different 4-bank groups: no
@@ -263,7 +267,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     uint32_t a_off[UA];                                        // byte offset of this lane's units inside the slab
 #pragma unroll
     for (int p = 0; p < UA; p++) {
-        const int u = (p * WN + wn) * 64 + lane;
+        const int u = min(p * WN + wn, C::AB - 1) * 64 + lane;
         const int row = u / 8, c8 = (u % 8) ^ ((row >> 1) & 7);
         a_off[p] = ((uint32_t)min(row, m_total - 1 - m_blk) * C::K + c8 * 8) * 2u;   // rows past the end re-read the last one
     }
@@ -272,9 +276,9 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     auto load_a = [&](int buf, int it) {
         if (QF_GEMM_EXPERIMENT & 8) return;
         const uint8_t* base = a_slab + (size_t)k_of(it) * 2;
-        uint8_t* dst = as_b + (size_t)buf * BM * C::ROWB + (size_t)wn * 1024;
+        uint8_t* dst = as_b + (size_t)buf * BM * C::ROWB;
 #pragma unroll
-        for (int p = 0; p < UA; p++) load_to_lds_16(base + a_off[p], dst + (size_t)p * WN * 1024);
+        for (int p = 0; p < UA; p++) load_to_lds_16(base + a_off[p], dst + (size_t)min(p * WN + wn, C::AB - 1) * 1024);
     };
 
     // ---- one super of this wave's TN weight rows: packed fields, scales, zero-points ----
@@ -659,7 +663,6 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::GS > C::SUPK && C::GS % C::SUPK != 0) why = "GS must divide 1024/NBITS or be a multiple of it";
     else if (C::NGS > 8 || C::ZBITS > 32) why = "too many groups per 128 packed bytes";
     else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
-    else if ((C::BM * (C::BK / 8)) % C::TG != 0) why = "the activation tile must split evenly over a group's threads";
     else if (C::PA < 3 || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12";
     else if (C::LDS_BYTES > 160 * 1024) why = "tiles exceed the 160 KB of LDS";
     else if (C::ACC_PER_THREAD > 256) why = "accumulator tile exceeds the register file";

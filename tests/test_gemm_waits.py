@@ -41,6 +41,21 @@ def test_every_counted_load_is_issued(M, N, K, nbits, gs, tmp_path):
     assert ok, detail
 
 
+@pytest.mark.parametrize("M,N,K,tile", [(256, 57344, 8192, {"BM": 256, "NT32": 1, "WN": 7, "WK": 1, "PA": 3}),
+                                        (64, 22016, 4096, {"BM": 64, "NT32": 1, "WN": 3, "WK": 2, "PA": 4}),
+                                        (128, 960, 2048, {"BM": 128, "NT32": 2, "WN": 5, "WK": 1, "PA": 4})])
+def test_wave_counts_that_do_not_divide_the_activation_tile(M, N, K, tile, tmp_path):
+    """Seven (three, five) waves along N: the tile's 1 KB blocks do not split evenly over them, the waves past the
+    last block fetch it once more, and every wave still issues the loads its waits count."""
+    from qfactory.core import tiling
+    from qfactory.jit.verify import gemm_waits_hold
+    assert tiling.gemm_valid(tile, K, 4, 128)
+    q = _gemm_qfunc(M, N, K, 4, 128)
+    q.tiling_configs = dict(tile)
+    ok, detail = gemm_waits_hold(_isa_of(q, tmp_path), tile["PA"])
+    assert ok, detail
+
+
 def test_checker_rejects_a_missing_load():
     from qfactory.jit.verify import gemm_waits_hold
     load = "\tglobal_load_dwordx4 v[0:3], v4, s[0:1]"

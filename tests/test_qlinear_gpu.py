@@ -313,3 +313,32 @@ def test_the_other_decode_strategy(oracle, case):
     for out, qfunc in zip(outs, variants):
         assert_close(oracle, out, ref, f"{_id(case)} decode={qfunc.decode_strategy}")
     assert not np.array_equal(outs[0], outs[1]) or M * N < 64          # two different computations, not one object twice
+
+
+@pytest.mark.parametrize("case", prebuild.odd_wave_cases(), ids=_id)
+def test_gemm_with_wave_counts_that_do_not_divide_the_activation_tile(oracle, case):
+    """3, 5, 6 or 7 waves along N (57344 columns are 256 tiles of 7 x 32: one per CU): the tiling is pinned, the
+    object is called through its ``launch_m`` and checked against the oracle like any other."""
+    from qfactory.jit import jit
+    M, N, K, nbits, GS, sym = (case[k] for k in ("M", "N", "K", "NBITS", "GS", "sym"))
+    tile = dict(case["tiling"])
+    print(f"[case] gemm {_id(case)} {tile}", flush=True)
+    from qfactory import QLinear
+    A, weight, scale, zero = make_problem(4321 + N + K + M, M, N, K, nbits, GS, sym)
+    layer = QLinear.init(M, K, N, nbits, weight.cuda(), GS, scale.cuda(), None if zero is None else zero.cuda(),
+                         compile_flags=NO_SEARCH)
+    (qfunc,) = prebuild.qfuncs_of(case)
+    assert qfunc.regime == "gemm" and qfunc.tiling_configs == tile
+    runtime = jit.compile(qfunc)
+    assert all(f"{k}={v}" in runtime.description for k, v in tile.items())
+    x = A.cuda()
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    z = layer.z if layer.z is not None else torch.empty(1, dtype=torch.int8, device="cuda")
+    rc = runtime.run_raw(M, (x.data_ptr(), layer.w.data_ptr(), out.data_ptr(), layer.s.data_ptr(), z.data_ptr()),
+                         torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    ref = reference_output(oracle, A, layer.w, layer.s, layer.z, nbits, GS)
+    assert_close(oracle, out.cpu().numpy(), ref, _id(case))
+    # the default tiling of the same problem gives the same values up to the order of the fp32 sums
+    assert ((out.float() - layer(x).float()).norm() / layer(x).float().norm()).item() <= 5e-4
