@@ -718,7 +718,9 @@ def _gemm_tiling_many_rows(M, N, K, nbits, group_size):
     with 0.75 + 0.25 the model kept 128 x 128 tiles in 2.5 rounds on 10240 x 8192 at M = 1024, 294 us,
     where 160 tiles of 256 x 256 take 224 us, and on 22016 x 4096 at M = 512, 146 against 123 us).
     Picks within 4 % of the best of the sweep on 22 of 24 cells (before: 17; worst case 1.35x -> 1.16x).  None when the launch is a
-    single round: the small-M model, which splits K over wave groups, serves those."""
+    single round: the small-M model, which splits K over wave groups, serves those.  (Wave counts of 3, 5, 6, 7
+    along N, which pay for single-round launches, were measured here too: within 2 % of the eight-wave tiles at best
+    over several rounds, and the round model mis-ranks them by up to 12 %; not offered.)"""
     best = None
     for bm, nt32, wn in ((256, 1, 8), (128, 2, 4), (128, 1, 4), (64, 1, 4)):
         cfg = {"BM": bm, "NT32": nt32, "WN": wn, "WK": 1, "PA": 4 if bm <= 128 else 3}
