@@ -122,10 +122,12 @@ def kernel_event_time_us(func, sets, x, n_out, reps=None):
     `reps` back-to-back launches (rotating over the distinct weight sets, at least 512 MB of them) are
     captured in a HIP graph on a side stream; the replay is bracketed by HIP events recorded on the stream
     it is launched on, and the elapsed time is divided by `reps`.  Back-to-back launches on one stream
-    serialise on this GPU, so this is the per-launch duration a kernel trace reports.
+    serialise on this GPU, so this is the per-launch duration a kernel trace reports -- once the replay's own
+    fixed cost (about 9 us between the first event and the first kernel, measured) is spread over enough
+    launches: at least 64 and two passes over the weight sets; 16 launches read 0.5 us per launch high.
     """
     import torch
-    reps = reps or max(16, len(sets))
+    reps = reps or max(64, 2 * len(sets))
     out = torch.empty(x.shape[0], n_out, dtype=torch.float16, device="cuda")
 
     def launches():
@@ -143,7 +145,8 @@ def kernel_event_time_us(func, sets, x, n_out, reps=None):
         with torch.cuda.graph(graph, stream=side):
             launches()
     torch.cuda.current_stream().wait_stream(side)
-    graph.replay()
+    for _ in range(2):                      # the first replay after the allocations above reads 5 - 10 % slow
+        graph.replay()
     torch.cuda.synchronize()
     best = []
     for _ in range(5):
@@ -166,7 +169,7 @@ def stream_read_time_us(nbytes):
     n = cold_copies(nbytes)
     bufs = [torch.randint(-128, 128, (nbytes,), dtype=torch.int8, device="cuda") for _ in range(n)]
     sink = torch.zeros(4096, dtype=torch.int32, device="cuda")          # qf_stream_read writes one word per block, index modulo 4096
-    reps = max(16, n)
+    reps = max(64, 2 * n)
 
     def launches():
         for i in range(reps):
@@ -179,7 +182,8 @@ def stream_read_time_us(nbytes):
     with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
         launches()
     torch.cuda.current_stream().wait_stream(side)
-    graph.replay()
+    for _ in range(2):
+        graph.replay()
     torch.cuda.synchronize()
     times = []
     for _ in range(5):
@@ -204,7 +208,8 @@ def _graph_time_us(launches, reps):
     with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
         launches()
     torch.cuda.current_stream().wait_stream(side)
-    graph.replay()
+    for _ in range(2):
+        graph.replay()
     torch.cuda.synchronize()
     times = []
     for _ in range(5):
@@ -286,7 +291,7 @@ def dense_fp16_time_us(M, N, K, total_bytes=COLD_BYTES):
     for w in ws:
         torch.matmul(x, w.T)
     torch.cuda.synchronize()
-    reps = max(8, n)
+    reps = max(32, 2 * n)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(reps):
@@ -308,7 +313,7 @@ def gemm_report(M=256):
         lin = QLinear.empty(M, K, N, NBITS, GS, sym=False, compile_flags=flags)
         sets = weight_sets(lin, cold_copies(N * K // 2), g)
         x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
-        us = kernel_event_time_us(lin.func, sets, x, N, reps=max(8, len(sets)))
+        us = kernel_event_time_us(lin.func, sets, x, N)
         description = lin.func.runtime.description
         del lin, sets
         torch.cuda.empty_cache()
