@@ -10,11 +10,11 @@ The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear 
 (M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
 regimes through the layers' own row-count dispatch.  ``forward`` runs everything else (embedding,
 RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch; ``prefill``
-replaces its norm and SiLU steps by single launches.  A decode step has no PyTorch op between the linears:
+replaces its norm steps by single launches and forms SiLU * up in the gate+up projection's epilogue.  A decode step has no PyTorch op between the linears:
 up to 32 sequences a layer is five launches -- qkv with the RMSNorm in front of its dot products, RoPE + cache
 append + attention of the new position (libqfactory_hip.so), o adding its result to the residual stream, gate+up
-with the RMSNorm in front and SiLU * up behind, down adding to the residual stream; for more sequences eight
-(residual add + RMSNorm and SiLU * up as launches of their own) -- instead of about fifty; ``--torch-glue`` keeps
+with the RMSNorm in front and SiLU * up behind, down adding to the residual stream; for more sequences seven
+(residual add + RMSNorm twice as launches of their own, SiLU * up in the GEMM kernel's epilogue) -- instead of about fifty; ``--torch-glue`` keeps
 PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
@@ -136,8 +136,9 @@ class QuantLlama:
         return last @ self.lm_head.T
 
     def prefill(self, tokens, pos):
-        """``forward`` with the residual add + RMSNorm and SiLU * up steps as single launches of
-        libqfactory_hip.so (any number of rows); RoPE, the cache update and causal attention stay PyTorch ops."""
+        """``forward`` with the residual add + RMSNorm as single launches of libqfactory_hip.so (any number of rows)
+        and SiLU * up in the gate+up projection's epilogue (or a launch of its own where the kernel cannot); RoPE,
+        the cache update and causal attention stay PyTorch ops."""
         from qfactory import native
         shape = self.shape
         B, T = tokens.shape
@@ -156,7 +157,10 @@ class QuantLlama:
             att = F.scaled_dot_product_attention(q, self.k_cache[li], self.v_cache[li], attn_mask=mask)
             delta = self.linear(layer["o"], att.permute(0, 2, 1, 3).reshape(B * T, shape.hidden))
             native.add_rmsnorm(x, delta, layer["norm2"], hdn, shape.eps)
-            native.silu_mul(self.linear(layer["gate_up"], hdn), act)
+            if self.linear is self._own_linear:
+                act = layer["gate_up"].forward_silu_mul(hdn)          # SiLU(gate) * up in the projection's epilogue where it can
+            else:
+                native.silu_mul(self.linear(layer["gate_up"], hdn), act)
             delta = self.linear(layer["down"], act)
         last = (x + delta).reshape(B, T, shape.hidden)[:, -1].contiguous()
         native.add_rmsnorm(last, None, self.final_norm, last, shape.eps)
@@ -282,6 +286,8 @@ def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
             "between_linears": "torch ops" if torch_glue else (
                 "attention one HIP launch (libqfactory_hip.so); residual add + RMSNorm and SiLU * up inside the projections"
                 if model.layers[0]["gate_up"].fuses_add_rmsnorm(batch, silu_mul=True) and model.fuse_norm
+                else "one HIP launch per step (libqfactory_hip.so); SiLU * up inside the gate+up projection"
+                if model.layers[0]["gate_up"].fuses_silu_mul(batch)
                 else "one HIP launch per step (libqfactory_hip.so)")}
 
 

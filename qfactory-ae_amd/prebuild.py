@@ -205,6 +205,11 @@ def silu_mul_cases():
              # every bit width, a last block with fewer pairs
              _case(16, 22016, 4096), _case(16, 1024, 256, 4, 64), _case(5, 96, 1024, 4, 128), _case(12, 4128, 2048, 3, 64),
              _case(32, 160, 4096, 2, 128, True), _case(7, 18016, 2048, 8, 128)]
+    # the GEMM kernel: the decode loop's at batch 64 and at prefill row counts, the tiny model's, ragged M,
+    # every bit width, a last block with waves past N
+    cases += [_case(M, 22016, 4096) for M in (64, 128, 256, 512, 1024)]
+    cases += [_case(64, 1024, 256, 4, 64), _case(100, 4128, 2048, 3, 64), _case(40, 160, 4096, 2, 128, True),
+              _case(200, 2208, 2048, 8, 128), _case(33, 96, 1024, 4, 128)]
     return [dict(c, epilogue="silu_mul") for c in cases]
 
 

@@ -254,9 +254,9 @@ class QMatmulQFunc(QFunc):
                 "only the kernels for up to 32 rows, on fp16, add their result to the output"
             defines["QF_OUT_ACCUMULATE"] = 1
         elif self.output_epilogue != "none":
-            assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
-                "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, write silu(gate) * up"
-            defines["QF_GEMV_GATE_UP_SILU" if self.regime == "gemv" else "QF_MGEMV_GATE_UP_SILU"] = 1
+            assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv", "gemm") and self.act_dtype == torch.float16, \
+                "only the dot2 GEMV, the A-stationary and the GEMM kernel, on fp16, write silu(gate) * up"
+            defines[{"gemv": "QF_GEMV_GATE_UP_SILU", "mgemv": "QF_MGEMV_GATE_UP_SILU", "gemm": "QF_GEMM_GATE_UP_SILU"}[self.regime]] = 1
         if self.input_prologue != "none":
             assert self.input_prologue == "add_rmsnorm" and self.regime in ("gemv", "mgemv") and self.act_dtype == torch.float16, \
                 "only the dot2 GEMV kernel and the A-stationary kernel, on fp16, run the residual add and RMSNorm themselves"

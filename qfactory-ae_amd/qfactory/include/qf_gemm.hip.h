@@ -77,6 +77,16 @@
 #define QF_GEMM_XCD_MAP 0
 #endif
 
+// 1: the weight matrix is a fused gate+up projection (rows 0 .. N/2-1 gate, rows N/2 .. N-1 up) and the kernel
+// writes the (M, N/2) SwiGLU activation out[m][i] = fp16(silu(gate[m][i])) * up[m][i] instead of the (M, N)
+// projection.  A wave's TN weight rows alternate between a gate row and its up row (local row r is packed row
+// first/2 + r/2 + (r % 2) * N/2), so a lane's four consecutive accumulators of one m are two (gate, up) pairs and
+// the epilogue needs nothing from another lane.  Same roundings as the projection followed by qf_silu_mul of
+// libqfactory_hip.so (silu_mul_f16 in qf_common.hip.h).  The reference has no such fusion.
+#ifndef QF_GEMM_GATE_UP_SILU
+#define QF_GEMM_GATE_UP_SILU 0
+#endif
+
 // The activation tiles go from global memory to LDS without passing through registers, so this kernel
 // cannot convert them on the way: it reads fp16 activations only (its output may be bf16).
 static_assert(!QF_IN_BF16, "the GEMM kernel takes fp16 activations: convert bf16 rows before the launch");
@@ -210,6 +220,7 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     constexpr int MT32 = C::MT32, NT32 = C::NT32, WPP = C::WPP;
     constexpr int SUP = C::SUP, UPS = C::UPS, UA = C::UA, LW = C::LW, NGS = C::NGS, SREGS = C::SREGS;
     constexpr uint32_t ZMASK = (1u << C::ZFB) - 1u;
+    constexpr bool SILU = QF_GEMM_GATE_UP_SILU != 0;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
@@ -285,22 +296,26 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     struct Quant { uint32_t s[NT32][SREGS]; uint32_t z[NT32]; };
     struct WStage { u32x4 w[UPS]; u32x4 h[C::HI ? C::UPH : 1]; };
     uint32_t w_off[UPS], h_off[C::HI ? C::UPH : 1], s_off[NT32], z_off[NT32];   // per-lane byte offsets from the wave's first row
-    const int n_base = min(n_wave, C::N - 1);                  // a wave wholly past the last row re-reads it
+    // first packed row of the wave and the packed row of its local row r, relative to it.  Plain: rows n_wave + r,
+    // clamped to the last row (a wave wholly past the last row re-reads it).  Gate+up (N a multiple of TN, so a
+    // wave is inside or wholly outside): local rows 2i, 2i+1 are gate row first/2 + i and its up row N/2 further on.
+    const int n_base = SILU ? min(n_wave, C::N - TN) / 2 : min(n_wave, C::N - 1);
+    auto rel_row = [&](int r) { return SILU ? (r >> 1) + (r & 1) * (C::N / 2) : min(r, C::N - 1 - n_base); };
 #pragma unroll
     for (int p = 0; p < UPS; p++) {
         const int u = lane + 64 * p;
-        w_off[p] = (uint32_t)min(u / 8, C::N - 1 - n_base) * C::RB + (u % 8) * 16;
+        w_off[p] = (uint32_t)rel_row(u / 8) * C::RB + (u % 8) * 16;
     }
     if constexpr (C::HI) {
 #pragma unroll
         for (int p = 0; p < C::UPH; p++) {
             const int u = lane + 64 * p;                        // four lanes share a row: 64 bytes per super
-            h_off[p] = (uint32_t)min(u / 4, C::N - 1 - n_base) * C::RB + C::HI_OFF + (u % 4) * 16;
+            h_off[p] = (uint32_t)rel_row(u / 4) * C::RB + C::HI_OFF + (u % 4) * 16;
         }
     }
 #pragma unroll
     for (int j = 0; j < NT32; j++) {
-        const uint32_t row = (uint32_t)min(j * 32 + li, C::N - 1 - n_base);
+        const uint32_t row = (uint32_t)rel_row(j * 32 + li);
         s_off[j] = row * C::G * 2u;
         z_off[j] = row * C::ZRB;
     }
@@ -633,6 +648,15 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int n = n_wave + j * 32 + 8 * q + 4 * kb;
+                if constexpr (SILU) {
+                    // columns n, n+1 and n+2, n+3 are (gate, up) of outputs n/2 and n/2 + 1
+                    if (n < C::N) {
+                        const uint32_t lo = silu_mul_f16(acc[j][i][4 * q], acc[j][i][4 * q + 1]);
+                        const uint32_t hi = silu_mul_f16(acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]);
+                        *reinterpret_cast<uint32_t*>(Cout + (size_t)m * (C::N / 2) + (n >> 1)) = lo | (hi << 16);
+                    }
+                    continue;
+                }
                 uint16_t h[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) h[e] = f32_to_out_bits(acc[j][i][4 * q + e]);
@@ -666,6 +690,9 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::PA < 3 || C::PA > 12) why = "PA (activation tiles in flight) must be 3 .. 12";
     else if (C::LDS_BYTES > 160 * 1024) why = "tiles exceed the 160 KB of LDS";
     else if (C::ACC_PER_THREAD > 256) why = "accumulator tile exceeds the register file";
+    else if (QF_GEMM_GATE_UP_SILU && (C::N % 2 != 0 || C::N % C::TN != 0)) why = "gate+up rows come in pairs inside a wave: N must be a multiple of 32 * NT32";
+    else if (QF_GEMM_GATE_UP_SILU && QF_OUT_BF16) why = "the SwiGLU epilogue is fp16 only";
+    else if (QF_GEMM_GATE_UP_SILU && ((size_t)C::N / 2 + C::TN) * C::RB >= ((size_t)1 << 32)) why = "gate+up: half the packed weight does not fit a 32-bit row offset";
     if (why) {
         fprintf(stderr, "qfactory gemm: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d BM=%d NT32=%d WN=%d WK=%d PA=%d)\n",
                 why, C::NBITS, C::GS, C::N, C::K, C::BM, C::NT32, C::WN, C::WK, C::PA);

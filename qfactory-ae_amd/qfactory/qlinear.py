@@ -138,13 +138,17 @@ class GPTQLinear(torch.nn.Module):
 
     def fuses_silu_mul(self, m, dtype=torch.float16):
         """Does ``forward_silu_mul`` on ``m`` rows run as one launch?  Where the dot2 GEMV kernel serves and its
-        rows come in pairs, or the A-stationary kernel and gate and up are whole 16-row tiles."""
+        rows come in pairs, or the A-stationary kernel and gate and up are whole 16-row tiles, or the GEMM kernel
+        and every wave holds whole (gate, up) pairs of its own (N a multiple of the wave's weight rows)."""
         bucket = _m_bucket(m)
         if dtype != torch.float16 or self.out_features % 2:
             return False
         regime = tiling.regime_for(bucket, self.in_features, self.n_bits, self.group_size, self.out_features)
         if regime == "mgemv":
             return self.out_features % 32 == 0
+        if regime == "gemm":
+            t = tiling.gemm_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)
+            return self.out_features % (32 * t["NT32"]) == 0
         if regime != "gemv":
             return False
         return tiling.gemv_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)["U"] % 2 == 0
@@ -218,9 +222,9 @@ class GPTQLinear(torch.nn.Module):
 
     def forward_silu_mul(self, x: torch.Tensor):
         """For a fused gate+up projection (rows 0 .. N/2-1 gate, the rest up): the SwiGLU activation
-        ``silu(gate) * up`` of shape (M, N/2), i.e. ``silu_mul(self(x))``.  Up to 32 rows the product is formed in
-        the kernel's final sum (one launch); otherwise by ``forward`` followed by ``qf_silu_mul``.  Both give
-        the same bits.  Not in the reference, whose end-to-end runs leave the step to vLLM's ``SiluAndMul``."""
+        ``silu(gate) * up`` of shape (M, N/2), i.e. ``silu_mul(self(x))``.  The product is formed in the kernel's
+        epilogue (one launch) wherever ``fuses_silu_mul`` says so; otherwise by ``forward`` followed by
+        ``qf_silu_mul``.  Both give the same bits.  Not in the reference, whose end-to-end runs leave the step to vLLM's ``SiluAndMul``."""
         m, half = x.shape[0], self.out_features // 2
         output = torch.empty(m, half, dtype=x.dtype, device=x.device)
         if m == 0:

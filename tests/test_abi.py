@@ -107,6 +107,23 @@ def test_add_to_output_epilogue_is_a_header_switch_of_the_small_row_kernels():
         bf.emit()
 
 
+def test_swiglu_epilogue_is_a_header_switch_of_three_kernels():
+    from qfactory.core.qfunc import QMatmulQFunc
+    from qfactory.core.qtile import AsymQTile, QTile
+    for m, k, regime, define in ((1, 512, "gemv", "QF_GEMV_GATE_UP_SILU"), (16, 1024, "mgemv", "QF_MGEMV_GATE_UP_SILU"),
+                                 (64, 512, "gemm", "QF_GEMM_GATE_UP_SILU")):
+        q = QMatmulQFunc(QTile((m, k), torch.float16, 16), AsymQTile((64, k), torch.int8, 4, (1, 128)), "nt")
+        assert q.regime == regime
+        q.output_epilogue = "silu_mul"
+        src = q.emit()
+        assert f"#define {define} 1" in src and "epilogue=silu_mul" in src
+    skinny = QMatmulQFunc(QTile((16, 11008), torch.float16, 16), AsymQTile((64, 11008), torch.int8, 4, (1, 128)), "nt")
+    assert skinny.regime == "skinny"
+    skinny.output_epilogue = "silu_mul"
+    with pytest.raises(AssertionError):
+        skinny.emit()
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from qfactory import native
     monkeypatch.setattr(native, "_lib", None)
