@@ -10,11 +10,11 @@ The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear 
 (M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
 regimes through the layers' own row-count dispatch.  ``forward`` runs everything else (embedding,
 RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch; ``prefill``
-replaces its norm steps by single launches and forms SiLU * up in the gate+up projection's epilogue.  A decode step has no PyTorch op between the linears:
+replaces its norm steps by single launches and forms the residual adds and SiLU * up in the projections' epilogues.  A decode step has no PyTorch op between the linears:
 up to 32 sequences a layer is five launches -- qkv with the RMSNorm in front of its dot products, RoPE + cache
 append + attention of the new position (libqfactory_hip.so), o adding its result to the residual stream, gate+up
 with the RMSNorm in front and SiLU * up behind, down adding to the residual stream; for more sequences seven
-(residual add + RMSNorm twice as launches of their own, SiLU * up in the GEMM kernel's epilogue) -- instead of about fifty; ``--torch-glue`` keeps
+(the two RMSNorms as launches of their own; residual adds and SiLU * up in the GEMM kernel's epilogues) -- instead of about fifty; ``--torch-glue`` keeps
 PyTorch ops there for comparison.  One decode step --
 including the argmax and the position update -- is captured in a HIP graph and replayed per token.
 
@@ -136,16 +136,17 @@ class QuantLlama:
         return last @ self.lm_head.T
 
     def prefill(self, tokens, pos):
-        """``forward`` with the residual add + RMSNorm as single launches of libqfactory_hip.so (any number of rows)
-        and SiLU * up in the gate+up projection's epilogue (or a launch of its own where the kernel cannot); RoPE,
-        the cache update and causal attention stay PyTorch ops."""
+        """``forward`` with the RMSNorm as a single launch of libqfactory_hip.so (any number of rows), the residual
+        adds in the o and down projections' epilogues and SiLU * up in the gate+up projection's (or launches of their
+        own where a kernel cannot); RoPE, the cache update and causal attention stay PyTorch ops."""
         from qfactory import native
         shape = self.shape
         B, T = tokens.shape
         H, hd = shape.heads, shape.hidden // shape.heads
         x = self.embed[tokens].reshape(B * T, shape.hidden)                          # residual stream, updated in place
         hdn = torch.empty_like(x)
-        act = torch.empty(B * T, shape.mlp, dtype=torch.float16, device="cuda")
+        own = self.linear is self._own_linear
+        act = None if own else torch.empty(B * T, shape.mlp, dtype=torch.float16, device="cuda")
         mask = (torch.arange(shape.max_len, device="cuda")[None, :] <= pos[:, None])[None, None]
         delta = None
         for li, layer in enumerate(self.layers):
@@ -155,14 +156,19 @@ class QuantLlama:
             self.k_cache[li].index_copy_(2, pos, k)
             self.v_cache[li].index_copy_(2, pos, v)
             att = F.scaled_dot_product_attention(q, self.k_cache[li], self.v_cache[li], attn_mask=mask)
-            delta = self.linear(layer["o"], att.permute(0, 2, 1, 3).reshape(B * T, shape.hidden))
+            att = att.permute(0, 2, 1, 3).reshape(B * T, shape.hidden)
+            if own:
+                # the o and down projections add their result to the residual stream themselves (the norms then only
+                # read it), SiLU(gate) * up is the gate+up projection's epilogue where it can be
+                layer["o"].forward_accumulate(att, x)
+                native.add_rmsnorm(x, None, layer["norm2"], hdn, shape.eps)
+                layer["down"].forward_accumulate(layer["gate_up"].forward_silu_mul(hdn), x)
+                continue
+            delta = self.linear(layer["o"], att)
             native.add_rmsnorm(x, delta, layer["norm2"], hdn, shape.eps)
-            if self.linear is self._own_linear:
-                act = layer["gate_up"].forward_silu_mul(hdn)          # SiLU(gate) * up in the projection's epilogue where it can
-            else:
-                native.silu_mul(self.linear(layer["gate_up"], hdn), act)
+            native.silu_mul(self.linear(layer["gate_up"], hdn), act)
             delta = self.linear(layer["down"], act)
-        last = (x + delta).reshape(B, T, shape.hidden)[:, -1].contiguous()
+        last = (x if delta is None else x + delta).reshape(B, T, shape.hidden)[:, -1].contiguous()
         native.add_rmsnorm(last, None, self.final_norm, last, shape.eps)
         return last @ self.lm_head.T
 
@@ -186,6 +192,18 @@ class QuantLlama:
                 layer["o"].forward_accumulate(self._att, x)
                 act = layer["gate_up"].forward_add_rmsnorm(x, None, layer["norm2"], shape.eps, silu_mul=True)
                 layer["down"].forward_accumulate(act, x)
+            native.add_rmsnorm(x, None, self.final_norm, self._hdn, shape.eps)
+            return self._hdn @ self.lm_head.T
+        if self.linear is self._own_linear and first["o"].fuses_accumulate(rows) and first["down"].fuses_accumulate(rows):
+            # seven launches per layer: the o and down projections add their result to the residual stream themselves
+            # (the norms then only read it), SiLU(gate) * up is the gate+up projection's epilogue where it can be
+            for li, layer in enumerate(self.layers):
+                native.add_rmsnorm(x, None, layer["norm1"], self._hdn, shape.eps)
+                qkv = layer["qkv"](self._hdn)
+                native.rope_decode_attention(qkv, pos, self.cos, self.sin, self.k_cache[li], self.v_cache[li], self._att)
+                layer["o"].forward_accumulate(self._att, x)
+                native.add_rmsnorm(x, None, layer["norm2"], self._hdn, shape.eps)
+                layer["down"].forward_accumulate(layer["gate_up"].forward_silu_mul(self._hdn), x)
             native.add_rmsnorm(x, None, self.final_norm, self._hdn, shape.eps)
             return self._hdn @ self.lm_head.T
         for li, layer in enumerate(self.layers):

@@ -245,7 +245,7 @@ def norm_prologue_cases():
 
 
 def accumulate_cases():
-    """Projections that add their result to the output (GPTQLinear.forward_accumulate, up to 32 rows): the decode
+    """Projections that add their result to the output (GPTQLinear.forward_accumulate): the decode
     loop's o and down at batch 1 / 2 / 16, the tiny test model's, and the shapes of tests/test_norm_prologue_gpu.py
     (dot2 GEMV with one wave per team -- stored from the lane -- and several; A-stationary and streaming kernels;
     every bit width; ragged M and N)."""
@@ -254,6 +254,11 @@ def accumulate_cases():
     cases += [_case(1, 100, 256), _case(2, 77, 1024, 3, 128, True), _case(1, 130, 2048, 8, 128, True), _case(1, 48, 4096, 2, 128),
               _case(5, 96, 1024), _case(12, 100, 2048, 3, 64), _case(32, 40, 1024, 8, 128),
               _case(5, 100, 11008), _case(16, 64, 14336, 2, 512, True), _case(9, 64, 8192, 8, 128)]
+    # the GEMM kernel: the decode loop's at batch 64 and at prefill row counts, the tiny model's, ragged M, N not a
+    # multiple of four (element-wise stores), every bit width
+    cases += [_case(M, N, K) for N, K in ((4096, 4096), (4096, 11008)) for M in (64, 128, 256, 512, 1024)]
+    cases += [_case(64, N, K, 4, 64) for N, K in ((256, 256), (256, 512))]
+    cases += [_case(40, 96, 1024), _case(100, 77, 1024, 3, 128, True), _case(33, 130, 2048, 8, 128, True), _case(200, 2208, 4096, 2, 128)]
     return [dict(c, epilogue="accumulate") for c in cases]
 
 

@@ -250,8 +250,8 @@ class QMatmulQFunc(QFunc):
             if self.converts_activations:
                 defines["QF_IN_BF16"] = 1
         if self.output_epilogue == "accumulate":
-            assert self.regime in ("gemv", "mgemv", "skinny") and self.act_dtype == torch.float16, \
-                "only the kernels for up to 32 rows, on fp16, add their result to the output"
+            assert self.regime in ("gemv", "mgemv", "skinny", "gemm") and self.act_dtype == torch.float16, \
+                "every kernel but the generic matrix-core fallback, on fp16, can add its result to the output"
             defines["QF_OUT_ACCUMULATE"] = 1
         elif self.output_epilogue != "none":
             assert self.output_epilogue == "silu_mul" and self.regime in ("gemv", "mgemv", "gemm") and self.act_dtype == torch.float16, \

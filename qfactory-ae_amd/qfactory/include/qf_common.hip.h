@@ -93,7 +93,7 @@ __device__ __forceinline__ uint16_t f32_to_out_bits(float f) {
 // 1: the kernel adds its result to what the output already holds -- out = fp16(out + fp16(result)), the two roundings
 // of a projection followed by a residual add -- instead of overwriting it: the o and down projections of a decoder
 // layer writing straight into the residual stream.  Every element is still touched by exactly one lane (read, then
-// written).  fp16 only; the kernels for up to 32 rows.  Not in the reference.
+// written).  fp16 only.  Not in the reference.
 #ifndef QF_OUT_ACCUMULATE
 #define QF_OUT_ACCUMULATE 0
 #endif

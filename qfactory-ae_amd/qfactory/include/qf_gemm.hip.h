@@ -662,11 +662,21 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
                 for (int e = 0; e < 4; e++) h[e] = f32_to_out_bits(acc[j][i][4 * q + e]);
                 uint16_t* dst = Cout + (size_t)m * C::N + n;
                 if constexpr (C::N % 4 == 0) {
-                    if (n < C::N) *reinterpret_cast<u32x2*>(dst) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                    if (n < C::N) {
+                        if constexpr (QF_OUT_ACCUMULATE != 0) {
+                            // out = fp16(out + fp16(projection)): the lane reads the four elements it is about to write
+                            const u32x2 old = *reinterpret_cast<const u32x2*>(dst);
+                            const uint16_t o[4] = {(uint16_t)old.x, (uint16_t)(old.x >> 16), (uint16_t)old.y, (uint16_t)(old.y >> 16)};
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                h[e] = __builtin_bit_cast(uint16_t, (_Float16)(__builtin_bit_cast(_Float16, o[e]) + __builtin_bit_cast(_Float16, h[e])));
+                        }
+                        *reinterpret_cast<u32x2*>(dst) = u32x2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                    }
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (n + e < C::N) dst[e] = h[e];
+                        if (n + e < C::N) store_out(dst + e, acc[j][i][4 * q + e]);
                 }
             }
         }
@@ -692,6 +702,7 @@ int gemm_launch(const void* A, const void* W, void* Cout, const void* S, const v
     else if (C::ACC_PER_THREAD > 256) why = "accumulator tile exceeds the register file";
     else if (QF_GEMM_GATE_UP_SILU && (C::N % 2 != 0 || C::N % C::TN != 0)) why = "gate+up rows come in pairs inside a wave: N must be a multiple of 32 * NT32";
     else if (QF_GEMM_GATE_UP_SILU && QF_OUT_BF16) why = "the SwiGLU epilogue is fp16 only";
+    else if (QF_OUT_ACCUMULATE && (QF_OUT_BF16 || QF_GEMM_GATE_UP_SILU)) why = "adding to the output is fp16 only and not combined with the SwiGLU epilogue";
     else if (QF_GEMM_GATE_UP_SILU && ((size_t)C::N / 2 + C::TN) * C::RB >= ((size_t)1 << 32)) why = "gate+up: half the packed weight does not fit a 32-bit row offset";
     if (why) {
         fprintf(stderr, "qfactory gemm: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d BM=%d NT32=%d WN=%d WK=%d PA=%d)\n",

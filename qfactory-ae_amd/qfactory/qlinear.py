@@ -154,15 +154,16 @@ class GPTQLinear(torch.nn.Module):
         return tiling.gemv_tiling(bucket, self.out_features, self.in_features, self.n_bits, self.group_size)["U"] % 2 == 0
 
     def fuses_accumulate(self, m, dtype=torch.float16):
-        """Does ``forward_accumulate`` on ``m`` rows run as one launch?  Up to 32 rows, fp16."""
+        """Does ``forward_accumulate`` on ``m`` rows run as one launch?  fp16, every kernel but the generic fallback."""
         regime = tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features)
-        return dtype == torch.float16 and regime in ("gemv", "mgemv", "skinny")
+        return dtype == torch.float16 and regime in ("gemv", "mgemv", "skinny", "gemm")
 
     def forward_accumulate(self, x: torch.Tensor, out: torch.Tensor):
         """``out += self(x)`` in place: ``out = fp16(out + fp16(projection))``, the two roundings of the projection
         followed by a residual add -- the o and down projections of a decoder layer writing into the residual stream.
-        One launch up to 32 rows (the kernel's final sum reads the output element it is about to write); otherwise
-        ``forward`` and an in-place add, which give the same bits.  Not in the reference."""
+        One launch (the kernel's final sum reads the output element it is about to write) wherever
+        ``fuses_accumulate`` says so; otherwise ``forward`` and an in-place add, which give the same bits.  Not in
+        the reference."""
         m = x.shape[0]
         assert out.shape == (m, self.out_features) and out.dtype == x.dtype and out.is_contiguous()
         if m == 0:

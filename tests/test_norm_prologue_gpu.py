@@ -83,7 +83,7 @@ def test_projection_with_residual_add_and_rmsnorm_in_front(oracle, case, with_de
     assert int(ulp.max()) <= 2 and float((ulp > 0).float().mean()) < 0.02
 
 
-@pytest.mark.parametrize("case", prebuild.accumulate_cases() + [dict(prebuild._case(40, 96, 1024), epilogue="accumulate")], ids=_id)
+@pytest.mark.parametrize("case", prebuild.accumulate_cases(), ids=_id)
 def test_projection_added_to_the_output_in_place(case):
     """``forward_accumulate``: out = fp16(out + fp16(projection)) -- the kernel's own projection (checked against the
     oracle in tests/test_qlinear_gpu.py) and one fp16 add, so the result equals ``out + layer(x)`` bit for bit."""
@@ -101,11 +101,9 @@ def test_projection_added_to_the_output_in_place(case):
     want = before + layer(x)
     torch.cuda.synchronize()
     assert torch.equal(out, want)
-    if layer.fuses_accumulate(M):
-        desc = layer._funcs[(_m_bucket(M), torch.float16, "accumulate")].runtime.description
-        assert "epilogue=accumulate" in desc
-    else:
-        assert M > 32
+    assert layer.fuses_accumulate(M)
+    desc = layer._funcs[(_m_bucket(M), torch.float16, "accumulate")].runtime.description
+    assert "epilogue=accumulate" in desc and ("regime=gemm" in desc) == (M > 32)
     assert layer.forward_accumulate(x[:0], out[:0]).shape == (0, N)
 
 
