@@ -124,6 +124,7 @@ def large_parity_cases():
     return ([_case(M, N, K) for N, K in LLAMA3_70B for M in (32, 64, 128, 256)]
             + [_case(64, N, K) for N, K in LLAMA2_7B]              # the batch-64 decode linears
             + [_case(512, 10240, 8192), _case(1024, 12288, 4096), _case(700, 22016, 4096), _case(512, 22016, 4096), _case(1024, 10240, 8192)]
+            + [_case(2048, 12288, 4096), _case(3000, 4096, 11008), _case(8192, 4096, 4096)]      # the 2048- and 4096-row buckets
             # the large block tiles at the other bit widths, group sizes and with a partial last window
             + [_case(256, 16384, 4096, 2, 64), _case(256, 16384, 4096, 3, 128, True), _case(256, 16384, 4096, 8, 32),
                _case(512, 16384, 4224, 4, 64), _case(256, 57344, 2816, 2, 128, True), _case(1024, 16384, 4096, 3, 128, True)])
@@ -189,7 +190,7 @@ TINY_LLAMA = [(768, 256), (256, 256), (1024, 256), (256, 512)]      # the decode
 def decode_cases():
     """decode_llama.py: Llama-2-7B shapes at batch 1 / 16 / 64 (decode) and at prefill row counts,
     plus the tiny model tests/test_decode_gpu.py runs."""
-    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 512, 1024)]
+    cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 512, 1024, 2048, 4096)]
     cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
     return cases + silu_mul_cases()
 
@@ -207,7 +208,7 @@ def silu_mul_cases():
              _case(32, 160, 4096, 2, 128, True), _case(7, 18016, 2048, 8, 128)]
     # the GEMM kernel: the decode loop's at batch 64 and at prefill row counts, the tiny model's, ragged M,
     # every bit width, a last block with waves past N
-    cases += [_case(M, 22016, 4096) for M in (64, 128, 256, 512, 1024)]
+    cases += [_case(M, 22016, 4096) for M in (64, 128, 256, 512, 1024, 2048, 4096)]
     cases += [_case(64, 1024, 256, 4, 64), _case(100, 4128, 2048, 3, 64), _case(40, 160, 4096, 2, 128, True),
               _case(200, 2208, 2048, 8, 128), _case(33, 96, 1024, 4, 128)]
     return [dict(c, epilogue="silu_mul") for c in cases]
@@ -256,7 +257,7 @@ def accumulate_cases():
               _case(5, 100, 11008), _case(16, 64, 14336, 2, 512, True), _case(9, 64, 8192, 8, 128)]
     # the GEMM kernel: the decode loop's at batch 64 and at prefill row counts, the tiny model's, ragged M, N not a
     # multiple of four (element-wise stores), every bit width
-    cases += [_case(M, N, K) for N, K in ((4096, 4096), (4096, 11008)) for M in (64, 128, 256, 512, 1024)]
+    cases += [_case(M, N, K) for N, K in ((4096, 4096), (4096, 11008)) for M in (64, 128, 256, 512, 1024, 2048, 4096)]
     cases += [_case(64, N, K, 4, 64) for N, K in ((256, 256), (256, 512))]
     cases += [_case(40, 96, 1024), _case(100, 77, 1024, 3, 128, True), _case(33, 130, 2048, 8, 128, True), _case(200, 2208, 4096, 2, 128)]
     return [dict(c, epilogue="accumulate") for c in cases]

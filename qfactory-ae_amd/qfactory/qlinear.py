@@ -27,7 +27,9 @@ def _m_bucket(m):
     if m <= 16:
         return 16
     bucket = 32
-    while bucket < m and bucket < 1024:        # 512 and 1024: prefill-sized tiles (256 x 256 blocks on wide layers)
+    # 512 .. 4096: prefill-sized tiles.  Several rounds of blocks pay for 256 x 256 tiles where one round of the
+    # same layer does not (4096 x 11008: 128 x 128 tiles at 1024 rows, 256 x 256 from 4096 rows on, 884 -> 699 us at 8192 rows)
+    while bucket < m and bucket < 4096:
         bucket *= 2
     return bucket
 
@@ -70,7 +72,8 @@ class GPTQLinear(torch.nn.Module):
 
         self._funcs = {}
         self._launchers = {}            # (rows, dtype) -> launch(activation, output) bound to this layer's packed tensors
-        self.func = self._compile(batch_size, self.compile_flags)
+        # the specialisation of the hint's row-count bucket: the one forward() looks up for that many rows
+        self.func = self._compile(_m_bucket(batch_size), self.compile_flags)
         self._funcs[(_m_bucket(batch_size), torch.float16)] = self.func
 
     def __setattr__(self, name, value):

@@ -110,8 +110,8 @@ def test_emit_names_the_kernel_of_the_regime(regime, M, N, K, nbits):
 
 def test_row_count_buckets():
     from qfactory.qlinear import _m_bucket
-    assert [_m_bucket(m) for m in (1, 2, 3, 16, 17, 32, 33, 100, 256, 257, 512, 700, 1024, 5000)] == \
-        [1, 2, 16, 16, 32, 32, 64, 128, 256, 512, 512, 1024, 1024, 1024]
+    assert [_m_bucket(m) for m in (1, 2, 3, 16, 17, 32, 33, 100, 256, 257, 512, 700, 1024, 1025, 2048, 3000, 5000, 8192)] == \
+        [1, 2, 16, 16, 32, 32, 64, 128, 256, 512, 512, 1024, 1024, 2048, 2048, 4096, 4096, 4096]
 
 
 def test_prefill_sizes_use_the_many_rows_model_only_for_several_rounds():
