@@ -17,8 +17,9 @@ read of the same number of bytes, and a large dense fp16 GEMM of the vendor libr
 `cpu_baseline` = the torch CPU dequant+matmul port of the reference's test path on the same four
 shapes, on this machine's host cores.  Further sections, none of them part of `value`:
 `small_m` (configs[1] at M = 4 / 16, configs[2]: the bit-width sweep at N = K = 8192, and the
-Llama-3-70B shapes at M = 1), `gemm_m256` and `gemm_m32_m64_m128` (configs[3]) and `decode`
-(configs[4]: the Llama-2-7B-shaped decode loop at batch 1 / 16 / 64).
+Llama-3-70B shapes at M = 1), `gemm_m256` and `gemm_m32_m64_m128` (configs[3]), `gemm_prefill_m8192`
+(the Llama-2-7B layers at configs[4]'s prefill row count) and `decode` (configs[4]: the Llama-2-7B-shaped
+decode loop at batch 1 / 16 / 64).
 
 Every per-kernel timing rotates over at least 512 MB of distinct packed weights (twice the 256 MB
 Infinity Cache), so each launch streams its weights from HBM.
@@ -280,7 +281,7 @@ def module_time_us(lins, x, reps=256, out=None):
     return (time.perf_counter() - t0) / reps * 1e6
 
 
-def dense_fp16_time_us(M, N, K, total_bytes=COLD_BYTES):
+def dense_fp16_time_us(M, N, K, total_bytes=COLD_BYTES, reps=None):
     """The vendor library's dense fp16 GEMM of the same shape (torch.matmul on hipBLASLt / rocBLAS), cold
     weights: the comparison the reference's own evaluation makes against cuBLAS
     (qfactory/testing.py:36-41).  A reported yardstick, not part of the path."""
@@ -291,7 +292,7 @@ def dense_fp16_time_us(M, N, K, total_bytes=COLD_BYTES):
     for w in ws:
         torch.matmul(x, w.T)
     torch.cuda.synchronize()
-    reps = max(32, 2 * n)
+    reps = reps or max(32, 2 * n)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(reps):
@@ -301,23 +302,25 @@ def dense_fp16_time_us(M, N, K, total_bytes=COLD_BYTES):
     return e0.elapsed_time(e1) * 1e3 / reps
 
 
-def gemm_report(M=256):
+def gemm_report(M=256, shapes=None, reps=None):
     """BASELINE.json configs[3]: W4A16 g128 GEMM on Llama-3-70B-style shapes, per shape microseconds, TFLOP/s,
-    the fraction of the dense fp16 MFMA peak and of the HBM peak (M <= 64 is HBM-bound by arithmetic intensity)."""
+    the fraction of the dense fp16 MFMA peak and of the HBM peak (M <= 64 is HBM-bound by arithmetic intensity).
+    With ``shapes`` / ``reps``: the same report on other layers (the prefill section: launches of a millisecond
+    need no 64 per graph to reach the sustained clock)."""
     import torch
     from qfactory import QLinear
     flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
     g = torch.Generator(device="cuda").manual_seed(1)
     report = []
-    for name, N, K in GEMM_SHAPES:
+    for name, N, K in (shapes or GEMM_SHAPES):
         lin = QLinear.empty(M, K, N, NBITS, GS, sym=False, compile_flags=flags)
         sets = weight_sets(lin, cold_copies(N * K // 2), g)
         x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
-        us = kernel_event_time_us(lin.func, sets, x, N)
+        us = kernel_event_time_us(lin.func, sets, x, N, reps=reps)
         description = lin.func.runtime.description
         del lin, sets
         torch.cuda.empty_cache()
-        dense_us = dense_fp16_time_us(M, N, K)
+        dense_us = dense_fp16_time_us(M, N, K, reps=reps)
         flops = 2.0 * M * N * K
         rec = {"name": name, "N": N, "K": K, "M": M, "us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1),
                "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
@@ -590,6 +593,8 @@ def main():
         result["gemm_m256"] = {"peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS, "dense_fp16_TFLOP/s_measured": round(dense_tflops, 1),
                                "shapes": gemm_report(256)}
         result["gemm_m32_m64_m128"] = [rec for m_rows in (32, 64, 128) for rec in gemm_report(m_rows)]
+        # configs[4]'s prefill: 64 sequences x 128 prompt tokens through the Llama-2-7B layers
+        result["gemm_prefill_m8192"] = gemm_report(8192, shapes=SHAPES, reps=16)
     if not args.no_small_m:
         result["small_m"] = small_m_report()
     if not args.no_decode:
