@@ -80,6 +80,10 @@ int qf_empty_launch(int64_t blocks, int64_t threads, void* stream);
  *   caches are (batch, heads, max_len, head_dim); rotation of pairs (2i, 2i+1) by the angles in row
  *   *pos of cos_table / sin_table (max_len, head_dim/2) fp32.  Writes nothing if *pos is outside
  *   [0, max_len).
+ * qf_rope_kv_store_rows: the same for `tokens` positions per sequence (prefill): qkv (batch * tokens, 3, heads,
+ *   head_dim), row b * tokens + t being token t of sequence b at position pos[t] (tokens device int64 values shared
+ *   by the sequences); q_out (batch, heads, tokens, head_dim) = rotate(q), k_cache[b][h][pos[t]] = rotate(k),
+ *   v_cache[b][h][pos[t]] = v.  head_dim a multiple of 8; a token whose position is outside [0, max_len) writes nothing.
  * qf_decode_attention: out (batch, heads*head_dim) = softmax(q k^T / sqrt(head_dim)) v over cache
  *   positions 0 .. *pos.  head_dim in {32, 64, 128, 256}.
  * qf_rope_decode_attention: the two above in one launch, straight from the QKV projection: rotates q and k
@@ -92,6 +96,9 @@ int qf_add_rmsnorm(uint16_t* x, const uint16_t* delta, const uint16_t* weight, u
 int qf_rope_kv_store(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
                      uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int64_t batch, int64_t heads,
                      int64_t head_dim, int64_t max_len, void* stream);
+int qf_rope_kv_store_rows(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
+                          uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int64_t batch, int64_t tokens,
+                          int64_t heads, int64_t head_dim, int64_t max_len, void* stream);
 int qf_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int64_t* pos,
                         uint16_t* out, int64_t batch, int64_t heads, int64_t head_dim, int64_t max_len, void* stream);
 int qf_rope_decode_attention(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,

@@ -160,6 +160,42 @@ __device__ __forceinline__ f16x8 rotate8(const f16x8 x, const float* __restrict_
     return r;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same rotation and cache write for `tokens` positions per sequence (prefill): qkv row b * tokens + t is
+// [3][H][hd] of token t of sequence b, pos[t] its position (shared by the sequences).  q goes out as
+// (batch, heads, tokens, hd) -- the layout an attention over (batch, heads, *, hd) caches takes --, k and v to cache
+// row pos[t].  One thread per eight elements; a token whose position is outside the cache writes nothing.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void rope_kv_store_rows_kernel(const f16* __restrict__ qkv, const int64_t* __restrict__ pos_ptr,
+                                                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                      f16* __restrict__ q_out, f16* __restrict__ k_cache,
+                                                                      f16* __restrict__ v_cache, int batch, int tokens, int heads, int hd,
+                                                                      int max_len) {
+    const int per_head = hd / 8;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= (int64_t)batch * tokens * heads * per_head) return;
+    const int j = (int)(idx % per_head);
+    const int h = (int)((idx / per_head) % heads);
+    const int64_t bt = idx / ((int64_t)per_head * heads);
+    const int t = (int)(bt % tokens), b = (int)(bt / tokens);
+    const int64_t pos = pos_ptr[t];
+    if (pos < 0 || pos >= max_len) return;
+    float c[4], s[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        c[i] = cos_t[pos * (hd / 2) + j * 4 + i];
+        s[i] = sin_t[pos * (hd / 2) + j * 4 + i];
+    }
+    const f16* row = qkv + (size_t)bt * 3 * heads * hd + (size_t)h * hd + j * 8;
+    const f16x8 q = rotate8(*reinterpret_cast<const f16x8*>(row), c, s);
+    const f16x8 k = rotate8(*reinterpret_cast<const f16x8*>(row + (size_t)heads * hd), c, s);
+    const f16x8 v = *reinterpret_cast<const f16x8*>(row + (size_t)2 * heads * hd);
+    *reinterpret_cast<f16x8*>(q_out + (((size_t)b * heads + h) * tokens + t) * hd + j * 8) = q;
+    const size_t cache_off = (((size_t)b * heads + h) * max_len + (size_t)pos) * hd + j * 8;
+    *reinterpret_cast<f16x8*>(k_cache + cache_off) = k;
+    *reinterpret_cast<f16x8*>(v_cache + cache_off) = v;
+}
+
 template <int LPK, bool FUSED, int THREADS>
 __global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __restrict__ q_or_qkv, f16* __restrict__ k_cache,
                                                                         f16* __restrict__ v_cache, const int64_t* __restrict__ pos_ptr,
@@ -344,6 +380,22 @@ extern "C" int qf_rope_kv_store(const uint16_t* qkv, const int64_t* pos, const f
                        (const f16*)qkv, pos, cos_table, sin_table, (f16*)q_out, (f16*)k_cache, (f16*)v_cache, (int)batch,
                        (int)heads, (int)head_dim, (int)max_len);
     return launched("qf_rope_kv_store");
+}
+
+extern "C" int qf_rope_kv_store_rows(const uint16_t* qkv, const int64_t* pos, const float* cos_table, const float* sin_table,
+                                     uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, int64_t batch, int64_t tokens,
+                                     int64_t heads, int64_t head_dim, int64_t max_len, void* stream) {
+    if (!qkv || !pos || !cos_table || !sin_table || !q_out || !k_cache || !v_cache) return fail("qf_rope_kv_store_rows", "null pointer");
+    if (batch <= 0 || tokens <= 0 || heads <= 0 || head_dim <= 0 || head_dim % 8 != 0 || max_len <= 0)
+        return fail("qf_rope_kv_store_rows", "batch, tokens, heads, max_len positive and head_dim a multiple of 8");
+    if (tokens > 0x7fffffff || heads > 0x7fffffff || head_dim > 0x7fffffff || max_len > 0x7fffffff || batch > 0x7fffffff)
+        return fail("qf_rope_kv_store_rows", "dimension too large");
+    const int64_t units = batch * tokens * heads * (head_dim / 8);
+    if (units > (int64_t)0x7fffffff * kThreads) return fail("qf_rope_kv_store_rows", "problem too large");
+    hipLaunchKernelGGL(rope_kv_store_rows_kernel, dim3((unsigned)((units + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                       (hipStream_t)stream, (const f16*)qkv, pos, cos_table, sin_table, (f16*)q_out, (f16*)k_cache, (f16*)v_cache,
+                       (int)batch, (int)tokens, (int)heads, (int)head_dim, (int)max_len);
+    return launched("qf_rope_kv_store_rows");
 }
 
 extern "C" int qf_decode_attention(const uint16_t* q, const uint16_t* k_cache, const uint16_t* v_cache, const int64_t* pos,

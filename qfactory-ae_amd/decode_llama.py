@@ -138,7 +138,8 @@ class QuantLlama:
     def prefill(self, tokens, pos):
         """``forward`` with the RMSNorm as a single launch of libqfactory_hip.so (any number of rows), the residual
         adds in the o and down projections' epilogues and SiLU * up in the gate+up projection's (or launches of their
-        own where a kernel cannot); RoPE, the cache update and causal attention stay PyTorch ops."""
+        own where a kernel cannot), RoPE and the cache update of all positions as one launch; causal attention stays
+        a PyTorch op."""
         from qfactory import native
         shape = self.shape
         B, T = tokens.shape
@@ -149,12 +150,19 @@ class QuantLlama:
         act = None if own else torch.empty(B * T, shape.mlp, dtype=torch.float16, device="cuda")
         mask = (torch.arange(shape.max_len, device="cuda")[None, :] <= pos[:, None])[None, None]
         delta = None
+        q = torch.empty(B, H, T, hd, dtype=torch.float16, device="cuda") if own else None
+        pos = pos.contiguous()
         for li, layer in enumerate(self.layers):
             native.add_rmsnorm(x, delta, layer["norm1"], hdn, shape.eps)
-            qkv = self.linear(layer["qkv"], hdn).reshape(B, T, 3, H, hd).permute(2, 0, 3, 1, 4)
-            q, k, v = self._rope(qkv[0], pos), self._rope(qkv[1], pos), qkv[2]
-            self.k_cache[li].index_copy_(2, pos, k)
-            self.v_cache[li].index_copy_(2, pos, v)
+            qkv = self.linear(layer["qkv"], hdn)
+            if own:
+                # RoPE of q and k and the cache write of k and v for all T positions: one launch
+                native.rope_kv_store_rows(qkv, pos, self.cos, self.sin, q, self.k_cache[li], self.v_cache[li])
+            else:
+                qkv = qkv.reshape(B, T, 3, H, hd).permute(2, 0, 3, 1, 4)
+                q, k, v = self._rope(qkv[0], pos), self._rope(qkv[1], pos), qkv[2]
+                self.k_cache[li].index_copy_(2, pos, k)
+                self.v_cache[li].index_copy_(2, pos, v)
             att = F.scaled_dot_product_attention(q, self.k_cache[li], self.v_cache[li], attn_mask=mask)
             att = att.permute(0, 2, 1, 3).reshape(B * T, shape.hidden)
             if own:

@@ -34,6 +34,7 @@ SIGNATURES = {
     "qf_empty_launch": (_INT, [_I64, _I64, _P]),
     "qf_add_rmsnorm": (_INT, [_P, _P, _P, _P, _I64, _I64, _F, _P]),
     "qf_rope_kv_store": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
+    "qf_rope_kv_store_rows": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _P]),
     "qf_decode_attention": (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_rope_decode_attention": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_silu_mul": (_INT, [_P, _P, _I64, _I64, _P]),
@@ -167,6 +168,22 @@ def rope_kv_store(qkv, pos, cos, sin, q_out, k_cache, v_cache):
     assert sin.dtype == torch.float32 and sin.is_contiguous()
     _check(load().qf_rope_kv_store(_f16(qkv), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), _f16(q_out), _f16(k_cache),
                                    _f16(v_cache), B, H, hd, max_len, _stream()), "qf_rope_kv_store")
+    return q_out
+
+
+def rope_kv_store_rows(qkv, pos, cos, sin, q_out, k_cache, v_cache):
+    """qkv (B * T, 3*H*hd), row b * T + t being token t of sequence b at position pos[t] (pos: T int64 device values):
+    rotated q to q_out (B, H, T, hd), rotated k and v to rows pos[t] of the caches (B, H, max_len, hd)."""
+    import torch
+    B, H, max_len, hd = k_cache.shape
+    T = pos.numel()
+    assert qkv.shape == (B * T, 3 * H * hd) and q_out.shape == (B, H, T, hd) and v_cache.shape == k_cache.shape
+    assert qkv.is_contiguous() and q_out.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert pos.is_cuda and pos.dtype == torch.int64 and pos.is_contiguous()
+    assert cos.dtype == torch.float32 and cos.is_contiguous() and cos.shape == (max_len, hd // 2) and sin.shape == cos.shape
+    assert sin.dtype == torch.float32 and sin.is_contiguous()
+    _check(load().qf_rope_kv_store_rows(_f16(qkv), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), _f16(q_out), _f16(k_cache),
+                                        _f16(v_cache), B, T, H, hd, max_len, _stream()), "qf_rope_kv_store_rows")
     return q_out
 
 

@@ -120,6 +120,55 @@ def test_rope_cache_append_and_attention_match_torch(B, H, hd, max_len, pos):
     assert (att.float() - want_att).abs().max() <= 1e-2 * want_att.abs().max() + 2e-3
 
 
+def test_rope_and_cache_write_of_a_whole_prompt():
+    """``qf_rope_kv_store_rows`` (prefill): every token of every sequence gets the rotation and the cache rows the
+    one-position kernel gives it, bit for bit, and what the PyTorch ops of ``QuantLlama.forward`` give within the
+    rounding of the rotation; a token outside the cache writes nothing."""
+    from qfactory import native
+    B, T, H, hd, max_len = 3, 6, 4, 64, 16
+    g = torch.Generator(device="cuda").manual_seed(5)
+    qkv = torch.randn(B * T, 3 * H * hd, device="cuda", generator=g).to(torch.float16)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, device="cuda", dtype=torch.float32) / hd))
+    ang = torch.arange(max_len, device="cuda", dtype=torch.float32)[:, None] * inv[None, :]
+    cos, sin = ang.cos(), ang.sin()
+    pos = torch.tensor([3, 4, 5, 9, max_len, 0], device="cuda", dtype=torch.int64)      # one token outside the cache
+    k0 = torch.randn(B, H, max_len, hd, device="cuda", generator=g).to(torch.float16)
+    v0 = torch.randn(B, H, max_len, hd, device="cuda", generator=g).to(torch.float16)
+    k_cache, v_cache = k0.clone(), v0.clone()
+    q_out = torch.full((B, H, T, hd), 7.0, dtype=torch.float16, device="cuda")
+    native.rope_kv_store_rows(qkv, pos, cos, sin, q_out, k_cache, v_cache)
+    torch.cuda.synchronize()
+    # token by token through the one-position kernel
+    want_k, want_v = k0.clone(), v0.clone()
+    want_q = torch.full_like(q_out, 7.0)
+    rows = qkv.reshape(B, T, 3 * H * hd)
+    for t in range(T):
+        q1 = torch.empty(B, H * hd, dtype=torch.float16, device="cuda")
+        p = int(pos[t])
+        native.rope_kv_store(rows[:, t].contiguous(), pos[t:t + 1].clone(), cos, sin, q1, want_k, want_v)
+        if 0 <= p < max_len:
+            want_q[:, :, t] = q1.reshape(B, H, hd)
+    torch.cuda.synchronize()
+    assert torch.equal(q_out, want_q) and torch.equal(k_cache, want_k) and torch.equal(v_cache, want_v)
+    # and the PyTorch ops
+    valid = (pos >= 0) & (pos < max_len)
+    x = rows.reshape(B, T, 3, H, hd).permute(2, 0, 3, 1, 4).float()                      # (3, B, H, T, hd)
+    c, s_ = cos.index_select(0, pos.clamp(0, max_len - 1))[None, None], sin.index_select(0, pos.clamp(0, max_len - 1))[None, None]
+
+    def rope(xf):
+        x0, x1 = xf[..., 0::2], xf[..., 1::2]
+        return torch.stack((x0 * c - x1 * s_, x0 * s_ + x1 * c), dim=-1).flatten(-2).to(torch.float16)
+
+    tq, tk = rope(x[0]), rope(x[1])
+    assert (q_out[:, :, valid].float() - tq[:, :, valid].float()).abs().max() <= 4e-3
+    assert (k_cache[:, :, pos[valid]].float() - tk[:, :, valid].float()).abs().max() <= 4e-3
+    assert torch.equal(v_cache[:, :, pos[valid]], x[2][:, :, valid].to(torch.float16))
+    untouched = torch.ones(max_len, dtype=torch.bool, device="cuda")
+    untouched[pos[valid]] = False
+    assert torch.equal(k_cache[:, :, untouched], k0[:, :, untouched]) and torch.equal(v_cache[:, :, untouched], v0[:, :, untouched])
+    assert torch.equal(q_out[:, :, ~valid], torch.full_like(q_out[:, :, ~valid], 7.0))
+
+
 def test_rope_writes_nothing_for_a_position_outside_the_cache():
     from qfactory import native
     B, H, hd, max_len = 2, 4, 64, 16
