@@ -82,7 +82,7 @@ int qf_empty_launch(int64_t blocks, int64_t threads, void* stream);
  *   [0, max_len).
  * qf_rope_kv_store_rows: the same for `tokens` positions per sequence (prefill): qkv (batch * tokens, 3, heads,
  *   head_dim), row b * tokens + t being token t of sequence b at position pos[t] (tokens device int64 values shared
- *   by the sequences); q_out (batch, heads, tokens, head_dim) = rotate(q), k_cache[b][h][pos[t]] = rotate(k),
+ *   by the sequences); q_out (batch, tokens, heads, head_dim) = rotate(q), k_cache[b][h][pos[t]] = rotate(k),
  *   v_cache[b][h][pos[t]] = v.  head_dim a multiple of 8; a token whose position is outside [0, max_len) writes nothing.
  * qf_decode_attention: out (batch, heads*head_dim) = softmax(q k^T / sqrt(head_dim)) v over cache
  *   positions 0 .. *pos.  head_dim in {32, 64, 128, 256}.

@@ -162,9 +162,9 @@ __device__ __forceinline__ f16x8 rotate8(const f16x8 x, const float* __restrict_
 
 // ---------------------------------------------------------------------------------------------
 // The same rotation and cache write for `tokens` positions per sequence (prefill): qkv row b * tokens + t is
-// [3][H][hd] of token t of sequence b, pos[t] its position (shared by the sequences).  q goes out as
-// (batch, heads, tokens, hd) -- the layout an attention over (batch, heads, *, hd) caches takes --, k and v to cache
-// row pos[t].  One thread per eight elements; a token whose position is outside the cache writes nothing.
+// [3][H][hd] of token t of sequence b, pos[t] its position (shared by the sequences).  q goes out in the same row
+// order, (batch, tokens, heads, hd) -- an attention that takes (batch, heads, tokens, hd) gets the transposed view and
+// returns its output in row order too --, k and v to cache row pos[t].  One thread per eight elements; a token whose position is outside the cache writes nothing.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void rope_kv_store_rows_kernel(const f16* __restrict__ qkv, const int64_t* __restrict__ pos_ptr,
                                                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t,
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_rows_kernel(const f16*
     const f16x8 q = rotate8(*reinterpret_cast<const f16x8*>(row), c, s);
     const f16x8 k = rotate8(*reinterpret_cast<const f16x8*>(row + (size_t)heads * hd), c, s);
     const f16x8 v = *reinterpret_cast<const f16x8*>(row + (size_t)2 * heads * hd);
-    *reinterpret_cast<f16x8*>(q_out + (((size_t)b * heads + h) * tokens + t) * hd + j * 8) = q;
+    *reinterpret_cast<f16x8*>(q_out + ((size_t)bt * heads + h) * hd + j * 8) = q;
     const size_t cache_off = (((size_t)b * heads + h) * max_len + (size_t)pos) * hd + j * 8;
     *reinterpret_cast<f16x8*>(k_cache + cache_off) = k;
     *reinterpret_cast<f16x8*>(v_cache + cache_off) = v;

@@ -150,14 +150,15 @@ class QuantLlama:
         act = None if own else torch.empty(B * T, shape.mlp, dtype=torch.float16, device="cuda")
         mask = (torch.arange(shape.max_len, device="cuda")[None, :] <= pos[:, None])[None, None]
         delta = None
-        q = torch.empty(B, H, T, hd, dtype=torch.float16, device="cuda") if own else None
+        q_rows = torch.empty(B, T, H, hd, dtype=torch.float16, device="cuda") if own else None
         pos = pos.contiguous()
         for li, layer in enumerate(self.layers):
             native.add_rmsnorm(x, delta, layer["norm1"], hdn, shape.eps)
             qkv = self.linear(layer["qkv"], hdn)
             if own:
                 # RoPE of q and k and the cache write of k and v for all T positions: one launch
-                native.rope_kv_store_rows(qkv, pos, self.cos, self.sin, q, self.k_cache[li], self.v_cache[li])
+                native.rope_kv_store_rows(qkv, pos, self.cos, self.sin, q_rows, self.k_cache[li], self.v_cache[li])
+                q = q_rows.transpose(1, 2)                      # (B, H, T, hd) view: the attention output comes back in row order
             else:
                 qkv = qkv.reshape(B, T, 3, H, hd).permute(2, 0, 3, 1, 4)
                 q, k, v = self._rope(qkv[0], pos), self._rope(qkv[1], pos), qkv[2]

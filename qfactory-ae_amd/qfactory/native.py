@@ -173,11 +173,11 @@ def rope_kv_store(qkv, pos, cos, sin, q_out, k_cache, v_cache):
 
 def rope_kv_store_rows(qkv, pos, cos, sin, q_out, k_cache, v_cache):
     """qkv (B * T, 3*H*hd), row b * T + t being token t of sequence b at position pos[t] (pos: T int64 device values):
-    rotated q to q_out (B, H, T, hd), rotated k and v to rows pos[t] of the caches (B, H, max_len, hd)."""
+    rotated q to q_out (B, T, H, hd), rotated k and v to rows pos[t] of the caches (B, H, max_len, hd)."""
     import torch
     B, H, max_len, hd = k_cache.shape
     T = pos.numel()
-    assert qkv.shape == (B * T, 3 * H * hd) and q_out.shape == (B, H, T, hd) and v_cache.shape == k_cache.shape
+    assert qkv.shape == (B * T, 3 * H * hd) and q_out.shape == (B, T, H, hd) and v_cache.shape == k_cache.shape
     assert qkv.is_contiguous() and q_out.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
     assert pos.is_cuda and pos.dtype == torch.int64 and pos.is_contiguous()
     assert cos.dtype == torch.float32 and cos.is_contiguous() and cos.shape == (max_len, hd // 2) and sin.shape == cos.shape

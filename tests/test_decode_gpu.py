@@ -135,12 +135,13 @@ def test_rope_and_cache_write_of_a_whole_prompt():
     k0 = torch.randn(B, H, max_len, hd, device="cuda", generator=g).to(torch.float16)
     v0 = torch.randn(B, H, max_len, hd, device="cuda", generator=g).to(torch.float16)
     k_cache, v_cache = k0.clone(), v0.clone()
-    q_out = torch.full((B, H, T, hd), 7.0, dtype=torch.float16, device="cuda")
-    native.rope_kv_store_rows(qkv, pos, cos, sin, q_out, k_cache, v_cache)
+    q_rows = torch.full((B, T, H, hd), 7.0, dtype=torch.float16, device="cuda")
+    native.rope_kv_store_rows(qkv, pos, cos, sin, q_rows, k_cache, v_cache)
     torch.cuda.synchronize()
+    q_out = q_rows.transpose(1, 2)                                                        # (B, H, T, hd)
     # token by token through the one-position kernel
     want_k, want_v = k0.clone(), v0.clone()
-    want_q = torch.full_like(q_out, 7.0)
+    want_q = torch.full((B, H, T, hd), 7.0, dtype=torch.float16, device="cuda")
     rows = qkv.reshape(B, T, 3 * H * hd)
     for t in range(T):
         q1 = torch.empty(B, H * hd, dtype=torch.float16, device="cuda")
