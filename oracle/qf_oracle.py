@@ -265,11 +265,11 @@ def error_metrics(out, ref):
 # packed tensors, dequantise to fp16, matmul with fp32 accumulation on all host threads.
 # ----------------------------------------------------------------------------------------------
 
-def torch_cpu_forward(A, w, s, z, nbits, GS):
-    """A (M,K) fp16 CPU tensor; w/s/z packed CPU tensors -> (M,N) fp16 tensor."""
+def torch_cpu_dequant(w, s, z, nbits, GS):
+    """Packed CPU tensors -> (N,K) fp16 tensor fp16((q - Z) * s) (tests/acc_gptq.py:31-38 over the packed layout)."""
     import torch
-    K = A.shape[1]
     N = w.shape[0]
+    K = w.shape[1] * 8 // nbits
     assert nbits in (2, 4, 8)
     p32 = 32 // nbits
     words = w.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF      # (N, K/p32)
@@ -288,6 +288,14 @@ def torch_cpu_forward(A, w, s, z, nbits, GS):
         p8 = 8 // nbits
         zb = z.contiguous().view(torch.uint8).to(torch.int32)
         Z = torch.stack([(zb >> (nbits * i)) & mask for i in range(p8)], dim=-1).reshape(N, G)
-    dq = ((q - Z.repeat_interleave(GS, dim=1)).to(torch.float32)
-          * s.to(torch.float32).repeat_interleave(GS, dim=1)).to(torch.float16)
+    return ((q - Z.repeat_interleave(GS, dim=1)).to(torch.float32)
+            * s.to(torch.float32).repeat_interleave(GS, dim=1)).to(torch.float16)
+
+
+def torch_cpu_forward(A, w, s, z, nbits, GS):
+    """A (M,K) fp16 CPU tensor; w/s/z packed CPU tensors -> (M,N) fp16 tensor (tests/acc_gptq.py:52 with fp32
+    accumulation)."""
+    import torch
+    assert A.shape[1] == w.shape[1] * 8 // nbits
+    dq = torch_cpu_dequant(w, s, z, nbits, GS)
     return (A.to(torch.float32) @ dq.to(torch.float32).T).to(torch.float16)

@@ -81,6 +81,9 @@ private:
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "allocate-and-launch fast path of the quantized linear layers";
+#ifdef QF_FASTPATH_SOURCE_DIGEST
+    m.attr("source_digest") = QF_FASTPATH_SOURCE_DIGEST;      // md5 of this file at build time: load() refuses a stale build
+#endif
     py::class_<BoundLaunch>(m, "BoundLaunch")
         .def(py::init<std::uintptr_t, std::uintptr_t, std::uintptr_t, std::uintptr_t, bool, std::int64_t, std::int64_t,
                       at::ScalarType, int>(),

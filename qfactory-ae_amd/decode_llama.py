@@ -6,10 +6,11 @@ RoPE; random-initialised weights; batch in {1, 16, 64}; 128 random prompt ids, 1
 tokens.  It stands in for the reference's end-to-end runs through vLLM (reproduce/fig11,
 third_party/vllm-qfactory.patch), which need vLLM and model downloads.
 
-The four projections of a layer (fused QKV, O, fused gate+up, down) are QLinear modules; prefill
+The four projections of a layer (fused QKV, O, fused gate+up, down) and the output projection are QLinear modules; prefill
 (M = batch * prompt length) lands in the matrix-core regime and decode (M = batch) in the GEMV
 regimes through the layers' own row-count dispatch.  ``forward`` runs everything else (embedding,
-RMSNorm, RoPE, attention over a static KV cache, SiLU, the fp16 lm_head) in plain PyTorch; ``prefill``
+RMSNorm, RoPE, attention over a static KV cache, SiLU) in plain PyTorch; the output projection (vocab x hidden)
+is a QLinear like the layers' four; ``prefill``
 replaces its norm steps by single launches and forms the residual adds and SiLU * up in the projections' epilogues.  A decode step has no PyTorch op between the linears:
 up to 32 sequences a layer is five launches -- qkv with the RMSNorm in front of its dot products, RoPE + cache
 append + attention of the new position (libqfactory_hip.so), o adding its result to the residual stream, gate+up
@@ -72,7 +73,6 @@ class QuantLlama:
         gen = torch.Generator(device="cuda").manual_seed(seed)
         h, hd = shape.hidden, shape.hidden // shape.heads
         self.embed = (torch.randn(shape.vocab, h, device="cuda", generator=gen) * 0.5).to(torch.float16)
-        self.lm_head = (torch.randn(shape.vocab, h, device="cuda", generator=gen) / h ** 0.5).to(torch.float16)
         self.final_norm = torch.ones(h, dtype=torch.float16, device="cuda")
         self.layers = []
         for _ in range(shape.layers):
@@ -84,6 +84,8 @@ class QuantLlama:
                 "gate_up": _random_qlinear(batch, h, 2 * shape.mlp, shape, gen),
                 "down": _random_qlinear(batch, shape.mlp, h, shape, gen),
             })
+        # the output projection is a quantized linear like the others (configs[4]: every linear), 32000 x 4096
+        self.lm_head = _random_qlinear(batch, h, shape.vocab, shape, gen)
         self.k_cache = torch.zeros(shape.layers, batch, shape.heads, shape.max_len, hd, dtype=torch.float16, device="cuda")
         self.v_cache = torch.zeros_like(self.k_cache)
         inv = 1.0 / (shape.rope_theta ** (torch.arange(0, hd, 2, device="cuda", dtype=torch.float32) / hd))
@@ -133,7 +135,7 @@ class QuantLlama:
             act = F.silu(gu[:, : shape.mlp]) * gu[:, shape.mlp:]
             x = x + self.linear(layer["down"], act.contiguous()).reshape(B, T, shape.hidden)
         last = self._norm(x[:, -1], self.final_norm)
-        return last @ self.lm_head.T
+        return self.linear(self.lm_head, last.contiguous())
 
     def prefill(self, tokens, pos):
         """``forward`` with the RMSNorm as a single launch of libqfactory_hip.so (any number of rows), the residual
@@ -179,7 +181,7 @@ class QuantLlama:
             delta = self.linear(layer["down"], act)
         last = (x if delta is None else x + delta).reshape(B, T, shape.hidden)[:, -1].contiguous()
         native.add_rmsnorm(last, None, self.final_norm, last, shape.eps)
-        return last @ self.lm_head.T
+        return self.linear(self.lm_head, last)
 
     def decode_step(self, tok, pos):
         """tok (B, 1) int64, pos one-element int64 device tensor: logits (B, vocab) of the next token, like
@@ -201,8 +203,8 @@ class QuantLlama:
                 layer["o"].forward_accumulate(self._att, x)
                 act = layer["gate_up"].forward_add_rmsnorm(x, None, layer["norm2"], shape.eps, silu_mul=True)
                 layer["down"].forward_accumulate(act, x)
-            native.add_rmsnorm(x, None, self.final_norm, self._hdn, shape.eps)
-            return self._hdn @ self.lm_head.T
+            # the final norm runs in front of the output projection's dot products, like a layer's
+            return self.lm_head.forward_add_rmsnorm(x, None, self.final_norm, shape.eps)
         if self.linear is self._own_linear and first["o"].fuses_accumulate(rows) and first["down"].fuses_accumulate(rows):
             # seven launches per layer: the o and down projections add their result to the residual stream themselves
             # (the norms then only read it), SiLU(gate) * up is the gate+up projection's epilogue where it can be
@@ -214,7 +216,7 @@ class QuantLlama:
                 native.add_rmsnorm(x, None, layer["norm2"], self._hdn, shape.eps)
                 layer["down"].forward_accumulate(layer["gate_up"].forward_silu_mul(self._hdn), x)
             native.add_rmsnorm(x, None, self.final_norm, self._hdn, shape.eps)
-            return self._hdn @ self.lm_head.T
+            return self.lm_head(self._hdn)
         for li, layer in enumerate(self.layers):
             native.add_rmsnorm(x, delta, layer["norm1"], self._hdn, shape.eps)
             qkv = self.linear(layer["qkv"], self._hdn)
@@ -225,12 +227,12 @@ class QuantLlama:
             act = layer["gate_up"].forward_silu_mul(self._hdn)
             delta = self.linear(layer["down"], act)
         native.add_rmsnorm(x, delta, self.final_norm, self._hdn, shape.eps)
-        return self._hdn @ self.lm_head.T
+        return self.linear(self.lm_head, self._hdn)
 
 
 def linears_time_us(model, M, reps=8):
-    """Time of the quantized linears of one decode step at M rows: every layer's four kernels once,
-    back to back in a HIP graph (cold weights: the whole model is streamed), averaged over `reps`."""
+    """Time of the quantized linears of one decode step at M rows: every layer's four kernels and the output
+    projection once, back to back in a HIP graph (cold weights: the whole model is streamed), averaged over `reps`."""
     xs = {K: torch.randn(M, K, device="cuda").to(torch.float16) for K in (model.shape.hidden, model.shape.mlp)}
 
     def one_pass():
@@ -238,6 +240,7 @@ def linears_time_us(model, M, reps=8):
             for name in ("qkv", "o", "gate_up", "down"):
                 lin = layer[name]
                 lin(xs[lin.in_features])
+        model.lm_head(xs[model.lm_head.in_features])
 
     one_pass()
     torch.cuda.synchronize()

@@ -125,6 +125,9 @@ def large_parity_cases():
             + [_case(64, N, K) for N, K in LLAMA2_7B]              # the batch-64 decode linears
             + [_case(512, 10240, 8192), _case(1024, 12288, 4096), _case(700, 22016, 4096), _case(512, 22016, 4096), _case(1024, 10240, 8192)]
             + [_case(2048, 12288, 4096), _case(3000, 4096, 11008), _case(8192, 4096, 4096)]      # the 2048- and 4096-row buckets
+            # the decode loop's prefill at 64 sequences x 128 prompt tokens, and its output projection
+            + [_case(8192, 12288, 4096), _case(8192, 22016, 4096), _case(8192, 4096, 11008)]
+            + [_case(M, 32000, 4096) for M in (1, 16, 64)]
             # the large block tiles at the other bit widths, group sizes and with a partial last window
             + [_case(256, 16384, 4096, 2, 64), _case(256, 16384, 4096, 3, 128, True), _case(256, 16384, 4096, 8, 32),
                _case(512, 16384, 4224, 4, 64), _case(256, 57344, 2816, 2, 128, True), _case(1024, 16384, 4096, 3, 128, True)])
@@ -192,6 +195,10 @@ def decode_cases():
     plus the tiny model tests/test_decode_gpu.py runs."""
     cases = [_case(M, N, K) for N, K in LLAMA2_7B for M in (1, 16, 64, 128, 256, 512, 1024, 2048, 4096)]
     cases += [_case(M, N, K, 4, 64) for N, K in TINY_LLAMA for M in (2, 16)]
+    # the output projection (vocab x hidden): once per sequence in prefill and per decode step
+    cases += [_case(M, 32000, 4096) for M in (1, 16, 64)] + [_case(M, 1000, 256, 4, 64) for M in (2, 16)]
+    cases += [dict(_case(M, 32000, 4096), prologue="add_rmsnorm") for M in (1, 16)]
+    cases += [dict(_case(M, 1000, 256, 4, 64), prologue="add_rmsnorm") for M in (2, 16)]
     return cases + silu_mul_cases()
 
 

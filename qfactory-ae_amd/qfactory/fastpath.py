@@ -26,11 +26,19 @@ _module = None
 _tried = False
 
 
+def source_digest():
+    """md5 of csrc/qf_fastpath.cpp: what a built extension must carry to be used."""
+    import hashlib
+    with open(SOURCE, "rb") as f:
+        return hashlib.md5(f.read()).hexdigest()
+
+
 def build_command(out_path):
     import torch
     from torch.utils import cpp_extension
     cxx = os.environ.get("CXX", "g++")
     cmd = [cxx, "-O2", "-shared", "-fPIC", "-std=c++17", "-fvisibility=hidden", f"-DTORCH_EXTENSION_NAME={MODULE_NAME}",
+           f'-DQF_FASTPATH_SOURCE_DIGEST="{source_digest()}"',
            "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
            SOURCE, "-o", out_path]
     for path in cpp_extension.include_paths() + [sysconfig.get_paths()["include"]]:
@@ -42,13 +50,19 @@ def build_command(out_path):
 
 def build(force=False):
     """Compile csrc/qf_fastpath.cpp into csrc/_qf_fastpath.so (host compiler only)."""
-    if not force and os.path.exists(LIBRARY) and os.path.getmtime(LIBRARY) >= os.path.getmtime(SOURCE):
-        return LIBRARY
+    if not force and os.path.exists(LIBRARY):
+        with open(LIBRARY, "rb") as f:
+            if source_digest().encode() in f.read():       # built from this very source
+                return LIBRARY
     tmp = f"{LIBRARY}.tmp.{os.getpid()}"
     proc = subprocess.run(build_command(tmp), capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"building {SOURCE} failed:\n{proc.stderr}")
     os.replace(tmp, LIBRARY)
+    global _tried
+    with _lock:
+        if _module is None:
+            _tried = False              # a first (or repaired) build: the next load() looks again
     return LIBRARY
 
 
@@ -66,7 +80,12 @@ def load():
                     spec = importlib.util.spec_from_file_location(MODULE_NAME, LIBRARY)
                     module = importlib.util.module_from_spec(spec)
                     spec.loader.exec_module(module)
-                    _module = module
+                    # a build of another version of the source calls launch with another argument list: never use it
+                    if os.path.exists(SOURCE) and getattr(module, "source_digest", None) != source_digest():
+                        warnings.warn(f"{LIBRARY} was built from another version of {os.path.basename(SOURCE)}; rebuild it "
+                                      "with qfactory.fastpath.build(force=True).  forward() keeps its ctypes path.")
+                    else:
+                        _module = module
                 except ImportError as err:
                     warnings.warn(f"{LIBRARY} does not load against this torch ({err}); rebuild it with "
                                   "qfactory.fastpath.build(force=True).  forward() keeps its ctypes path.")

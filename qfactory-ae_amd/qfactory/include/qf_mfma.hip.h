@@ -24,6 +24,7 @@
 //   * WK > 1 splits K over waves of the same block; partial tiles are summed through LDS.
 #pragma once
 
+#include <atomic>
 #include <cstdio>
 #include "qf_dequant.hip.h"
 
@@ -249,15 +250,15 @@ int mfma_launch(const void* A, const void* W, void* Cout, const void* S, const v
         return 1;
     }
     if (m <= 0) return 0;
-    static bool attr_set = false;
-    if (!attr_set && C::LDS_BYTES > 64 * 1024) {
+    static std::atomic<bool> attr_set{false};        // launch is re-entrant: the attribute call is idempotent, the flag only saves repeats
+    if (C::LDS_BYTES > 64 * 1024 && !attr_set.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mfma_kernel<C>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES);
         if (e != hipSuccess) {
             fprintf(stderr, "qfactory mfma: cannot reserve %zu bytes of LDS: %s\n", C::LDS_BYTES, hipGetErrorString(e));
             return 2;
         }
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     dim3 grid(C::GRID_X, (m + C::BM - 1) / C::BM);
     hipLaunchKernelGGL(mfma_kernel<C>, grid, dim3(C::THREADS), C::LDS_BYTES, stream, (const uint16_t*)A,

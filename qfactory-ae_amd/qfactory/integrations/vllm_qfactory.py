@@ -92,8 +92,11 @@ class QFactoryLinearMethod(LinearMethodBase):
         qweight = PackedvLLMParameter(
             data=torch.empty(input_size_per_partition // cfg.pack_factor, output_size_per_partition, dtype=torch.int32),
             input_dim=0, output_dim=1, packed_dim=0, packed_factor=cfg.pack_factor, weight_loader=weight_loader)
+        # starts as the trivial map k // group_size: a checkpoint without a g_idx tensor (older exports with
+        # desc_act=False) then means "no reordering" instead of leaving uninitialised memory for the check below
         g_idx = RowvLLMParameter(
-            data=torch.empty(input_size_per_partition, dtype=torch.int32), input_dim=0, weight_loader=weight_loader)
+            data=(torch.arange(input_size_per_partition, dtype=torch.int32) // cfg.group_size),
+            input_dim=0, weight_loader=weight_loader)
         scales = GroupQuantScaleParameter(
             data=torch.empty(groups, output_size_per_partition, dtype=params_dtype),
             input_dim=0, output_dim=1, weight_loader=weight_loader)

@@ -128,7 +128,7 @@ def bf16_to_f16(src, out=None):
 
 
 def stream_read(src, sink):
-    assert sink.numel() * sink.element_size() >= 4096 * 4, "qf_stream_read writes one checksum word per block into 4096 words"
+    assert sink.numel() * sink.element_size() >= 4096 * 4, "qf_stream_read writes one word per block, index modulo 4096: the sink holds 4096 words"
     _check(load().qf_stream_read(src.data_ptr(), src.numel() * src.element_size(), sink.data_ptr(), _stream()), "qf_stream_read")
 
 
@@ -148,9 +148,13 @@ def _f16(t):
     return t.data_ptr()
 
 
+ADD_RMSNORM_MAX_HIDDEN = 16384          # qf_add_rmsnorm holds a row in one block's registers
+
+
 def add_rmsnorm(x, delta, weight, out, eps):
     """x (rows, hidden) fp16 += delta (or None) in place; out = RMSNorm(x) * weight."""
     rows, hidden = x.shape
+    assert hidden <= ADD_RMSNORM_MAX_HIDDEN, f"qf_add_rmsnorm takes rows of up to {ADD_RMSNORM_MAX_HIDDEN} elements"
     assert out.shape == x.shape and weight.shape == (hidden,) and (delta is None or delta.shape == x.shape)
     _check(load().qf_add_rmsnorm(_f16(x), None if delta is None else _f16(delta), _f16(weight), _f16(out), rows, hidden,
                                  float(eps), _stream()), "qf_add_rmsnorm")

@@ -71,7 +71,8 @@ class GPTQLinear(torch.nn.Module):
         self.batch_size = batch_size
 
         self._funcs = {}
-        self._launchers = {}            # (rows, dtype) -> launch(activation, output) bound to this layer's packed tensors
+        self._launchers = {}            # (row-count bucket, dtype) -> launch(activation, output) bound to this layer's packed tensors
+        self._last = (None, None, None)  # (rows, dtype, launcher) of the previous call: decode repeats one row count
         # the specialisation of the hint's row-count bucket: the one forward() looks up for that many rows
         self.func = self._compile(_m_bucket(batch_size), self.compile_flags)
         self._funcs[(_m_bucket(batch_size), torch.float16)] = self.func
@@ -79,6 +80,7 @@ class GPTQLinear(torch.nn.Module):
     def __setattr__(self, name, value):
         if name in ("w", "s", "z") and getattr(self, "_launchers", None):
             self._launchers.clear()     # bound launchers hold the addresses of the tensors they were made for
+            super().__setattr__("_last", (None, None, None))
         super().__setattr__(name, value)
 
     def _compile(self, m, compile_flags, dtype=torch.float16, epilogue="none", prologue="none"):
@@ -111,7 +113,11 @@ class GPTQLinear(torch.nn.Module):
         """``launch(x, out)`` for ``m`` rows of ``dtype``: the bucket's closure with this layer's packed tensors
         validated once and bound (the reference re-checks all five tensors on every call, matmul.py:124-144; the
         three that belong to the layer cannot change between calls)."""
-        launch = self._launchers[(m, dtype)] = self.func_for(m, dtype).bind(self.w, self.s, self.z)
+        key = (_m_bucket(m), dtype)      # one launcher per bucket: it takes the row count at call time
+        launch = self._launchers.get(key)
+        if launch is None:
+            launch = self._launchers[key] = self.func_for(m, dtype).bind(self.w, self.s, self.z)
+        self._last = (m, dtype, launch)
         return launch
 
     def forward(self, x: torch.Tensor, out: torch.Tensor = None):
@@ -121,9 +127,8 @@ class GPTQLinear(torch.nn.Module):
         m, dtype = x.shape[0], x.dtype
         launch = None
         if m > 0:
-            launch = self._launchers.get((m, dtype))
-            if launch is None:
-                launch = self._launcher(m, dtype)
+            last = self._last
+            launch = last[2] if (last[0] == m and last[1] is dtype) else self._launcher(m, dtype)
         if out is None:
             if launch is not None and launch.alloc is not None:
                 out = launch.alloc(x)                      # allocation and launch in one native call
@@ -201,6 +206,10 @@ class GPTQLinear(torch.nn.Module):
         from . import native
         m = x.shape[0]
         assert delta is None or x_out is not None, "with delta, the sum needs a buffer to go to"
+        # the same operand contract at every row count, whichever path serves it
+        if x_out is not None:
+            assert x_out.data_ptr() != x.data_ptr(), "x_out must not alias the residual stream it is computed from"
+            assert delta is None or x_out.data_ptr() != delta.data_ptr(), "x_out must not alias delta"
         if m == 0 or not self.fuses_add_rmsnorm(m, x.dtype, silu_mul):
             h = x
             if delta is not None:
@@ -208,8 +217,13 @@ class GPTQLinear(torch.nn.Module):
             elif x_out is not None:
                 x_out.copy_(x)
             a = torch.empty_like(x)
-            if m > 0:
+            if m > 0 and x.dtype == torch.float16 and x.shape[1] <= native.ADD_RMSNORM_MAX_HIDDEN:
                 native.add_rmsnorm(h, None, gamma, a, eps)
+            elif m > 0:
+                # rows longer than qf_add_rmsnorm takes, or bf16: the same expression (and roundings) in torch ops
+                h32 = h.to(torch.float32)
+                normed = (h32 * torch.rsqrt(h32.pow(2).mean(dim=1, keepdim=True) + eps)).to(x.dtype)
+                torch.mul(normed, gamma, out=a)
             return self.forward_silu_mul(a) if silu_mul else self.forward(a)
         key = (_m_bucket(m), x.dtype, "add_rmsnorm+silu_mul" if silu_mul else "add_rmsnorm")
         func = self._funcs.get(key)

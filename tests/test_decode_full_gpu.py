@@ -79,3 +79,35 @@ def test_full_size_decode_step_matches_the_torch_evaluation(llama, batch):
         torch.cuda.synchronize()
         assert torch.equal(out.float(), got[i + 1]), f"graph replay of step {i} differs from the eager step"
     assert int(pos) == PROMPT + STEPS
+
+
+def test_full_size_prompt_of_128_tokens_then_decode_at_batch_1(llama):
+    """configs[4] as written, at batch 1: 128 prompt tokens through ``prefill`` (the GEMM kernels at 128 rows, one
+    launch for RoPE and the cache rows), then greedy tokens through the fused decode step, which then attends to
+    129 and more cache positions -- against the PyTorch evaluation fed the same tokens."""
+    prompt_len, steps = 128, 3
+    print("[case] Llama-2-7B shape, batch 1, prompt 128", flush=True)
+    shape = llama.LlamaShape(max_len=prompt_len + 128)
+    model = llama.QuantLlama(shape, 1, seed=21)
+    g = torch.Generator(device="cuda").manual_seed(22)
+    prompt = torch.randint(0, shape.vocab, (1, prompt_len), device="cuda", generator=g)
+    positions = torch.arange(prompt_len, device="cuda")
+    want, tokens = [model.forward(prompt, positions)], []
+    for i in range(steps):
+        tokens.append(want[-1].argmax(-1, keepdim=True))
+        want.append(model.forward(tokens[-1], torch.tensor([prompt_len + i], device="cuda")))
+    want = torch.stack(want).float()
+    want_k, want_v = model.k_cache.clone(), model.v_cache.clone()
+    model.k_cache.zero_(), model.v_cache.zero_()
+    got = [model.prefill(prompt, positions)]
+    for i in range(steps):
+        got.append(model.decode_step(tokens[i], torch.tensor([prompt_len + i], device="cuda")).clone())
+    got = torch.stack(got).float()
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all() and got.shape == (steps + 1, 1, shape.vocab)
+    assert _relative(got, want) <= 3e-3
+    assert _relative(model.k_cache, want_k) <= 3e-3 and _relative(model.v_cache, want_v) <= 3e-3
+    bound = 4 * (got - want).abs().max().item()
+    a, b = got.argmax(-1), want.argmax(-1)
+    margin = want.gather(-1, b[..., None])[..., 0] - want.gather(-1, a[..., None])[..., 0]
+    assert bool(((a == b) | (margin <= bound)).all())

@@ -204,22 +204,32 @@ def test_decode_step_matches_the_torch_evaluation_of_the_same_model():
     model = decode_llama.QuantLlama(shape, batch=2, seed=5)
     prompt = torch.randint(0, shape.vocab, (2, 8), device="cuda", generator=_gen(6))
 
-    def run(step_fn):
+    def run(step_fn, tokens=None):
+        """Prompt, then four steps: greedy, or fed ``tokens`` (so that a near-tie in the logits of random weights
+        cannot send two evaluations down different sequences)."""
         model.k_cache.zero_(), model.v_cache.zero_()
-        logits = [model.forward(prompt, torch.arange(8, device="cuda"))]
+        logits, fed = [model.forward(prompt, torch.arange(8, device="cuda"))], []
         for i in range(4):
-            tok = logits[-1].argmax(-1, keepdim=True)
-            logits.append(step_fn(tok, torch.tensor([8 + i], device="cuda")).clone())
-        return torch.stack(logits).float(), model.k_cache.clone(), model.v_cache.clone()
+            fed.append(logits[-1].argmax(-1, keepdim=True) if tokens is None else tokens[i])
+            logits.append(step_fn(fed[-1], torch.tensor([8 + i], device="cuda")).clone())
+        return torch.stack(logits).float(), model.k_cache.clone(), model.v_cache.clone(), fed
 
-    want, want_k, want_v = run(model.forward)
-    got, got_k, got_v = run(model.decode_step)
+    def same_choice(a, b):
+        """Equal greedy choices, except where b's own margin between the two candidates is within the rounding
+        distance of the two evaluations."""
+        bound = 4 * (a - b).abs().max().item()
+        ia, ib = a.argmax(-1), b.argmax(-1)
+        margin = b.gather(-1, ib[..., None])[..., 0] - b.gather(-1, ia[..., None])[..., 0]
+        return bool(((ia == ib) | (margin <= bound)).all()) and int((ia != ib).sum()) <= 1
+
+    want, want_k, want_v, tokens = run(model.forward)
+    got, got_k, got_v, _ = run(model.decode_step, tokens)
     # prefill with the norm and SiLU steps as single launches: same logits as the PyTorch evaluation
     pre = model.prefill(prompt, torch.arange(8, device="cuda")).float()
     assert ((pre - want[0]).norm() / want[0].norm()).item() <= 3e-3 and torch.equal(pre.argmax(-1), want[0].argmax(-1))
     assert torch.isfinite(got).all()
     assert ((got - want).norm() / want.norm()).item() <= 3e-3
-    assert torch.equal(got.argmax(-1), want.argmax(-1))
+    assert same_choice(got, want)
     assert ((got_k.float() - want_k.float()).norm() / want_k.float().norm()).item() <= 3e-3
     assert ((got_v.float() - want_v.float()).norm() / want_v.float().norm()).item() <= 3e-3
     # two rows: the residual adds and norms ran inside the qkv and gate+up projections (five launches per layer);
@@ -227,6 +237,6 @@ def test_decode_step_matches_the_torch_evaluation_of_the_same_model():
     keys = [k for layer in model.layers for name in ("qkv", "gate_up") for k in layer[name]._funcs]
     assert (2, torch.float16, "add_rmsnorm") in keys and (2, torch.float16, "add_rmsnorm+silu_mul") in keys
     model.fuse_norm = False
-    apart, apart_k, _ = run(model.decode_step)
-    assert ((apart - got).norm() / got.norm()).item() <= 1e-3 and torch.equal(apart.argmax(-1), got.argmax(-1))
+    apart, apart_k, _, _ = run(model.decode_step, tokens)
+    assert ((apart - got).norm() / got.norm()).item() <= 1e-3 and same_choice(apart, got)
     assert ((apart_k.float() - got_k.float()).norm() / got_k.float().norm()).item() <= 1e-3

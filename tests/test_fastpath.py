@@ -51,6 +51,17 @@ def test_switch_turns_it_off(monkeypatch, ext):
     assert fastpath.load() is ext
 
 
+def test_an_extension_built_from_another_source_is_not_used(monkeypatch, ext):
+    """load() compares the digest the module carries with the source's: a stale build would call launch with
+    another argument list."""
+    assert ext.source_digest == fastpath.source_digest()
+    monkeypatch.setattr(fastpath, "_module", None)
+    monkeypatch.setattr(fastpath, "_tried", False)
+    monkeypatch.setattr(fastpath, "source_digest", lambda: "0" * 32)
+    with pytest.warns(UserWarning, match="another version"):
+        assert fastpath.load() is None
+
+
 FLAGS = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
 
 
@@ -83,11 +94,18 @@ def test_forward_gives_the_same_bits_through_either_host_path(ext, gs, sym):
         into = torch.full((m, n), 7.0, device="cuda", dtype=torch.float16)
         assert lin.forward(x, out=into) is into                      # the extension, caller's tensor
         if m:
-            launch = lin._launchers[(m, torch.float16)] if gs != -1 else lin._launchers[torch.float16]
+            from qfactory.qlinear import _m_bucket
+            launch = lin._launchers[(_m_bucket(m), torch.float16)] if gs != -1 else lin._launchers[torch.float16]
             assert launch.alloc is not None, "the extension is built but the layer did not bind it"
         got = lin(x)                                                 # the extension, new tensor
         assert got.shape == (m, n) and got.dtype == torch.float16 and got.device == x.device
         assert torch.equal(got, expect) and torch.equal(into, expect)
+    if gs != -1:
+        # one bound launcher per row-count bucket, however many distinct row counts arrive
+        assert len(lin._launchers) == 4
+        for m in (3, 4, 7, 9, 13):
+            lin(torch.randn(m, k, device="cuda").half())
+        assert len(lin._launchers) == 4
 
 
 @pytest.mark.gpu

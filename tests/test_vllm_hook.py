@@ -53,6 +53,9 @@ def test_create_weights_registers_gptq_tensors(plugin):
     assert layer.qzeros.shape == (8, 48) and layer.qzeros.dtype == torch.int32
     assert layer.scales.shape == (8, 384) and layer.scales.dtype == torch.float16
     assert layer.g_idx.shape == (1024,)
+    # a checkpoint that carries no g_idx tensor leaves this value: it must already say "no reordering"
+    from qfactory.integrations import gptq_format as gf
+    gf.check_trivial_g_idx(layer.g_idx.data, 128)
     assert layer.qweight.attrs["packed_dim"] == 0 and layer.qzeros.attrs["packed_dim"] == 1
     assert layer.qweight.attrs["packed_factor"] == 8 and layer.qweight.attrs["weight_loader"] is loader
 
@@ -113,7 +116,9 @@ def test_loaded_layer_matches_oracle(plugin, oracle, rows):
     layer.qweight.data.copy_(gf.pack_qweight(W, bits))
     layer.qzeros.data.copy_(gf.pack_qzeros(Z, bits))
     layer.scales.data.copy_(S)
-    layer.g_idx.data.copy_(torch.arange(K, dtype=torch.int32) // GS)
+    if rows == 1:
+        layer.g_idx.data.copy_(torch.arange(K, dtype=torch.int32) // GS)
+    # rows == 40: g_idx is never written, as with a checkpoint that has no such tensor
     method.process_weights_after_loading(layer)
     assert layer.qweight is None and layer.qzeros is None
     x = torch.randn(2, rows // 2 if rows > 1 else 1, K, generator=g).to(torch.float16)[: (2 if rows > 1 else 1)]
