@@ -45,6 +45,25 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Sum over the LPK (4, 8, 16 or 32) neighbouring lanes that share a key row, in every one of them: lane-exchange steps
+// inside a row of sixteen lanes are data-parallel moves (no trip through the LDS crossbar), only the step across
+// two rows of sixteen is a shuffle.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+template <int LPK>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(LPK == 4 || LPK == 8 || LPK == 16 || LPK == 32, "lanes per key row");
+    v += dpp_move<0xB1>(v);                                    // quad_perm [1,0,3,2]: lane ^ 1
+    v += dpp_move<0x4E>(v);                                    // quad_perm [2,3,0,1]: lane ^ 2
+    if constexpr (LPK >= 8) v += dpp_move<0x141>(v);           // row_half_mirror: the other quad of the eight
+    if constexpr (LPK >= 16) v += dpp_move<0x140>(v);          // row_mirror: the other eight of the sixteen
+    if constexpr (LPK >= 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
 // Sum (MAX = false) or maximum (MAX = true) over a block of WAVES waves; `slots` holds WAVES floats and
 // may be reused right after the call returns.
 template <bool MAX, int WAVES>
@@ -143,10 +162,16 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_kernel(const f16* __re
 // store them), k and v are appended to the cache, and the new position is served from LDS rather than
 // re-read from memory the block has just written.
 // ---------------------------------------------------------------------------------------------
-// Few (sequence, head) pairs: 16 waves per block shorten the walk over the cache; many: 4 waves per block
-// keep more blocks resident (measured with 32 heads: 16 waves are faster at batch 16, slower at batch 64).
-constexpr int kAttnThreadsFew = 1024, kAttnThreadsMany = 256;
+// Few (sequence, head) pairs: 8 waves per block and the first 8 positions of every group requested up front; many:
+// 4 waves per block keep more blocks resident.  Measured with 32 heads of 128 at 130 / 191 / 250 cache positions,
+// cold caches: 8 waves with the up-front requests 5.4 / 5.6 / 6.0 us at batch 1 and 10.5 / 12.5 / 14.9 at batch 16;
+// 16 waves walking the cache two positions at a time 5.6 / 6.2 / 6.8 and 11.5 / 14.2 / 16.7.  Every wave repeats the
+// rotation of q and the merge steps, so more waves cost vector issue on the few CUs that have a block; a launch
+// costs 4.0 us before it touches the cache (the position, then the new token's q / k / v, then the stores: three
+// dependent round trips behind a 1.7 us launch).
+constexpr int kAttnThreadsFew = 512, kAttnThreadsMany = 256;
 constexpr int kAttnManyBlocks = 1024;
+constexpr int kAttnPrefetch = 8;          // positions per group requested up front by the few-blocks variant (256 at 128-wide heads)
 
 __device__ __forceinline__ f16x8 rotate8(const f16x8 x, const float* __restrict__ c, const float* __restrict__ s) {
 #pragma clang fp contract(off)                                // same roundings as rope_kv_store_kernel
@@ -196,7 +221,12 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_rows_kernel(const f16*
     *reinterpret_cast<f16x8*>(v_cache + cache_off) = v;
 }
 
-template <int LPK, bool FUSED, int THREADS>
+// PRE: how many of a group's first positions are requested before anything else -- before the position itself is
+// known (rows are clamped to the cache; what lies past the sequence is fetched and never used) and before q has
+// been rotated -- so that the cache rows, the position and the new token's q / k / v travel together instead of one
+// after the other.  For the few-blocks variant only: with many blocks the rows past a short sequence would cost
+// real bandwidth.
+template <int LPK, bool FUSED, int THREADS, int PRE>
 __global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __restrict__ q_or_qkv, f16* __restrict__ k_cache,
                                                                         f16* __restrict__ v_cache, const int64_t* __restrict__ pos_ptr,
                                                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t,
@@ -207,35 +237,54 @@ __global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __
     __shared__ float part[WAVES * HD], part_m[WAVES], part_l[WAVES];
     __shared__ __attribute__((aligned(16))) f16 new_k[HD], new_v[HD];
     const int h = blockIdx.x, b = blockIdx.y;
-    const int64_t pos = pos_ptr[0];
-    if (pos < 0 || (FUSED && pos >= max_len)) return;          // uniform over the block; nothing is written
-    const int n = (int)(pos < max_len ? pos + 1 : max_len);    // keys 0 .. n-1
     const int g = threadIdx.x / LPK, j = threadIdx.x % LPK;
     const size_t head = ((size_t)b * heads + h);
     f16* kc = k_cache + head * max_len * HD;
     f16* vc = v_cache + head * max_len * HD;
+    const int64_t pos = pos_ptr[0];
+    if (pos < 0 || (FUSED && pos >= max_len)) return;          // uniform over the block; nothing is written
+    const int n = (int)(pos < max_len ? pos + 1 : max_len);    // keys 0 .. n-1
 
-    f16x8 qv;
+    // Everything the block needs from memory is requested here, in one go, before anything is computed: the new
+    // token's q / k / v and angles first (they come from L2 and are needed first), then the group's first PRE
+    // cache positions (rows past the sequence are clamped to its last row: one row per wave, never used).
+    f16x8 qraw, kraw, vraw;
+    float c[4], s[4];
     if constexpr (FUSED) {
         const f16* row = q_or_qkv + (size_t)b * 3 * heads * HD + (size_t)h * HD + j * 8;
-        float c[4], s[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             c[i] = cos_t[pos * (HD / 2) + j * 4 + i];
             s[i] = sin_t[pos * (HD / 2) + j * 4 + i];
         }
-        qv = rotate8(*reinterpret_cast<const f16x8*>(row), c, s);
+        qraw = *reinterpret_cast<const f16x8*>(row);
         if (g == 0) {
-            const f16x8 kr = rotate8(*reinterpret_cast<const f16x8*>(row + (size_t)heads * HD), c, s);
-            const f16x8 vv = *reinterpret_cast<const f16x8*>(row + (size_t)2 * heads * HD);
+            kraw = *reinterpret_cast<const f16x8*>(row + (size_t)heads * HD);
+            vraw = *reinterpret_cast<const f16x8*>(row + (size_t)2 * heads * HD);
+        }
+    } else {
+        qraw = *reinterpret_cast<const f16x8*>(q_or_qkv + head * HD + j * 8);
+    }
+    f16x8 kpre[PRE > 0 ? PRE : 1], vpre[PRE > 0 ? PRE : 1];
+#pragma unroll
+    for (int i = 0; i < PRE; i++) {
+        // a position past the sequence, and the new position itself (which the block is about to write and serves
+        // from LDS), fetch row 0 instead: a row that is being read anyway, and never the line that is being written
+        const int p = (g + i * GROUPS < (FUSED ? n - 1 : n)) ? g + i * GROUPS : 0;
+        kpre[i] = *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
+        vpre[i] = *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
+    }
+    f16x8 qv = qraw;
+    if constexpr (FUSED) {
+        qv = rotate8(qraw, c, s);
+        if (g == 0) {
+            const f16x8 kr = rotate8(kraw, c, s);
             *reinterpret_cast<f16x8*>(kc + (size_t)pos * HD + j * 8) = kr;
-            *reinterpret_cast<f16x8*>(vc + (size_t)pos * HD + j * 8) = vv;
+            *reinterpret_cast<f16x8*>(vc + (size_t)pos * HD + j * 8) = vraw;
             *reinterpret_cast<f16x8*>(new_k + j * 8) = kr;
-            *reinterpret_cast<f16x8*>(new_v + j * 8) = vv;
+            *reinterpret_cast<f16x8*>(new_v + j * 8) = vraw;
         }
         __syncthreads();
-    } else {
-        qv = *reinterpret_cast<const f16x8*>(q_or_qkv + head * HD + j * 8);
     }
     float qf[8];
 #pragma unroll
@@ -244,22 +293,55 @@ __global__ __launch_bounds__(THREADS) void decode_attention_kernel(const f16* __
     // one pass over the cache with a running maximum: key and value row of a position are requested together
     float m = -INFINITY, l = 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-    for (int p = g; p < n; p += GROUPS) {
-        const bool fresh = FUSED && p == (int)pos;
-        const f16x8 kv = fresh ? *reinterpret_cast<const f16x8*>(new_k + j * 8) : *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8);
-        const f16x8 vv = fresh ? *reinterpret_cast<const f16x8*>(new_v + j * 8) : *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8);
+    auto visit = [&](const f16x8 kv, const f16x8 vv) {
         float d = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) d += qf[e] * (float)kv[e];
-#pragma unroll
-        for (int o = LPK / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);      // stays inside the group: all its lanes are here
+        d = group_sum<LPK>(d);                                                  // stays inside the group: all its lanes are here
         const float m_new = fmaxf(m, d);
         const float keep = __expf(m - m_new), w = __expf(d - m_new);           // m = -inf the first time: keep = 0
         l = l * keep + w;
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] = acc[e] * keep + w * (float)vv[e];
         m = m_new;
+    };
+    if constexpr (PRE > 0) {
+        // the positions requested at the top, all at once: their scores are independent of each other, so the dot
+        // products and the lane exchanges of the PRE positions overlap, and one maximum serves them all (no
+        // rescaling chain from position to position)
+        float d[PRE];
+        f16x8 vsel[PRE];
+#pragma unroll
+        for (int i = 0; i < PRE; i++) {
+            const bool fresh = FUSED && g + i * GROUPS == (int)pos;             // the block has just written this row: serve it from LDS
+            const f16x8 kv = fresh ? *reinterpret_cast<const f16x8*>(new_k + j * 8) : kpre[i];
+            vsel[i] = fresh ? *reinterpret_cast<const f16x8*>(new_v + j * 8) : vpre[i];
+            d[i] = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) d[i] += qf[e] * (float)kv[e];
+        }
+#pragma unroll
+        for (int i = 0; i < PRE; i++) d[i] = group_sum<LPK>(d[i]);
+#pragma unroll
+        for (int i = 0; i < PRE; i++) {
+            if (g + i * GROUPS >= n) d[i] = -INFINITY;                          // past the sequence (row 0 was fetched instead)
+            m = fmaxf(m, d[i]);
+        }
+        if (m != -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < PRE; i++) {
+                const float w = __expf(d[i] - m);                               // 0 for a position past the sequence
+                l += w;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] += w * (float)vsel[i][e];
+            }
+        }
+    }
+#pragma unroll 2
+    for (int p = g + PRE * GROUPS; p < n; p += GROUPS) {
+        const bool fresh = FUSED && p == (int)pos;
+        visit(fresh ? *reinterpret_cast<const f16x8*>(new_k + j * 8) : *reinterpret_cast<const f16x8*>(kc + (size_t)p * HD + j * 8),
+              fresh ? *reinterpret_cast<const f16x8*>(new_v + j * 8) : *reinterpret_cast<const f16x8*>(vc + (size_t)p * HD + j * 8));
     }
     // merge the 64/LPK groups of a wave (lanes that differ in the bits above log2(LPK)) ...
 #pragma unroll
@@ -328,10 +410,10 @@ int launch_attention(const char* fn, const f16* q_or_qkv, f16* k, f16* v, const 
     const float scale = 1.0f / sqrtf((float)HD);
     const bool many = (int64_t)batch * heads >= kAttnManyBlocks;
     if (many)
-        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsMany>), dim3(heads, batch), dim3(kAttnThreadsMany), 0,
+        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsMany, 0>), dim3(heads, batch), dim3(kAttnThreadsMany), 0,
                            stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
     else
-        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsFew>), dim3(heads, batch), dim3(kAttnThreadsFew), 0,
+        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsFew, kAttnPrefetch>), dim3(heads, batch), dim3(kAttnThreadsFew), 0,
                            stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
     return launched(fn);
 }
