@@ -370,14 +370,39 @@ def counter_pass(layers, acts, reps=5):
     log(f"[bench] counter pass: {reps} launches of each kernel and of a {COPY_BYTES} byte stream copy")
 
 
-def _timed_problem(M, N, K, nbits, sym):
+def counter_pass_matrix(reps=3):
+    """The launches of the matrix-core kernels to put under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: the
+    A-stationary kernel (gate_up at M = 16), the streaming skinny kernel (down at M = 16), the GEMM kernel on the four
+    Llama-3-70B shapes at M = 256 and on the Llama-2-7B qkv and gate_up layers at 8192 rows, each `reps` times over
+    two weight copies, and the 64 MiB stream copy that scales the counters."""
+    import torch
+    from qfactory import native
+    src = torch.randint(-128, 128, (COPY_BYTES,), dtype=torch.int8, device="cuda")
+    dst = torch.empty_like(src)
+    problems = [(16, 22016, 4096), (16, 4096, 11008)] + [(256, N, K) for _, N, K in GEMM_SHAPES] + [(8192, 12288, 4096), (8192, 22016, 4096)]
+    for M, N, K in problems:
+        lin, sets, x = _timed_problem(M, N, K, NBITS, False, copies=2)
+        out = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        torch.cuda.synchronize()
+        for r in range(reps):
+            w, s_, z = sets[r % len(sets)]
+            assert lin.func(x, w, out, s_, z) == 0
+            native.stream_copy(dst, src)
+        torch.cuda.synchronize()
+        log(f"[bench] counter pass: {reps} launches of {lin.func.runtime.description}")
+        del lin, sets, x, out
+        torch.cuda.empty_cache()
+    assert torch.equal(dst, src)
+
+
+def _timed_problem(M, N, K, nbits, sym, copies=None):
     """One QLinear of the problem plus enough random packed-tensor sets to defeat the caches (>= 512 MB)."""
     import torch
     from qfactory import QLinear
     flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
     g = torch.Generator(device="cuda").manual_seed(2)
     lin = QLinear.empty(M, K, N, nbits, GS, sym=sym, compile_flags=flags)
-    sets = weight_sets(lin, cold_copies(N * K * nbits // 8), g)
+    sets = weight_sets(lin, copies or cold_copies(N * K * nbits // 8), g)
     x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
     return lin, sets, x
 
@@ -413,6 +438,110 @@ def small_m_report():
     for name, N, K in GEMM_SHAPES:
         one("70b-gemv", 1, N, K, NBITS, False)
     return report
+
+
+def shape_set_problems():
+    """The reference's bandwidth and speed-up experiments as (figure, M, N, K, bits, group size) problems:
+    fig 9 (reproduce/fig9/plot_bandwidth_size.py:12,32-33: `squares-pure`, M = 1, W4 with and without groups),
+    fig 10 (reproduce/fig10/plot_bandwidth_bits.py:28-30: `squares-pure`, M = 1, 8 / 4 / 2 bits g128),
+    fig 6 (reproduce/fig6/bench_kernels.py:24-30: `operator`, M = 1, 8 / 4 / 2 bits g128) and
+    table 3 (reproduce/tab3/bench_kernels.py:25-33: `operator`, W4 g128 at M = 1 / 2 / 4)."""
+    with open(os.path.join(ROOT, "tests", "golden", "nkg_shapes.json")) as f:
+        sets = json.load(f)
+    problems, seen = [], set()
+
+    def add(fig, M, N, K, bits, gs):
+        key = (M, N, K, bits, gs)
+        entry = next((p for p in problems if p["key"] == key), None)
+        if entry is None:
+            entry = {"key": key, "figures": [], "M": M, "N": N, "K": K, "bits": bits, "GS": gs}
+            problems.append(entry)
+        if fig not in entry["figures"]:
+            entry["figures"].append(fig)
+
+    for N, K, _ in sets["squares-pure"]:
+        add("fig9", 1, N, K, 4, 128)
+        add("fig9", 1, N, K, 4, -1)
+        for bits in (8, 4, 2):
+            add("fig10", 1, N, K, bits, 128)
+    for N, K, _ in sets["operator"]:
+        for bits in (8, 4, 2):
+            add("fig6", 1, N, K, bits, 128)
+        for M in (1, 2, 4):
+            add("tab3", M, N, K, 4, 128)
+    return problems
+
+
+def footprint(M, N, K, bits, gs):
+    """reproduce/fig9/plot_bandwidth_size.py:37-44 (`get_memory_footprint`); bits == 16: the dense fp16 GEMM."""
+    if bits == 16:
+        return (M * K + K * N + M * N) * 2
+    if gs == -1:
+        return (M * K + M * N) * 2 + K * N * bits / 8
+    return (M * K + M * N) * 2 + K * N * (bits / 8 + (2 + bits / 8) / gs)
+
+
+def shape_sets_report():
+    """Kernel time, achieved bandwidth by the reference's footprint formula and speed-up over the vendor's dense fp16
+    GEMM for every problem of `shape_set_problems`, cold weights, timed like every other section."""
+    import torch
+    from qfactory import QLinear
+    flags = {"enable_transform": False, "enable_schedule": False, "enable_lower": False}
+    g = torch.Generator(device="cuda").manual_seed(4)
+    rows, dense = [], {}
+    for prob in shape_set_problems():
+        M, N, K, bits, gs = prob["key"]
+        if (M, N, K) not in dense:
+            dense[(M, N, K)] = dense_fp16_time_us(M, N, K)
+            torch.cuda.empty_cache()
+        try:
+            lin = QLinear.empty(M, K, N, bits, gs, sym=False, compile_flags=flags)
+        except Exception as exc:                        # a shape a kernel family rejects is reported, not hidden
+            rows.append({**{k: prob[k] for k in ("figures", "M", "N", "K", "bits", "GS")}, "error": str(exc)[:200]})
+            log(f"[bench] shape sets: M={M} N={N} K={K} b={bits} GS={gs}: {exc}")
+            continue
+        x = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
+        if gs == -1:
+            n_copies = cold_copies(N * K * bits // 8)
+            ws = [torch.randint(-128, 128, lin.w.shape, dtype=torch.int8, device="cuda", generator=g) for _ in range(n_copies)]
+            func = lin.func_for(torch.float16)
+            us = kernel_event_time_us(lambda a, w, out, s, z=None: func(a, w, out), [(w, None, None) for w in ws], x, N)
+            del ws
+        else:
+            sets = weight_sets(lin, cold_copies(N * K * bits // 8), g)
+            us = kernel_event_time_us(lin.func, sets, x, N)
+            del sets
+        b = footprint(M, N, K, bits, gs)
+        d_us = dense[(M, N, K)]
+        rows.append({"figures": prob["figures"], "M": M, "N": N, "K": K, "bits": bits, "GS": gs, "us": round(us, 3),
+                     "GB/s": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4),
+                     "dense_fp16_us": round(d_us, 3), "dense_fp16_GB/s": round(footprint(M, N, K, 16, -1) / d_us / 1e3, 1),
+                     "speedup_over_dense_fp16": round(d_us / us, 3)})
+        log(f"[bench] shape sets {'/'.join(prob['figures']):12s} M={M} N={N:6d} K={K:6d} b={bits} GS={gs:4d} {us:9.2f} us "
+            f"{rows[-1]['GB/s']:8.1f} GB/s  dense fp16 {d_us:9.2f} us (x{rows[-1]['speedup_over_dense_fp16']:.2f})")
+        del lin
+        torch.cuda.empty_cache()
+
+    def geomean(values):
+        values = [v for v in values if v > 0]
+        prod = 1.0
+        for v in values:
+            prod *= v
+        return round(prod ** (1.0 / len(values)), 3) if values else None
+
+    ok = [r for r in rows if "us" in r]
+    summary = {
+        "what": "speed-up over the vendor's dense fp16 GEMM (geometric mean, as reproduce/tab3/bench_kernels.py:36-47 and "
+                "reproduce/fig6/bench_kernels.py:54-59 form it) and achieved bandwidth by the reference's footprint formula",
+        "tab3_geomean_speedup_by_M": {str(M): geomean([r["speedup_over_dense_fp16"] for r in ok if "tab3" in r["figures"] and r["M"] == M])
+                                      for M in (1, 2, 4)},
+        "fig6_geomean_speedup_by_bits": {str(b): geomean([r["speedup_over_dense_fp16"] for r in ok if "fig6" in r["figures"] and r["bits"] == b])
+                                         for b in (8, 4, 2)},
+        "fig9_GB/s_by_size": [{"N": r["N"], "K": r["K"], "GS": r["GS"], "GB/s": r["GB/s"]} for r in ok if "fig9" in r["figures"]],
+        "fig10_GB/s_by_bits": [{"N": r["N"], "bits": r["bits"], "GB/s": r["GB/s"]} for r in ok if "fig10" in r["figures"]],
+        "problems": len(rows), "rejected": len(rows) - len(ok),
+    }
+    return {"summary": summary, "rows": rows}
 
 
 def decode_report(batches=(1, 16, 64), prompt_len=128, new_tokens=128):
@@ -577,6 +706,12 @@ def main():
     ap.add_argument("--counter-pass", action="store_true",
                     help="only launch each of the four kernels (cold weights) and a 64 MiB stream copy a few times, "
                          "eagerly: the run to put under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
+    ap.add_argument("--counter-pass-matrix", action="store_true",
+                    help="the same for the matrix-core kernels: gate_up and down at M = 16, the four GEMMs at M = 256, qkv and "
+                         "gate_up at 8192 rows")
+    ap.add_argument("--shape-sets", action="store_true",
+                    help="only the reference's bandwidth tables: its `squares` and `operator` shape sets at M in {1, 2, 4}, "
+                         "8 / 4 / 2 bits, with and without groups; prints one JSON object, writes gpurun_out/shape_sets.json")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the path; this build runs on exactly one GPU (--gpus 1)")
@@ -586,6 +721,19 @@ def main():
     torch.cuda.set_device(0)
     if args.launch_floor:
         print(json.dumps({"launch_floor": launch_floor_report()}), flush=True)
+        return
+    if args.counter_pass_matrix:
+        counter_pass_matrix()
+        return
+    if args.shape_sets:
+        report = shape_sets_report()
+        try:
+            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+            with open(os.path.join(ROOT, "gpurun_out", "shape_sets.json"), "w") as f:
+                json.dump(report, f, indent=1)
+        except OSError as exc:
+            log(f"[bench] could not write the side file: {exc}")
+        print(json.dumps(report["summary"]), flush=True)
         return
     M = 1
     layers, acts = build_layers(args.layers, M)

@@ -177,6 +177,20 @@ def bench_cases():
     return cases
 
 
+def shape_set_cases():
+    """bench.py --shape-sets: the reference's bandwidth / speed-up experiments (its `squares-pure` and `operator`
+    shape sets; bench.shape_set_problems holds the definitions)."""
+    import json
+    with open(os.path.join(os.path.dirname(HERE), "tests", "golden", "nkg_shapes.json")) as f:
+        sets = json.load(f)
+    cases = []
+    for N, K, _ in sets["squares-pure"]:
+        cases += [_case(1, N, K, 4, -1)] + [_case(1, N, K, nbits, 128) for nbits in (8, 4, 2)]
+    for N, K, _ in sets["operator"]:
+        cases += [_case(1, N, K, nbits, 128) for nbits in (8, 4, 2)] + [_case(M, N, K, 4, 128) for M in (2, 4)]
+    return cases
+
+
 def smoke_cases():
     return [_case(1, 512, 1024, 4, 128), _case(1, 512, 1024, 4, -1)]
 
@@ -305,7 +319,7 @@ def drain_cases(base=None):
 
 def all_cases(with_drain=True):
     seen, out = set(), []
-    for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + smoke_cases() + misc_test_cases()
+    for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + shape_set_cases() + smoke_cases() + misc_test_cases()
               + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases() + accumulate_cases() + odd_wave_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:

@@ -41,7 +41,7 @@ CONFIG_ATTRIBUTES = ("regime", "parallel_strategy", "tiling_configs", "decode_st
 # names `QFunc.defines` may hold.  (The headers' QF_*_EXPERIMENT timing knobs give wrong results and refuse to
 # compile unless the translation unit itself asks for them; the generator cannot.)
 TUNING_DEFINES = ("QF_FUSED_AND_OR", "QF_SCHED_FENCE_MODE", "QF_WIDE_HOLDERS", "QF_GEMV_A_FIRST",
-                  "QF_GEMV_QUANT_DEDUP", "QF_GEMV_WAVES_PER_EU", "QF_MGEMV_SB", "QF_GEMM_FULL_DRAIN")
+                  "QF_GEMV_QUANT_DEDUP", "QF_GEMV_WAVES_PER_EU", "QF_MGEMV_SB", "QF_GEMM_FULL_DRAIN", "QF_GEMM_XCD_MAP")
 
 
 def apply_config(qfunc, entry):
@@ -245,6 +245,15 @@ class QMatmulQFunc(QFunc):
             # stage) 8.85 -> 8.26; two chunks per lane (K = 28672) lose 6 %, K = 11008 is level.
             defines.setdefault("QF_FUSED_AND_OR", 2)
             defines.setdefault("QF_GEMV_QUANT_DEDUP", 1)
+        if self.regime == "gemm":
+            # Block -> tile map that puts the row slabs of one column of tiles on one XCD (its L2 then serves the weights to
+            # all of them) instead of the columns of one slab: pays where a launch has a few slabs -- measured, FETCH_SIZE
+            # and time, plain against mapped: 22016 x 4096 at 2048 rows 562 -> 471 MB and 380 -> 357 us, 10240 x 8192 at 256
+            # rows (two slabs) 125 -> 80 MB and 65.2 -> 62.8 us -- and loses where there are many, because the blocks of
+            # an XCD then share no activation slab: 12288 x 4096 at 8192 rows 806 -> 3260 MB, 753 -> 791 us.
+            slabs = -(-p["M"] // t["BM"])
+            if 2 <= slabs <= 8 and -(-p["N"] // (32 * t["NT32"] * t["WN"])) >= 8:
+                defines.setdefault("QF_GEMM_XCD_MAP", 1)
         if self.act_dtype == torch.bfloat16:
             defines["QF_OUT_BF16"] = 1
             if self.converts_activations:

@@ -72,8 +72,9 @@
 #endif
 
 // 1: block -> tile map that keeps the slabs of one column of tiles together on one XCD (see the
-// kernel), 0: plain blockIdx order.  Measured no faster (358 vs 365 us on 57344 x 8192 at M = 256, slower
-// with two 32-row tiles per wave): the Infinity Cache already serves the second fetch.  Off.
+// kernel), 0: plain blockIdx order.  The generator switches it on for launches of two to eight slabs (fewer bytes
+// past L2 and 4 - 6 % faster there); with one slab there is nothing to share, with many the blocks of an XCD
+// share no activation slab any more and the launch fetches four times the bytes.
 #ifndef QF_GEMM_XCD_MAP
 #define QF_GEMM_XCD_MAP 0
 #endif
@@ -246,11 +247,19 @@ __global__ __launch_bounds__(C::T) void gemm_kernel(
     // FETCH_SIZE: 552 MB instead of 240 MB on the 57344 x 8192 layer at M = 256).
     const int linear = blockIdx.x + gridDim.x * blockIdx.y;
     int col = blockIdx.x, slab = blockIdx.y;
-    if (QF_GEMM_XCD_MAP && C::GRID_X % 8 == 0) {
+    if (QF_GEMM_XCD_MAP && C::GRID_X >= 8) {
         const int per_group = 8 * gridDim.y;                    // tiles of 8 columns
-        const int grp8 = linear / per_group, rem = linear % per_group;
-        col = grp8 * 8 + rem % 8;
-        slab = rem / 8;
+        const int full = C::GRID_X / 8 * per_group;             // ids of the whole groups of 8 columns
+        if (linear < full) {
+            const int grp8 = linear / per_group, rem = linear % per_group;
+            col = grp8 * 8 + rem % 8;
+            slab = rem / 8;
+        } else {                                                // the last, narrower group: plain order inside it
+            constexpr int LAST = C::GRID_X % 8 ? C::GRID_X % 8 : 8;
+            const int rem = linear - full;
+            col = C::GRID_X / 8 * 8 + rem % LAST;
+            slab = rem / LAST;
+        }
     }
     const int n_blk = col * C::BN;
     const int m_blk = slab * BM;
