@@ -141,7 +141,8 @@ def bf16_cases():
              _case(1, 4096, 4096, 4, -1), _case(3, 100, 256, 8, -1),                                   # plain integer weights
              _case(16, 4096, 4096), _case(12, 100, 2048, 3, 64), _case(16, 100, 4096, 2, 128),        # A-stationary
              _case(7, 1000, 2048, 8, 128),
-             _case(5, 100, 11008, 4, 128), _case(9, 64, 8192, 8, 128), _case(12, 48, 14336, 2, 256),  # streaming skinny
+             _case(5, 100, 11008, 4, 128), _case(9, 64, 8192, 8, 128), _case(12, 48, 14336, 2, 256),  # A-stationary, long rows split over blocks
+             _case(16, 4096, 11008), _case(5, 100, 8192, 4, 64),                                         # ... long rows split over blocks
              _case(33, 100, 512, 4, 128), _case(300, 256, 2048, 4, 128), _case(64, 80, 11008, 2, 128, True),   # GEMM
              _case(48, 64, 2816, 3, 64, True), _case(40, 72, 4160, 8, 32), _case(256, 4096, 4096),
              _case(40, 100, 256, 2, 64),                                                               # generic fallback
@@ -284,6 +285,27 @@ def accumulate_cases():
     return [dict(c, epilogue="accumulate") for c in cases]
 
 
+def unsplit_cases():
+    """Long rows at 3 .. 16 activation rows served WITHOUT the split of K over blocks (``ksplit=False``: the kernels a
+    layer with the norm prologue or the SwiGLU epilogue is built on, and the streaming kernel, which the split has
+    replaced as the default of these shapes): ragged M and N, a last wave with dead steps, group per lane / per
+    chunk / per step, 2, 4 and 8 bits."""
+    cases = [_case(5, 100, 11008, 4, 128), _case(3, 77, 11008, 4, 32), _case(7, 130, 11008, 4, 64, True),
+             _case(16, 272, 14336, 4, 256), _case(12, 48, 14336, 2, 256), _case(16, 64, 14336, 2, 512, True),
+             _case(9, 64, 8192, 8, 128), _case(4, 100, 8192, 8, 64), _case(11, 40, 11008, 8, 32, True),
+             _case(8, 8200, 11008, 4, 128), _case(16, 4096, 11008), _case(16, 8192, 8192), _case(4, 100, 8192, 4, 64)]
+    return [dict(c, ksplit=False) for c in cases]
+
+
+def split_cases():
+    """The A-stationary kernel with K split over blocks (tests/test_ksplit_gpu.py), beyond what the parity lists above
+    already send there: 2, 4, 8 and 16 blocks along K, a last block with fewer chunks, waves past a block's share,
+    fewer column tiles than blocks, many batches per block, every bit width (bf16: the long rows of ``bf16_cases``)."""
+    return [_case(16, 4096, 7168), _case(3, 48, 7168, 4, 64), _case(16, 16384, 16384), _case(7, 1000, 28672), _case(4, 8192, 29696),
+            _case(16, 100, 53248, 4, 128, True), _case(13, 57344, 8192), _case(16, 2048, 16384, 8, 128), _case(5, 77, 12288, 2, 128),
+            _case(16, 272, 12288, 3, 128, True), _case(16, 5120, 13824)]
+
+
 def odd_wave_cases():
     """GEMM tilings whose wave count along N does not divide the activation tile's 1 KB blocks (3, 5, 6, 7 waves: the
     waves past the last block fetch it again), pinned explicitly (tests/test_qlinear_gpu.py): ragged M and N, one and two
@@ -320,7 +342,8 @@ def drain_cases(base=None):
 def all_cases(with_drain=True):
     seen, out = set(), []
     for c in (parity_cases() + grid_cases() + reference_sweep_cases() + large_parity_cases() + bench_cases() + shape_set_cases() + smoke_cases() + misc_test_cases()
-              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases() + accumulate_cases() + odd_wave_cases()):
+              + decode_cases() + bf16_cases() + smem_quant_cases() + eager_cases() + norm_prologue_cases() + accumulate_cases() + odd_wave_cases()
+              + unsplit_cases() + split_cases()):
         key = tuple(sorted(c.items()))
         if key not in seen:
             seen.add(key)
@@ -347,6 +370,12 @@ def qfuncs_of(case):
                          dtype, torch.int8, case["GS"])
         op.init_qfuncs()
         qfuncs += op.qfuncs
+    if case.get("ksplit") is False:
+        from qfactory.core.qfunc import QMatmulQFunc
+        from qfactory.core.qtile import AsymQTile, QTile, SymQTile
+        tile = SymQTile if case["sym"] else AsymQTile
+        qfuncs = [QMatmulQFunc(QTile((_m_bucket(case["M"]), case["K"]), torch.float16, 16),
+                               tile((case["N"], case["K"]), torch.int8, case["NBITS"], (1, case["GS"])), "nt", ksplit=False)]
     if case.get("tiling"):
         qfuncs = [q.clone(tiling_configs=dict(case["tiling"])) for q in qfuncs]
     if case.get("smem_quant"):

@@ -132,7 +132,7 @@ class QMatmul:
         self.qfuncs = [QMatmulQFunc(
             QTile((self.m, self.k), self.dtype_a, 16),
             tile_b((self.n, self.k), self.dtype_b, self.nbits, (1, self.group_size)),
-            "nt", self.base_impl)]
+            "nt", self.base_impl, ksplit=self.input_prologue == "none" and self.output_epilogue != "silu_mul")]
         self.qfuncs[0].output_epilogue = self.output_epilogue
         self.qfuncs[0].input_prologue = self.input_prologue
         q = self.qfuncs[0]

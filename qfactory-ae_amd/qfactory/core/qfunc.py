@@ -97,8 +97,11 @@ class QMatmulQFunc(QFunc):
     Beyond the reference (fp16 only, matmul.py:36): a bf16 activation tile gives a bf16 output; scales
     stay fp16, the packed tensors are the same."""
 
-    def __init__(self, qtile_a, qtile_b, layout, base_impl=False):
+    def __init__(self, qtile_a, qtile_b, layout, base_impl=False, ksplit=True):
         self.qtile_a, self.qtile_b, self.layout = qtile_a, qtile_b, layout
+        # may long rows be split over several blocks that meet through device memory?  Not with the norm prologue or
+        # the SwiGLU epilogue: a block that sees part of K can neither normalise a row nor pair gate with up
+        self.ksplit = ksplit
         assert qtile_a.quant_method == "none", "Quantization method not supported for A"
         assert qtile_b.quant_method in ("sym", "asym"), "Quantization method of B must be 'sym' or 'asym'"
         assert layout == "nt", f"Layout {layout} is not supported"
@@ -106,7 +109,7 @@ class QMatmulQFunc(QFunc):
         gs = qtile_b.quant_granularity[1]
 
         # Template-based code generation: which kernel family and how it is tiled
-        self.regime = tiling.regime_for(m, k, qtile_b.nbits, gs, n)
+        self.regime = tiling.regime_for(m, k, qtile_b.nbits, gs, n, ksplit=ksplit)
         self.parallel_strategy = "row"          # teams sweep rows, K split over lanes and waves
         self.tiling_configs = self.default_tiling(self.regime)
         # Computation transformation (reference: qfunc.py:85-91): "deferred" applies scale and zero once per
@@ -152,7 +155,8 @@ class QMatmulQFunc(QFunc):
         if regime == "gemv":
             return tiling.gemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "mgemv":
-            return tiling.mgemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
+            split = tiling.mgemv_ksplit_tiling(p["M"], p["N"], p["K"], nbits, gs) if self.ksplit else None
+            return split or tiling.mgemv_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "skinny":
             return tiling.skinny_tiling(p["M"], p["N"], p["K"], nbits, gs)
         if regime == "gemm":
@@ -254,6 +258,8 @@ class QMatmulQFunc(QFunc):
             slabs = -(-p["M"] // t["BM"])
             if 2 <= slabs <= 8 and -(-p["N"] // (32 * t["NT32"] * t["WN"])) >= 8:
                 defines.setdefault("QF_GEMM_XCD_MAP", 1)
+        assert t.get("KS", 1) == 1 or (self.input_prologue == "none" and self.output_epilogue != "silu_mul"), \
+            "a block that sees part of K can neither normalise a row nor pair gate with up: build the object with ksplit=False"
         if self.act_dtype == torch.bfloat16:
             defines["QF_OUT_BF16"] = 1
             if self.converts_activations:

@@ -33,9 +33,11 @@ MGEMV_MIN_M = 3         # below: dot2 GEMV; [MGEMV_MIN_M, MGEMV_MAX_M]: A-statio
 MGEMV_MAX_M = 32
 
 
-def regime_for(M, K=None, nbits=None, group_size=None, N=None):
+def regime_for(M, K=None, nbits=None, group_size=None, N=None, ksplit=True):
     if M < MGEMV_MIN_M or not MFMA_AVAILABLE:
         return "gemv"
+    if ksplit and K is not None and mgemv_ksplit_tiling(M, N or 0, K, nbits, group_size) is not None:
+        return "mgemv"
     if K is not None and nbits == 3:
         # 3-bit has three kernels: the dot2 GEMV (any M, tiled over grid.y), the A-stationary kernel and the GEMM
         if M <= MGEMV_MAX_M and mgemv_tiling(M, 0, K, nbits, group_size) is not None:
@@ -387,11 +389,59 @@ def mgemv_tiling(M, N, K, nbits, group_size, max_waves=16, **pins):
     return cfg
 
 
+KSPLIT_MIN_K = 7168         # shortest rows the A-stationary kernel splits over several blocks
+KSPLIT_MAX_M = 16
+KSPLIT_WAVE_K = 256         # elements of K whose activations one wave keeps in registers
+KSPLIT_BITS = (2, 3, 4, 8)
+
+
+def mgemv_ksplit_tiling(M, N, K, nbits, group_size):
+    """The A-stationary kernel with K split over KS blocks (``KS`` in the tiling; include/qf_mgemv.hip.h), for long rows
+    and 3 .. 16 activation rows; None where it does not apply.
+
+    A block then holds the activations of K / KS elements only -- sixteen waves of 256 elements each, the form that
+    measured best at K = 4096 -- and the KS partial results meet through a scratch buffer in device memory.  Measured on
+    MI355X (4 bits, groups of 128, cold weights, us per launch at M = 4 / 16, the kernel that served the shape before
+    -> split): 8192 x 8192 14.4 / 14.6 -> 10.9 / 12.1; 16384 x 16384 57.4 / 78.0 -> 30.1 / 32.2; 4096 x 11008 10.4 /
+    12.7 -> 9.4 / 10.3; 5120 x 13824 20.4 / 26.1 -> 14.7 / 15.5; 8192 x 28672 55.6 / 44.9 -> 28.2 / 29.8; 57344 x 8192
+    53.8 / 57.3 -> 48.4 / 49.7; 4096 x 7168 8.2 / 9.4 -> 7.4 / 7.8.  Shorter rows lose (15360 x 5120 11.6 -> 13.2,
+    22016 x 4096 12.1 -> 15.5: one block per CU already holds all of K there, and the split only adds the meeting), and
+    so does M = 2 against the dot2 kernel (8192 x 8192 8.6 -> 10.5).  KS is the smallest power of two that leaves a
+    block at most 4096 elements: more blocks than needed measured 15 - 30 % slower, fewer and fatter waves 3 - 50 %.
+    8 bits, the streaming kernel -> split: 8192 x 8192 20.1 / 22.1 -> 16.7 / 18.1, 16384 x 16384 116 / 121 -> 52 / 53,
+    4096 x 11008 13.7 / 17.2 -> 13.8 / 15.0.  2 and 3 bits: only where the unsplit kernel cannot hold the activations
+    (4096 x 12288: 10.2 / 11.8 -> 10.1 / 10.4 at 2 bits, 23.2 / 23.5 -> 11.6 / 11.8 at 3; 16384 x 16384 at 2 bits 62 / 107
+    -> 38 / 38); at K = 8192 the unsplit kernel is 1 - 2 us ahead."""
+    if nbits not in KSPLIT_BITS or not (MGEMV_MIN_M <= M <= KSPLIT_MAX_M) or K < KSPLIT_MIN_K:
+        return None
+    if not mgemv_supported(K, nbits, group_size):
+        return None
+    if nbits in (2, 3) and mgemv_tiling(M, N, K, nbits, group_size) is not None:
+        return None
+    chunk = 4 * (128 // plane_bits(nbits))
+    if group_size % chunk and chunk % group_size:
+        return None
+    nchunk = K // chunk
+    ch = max(1, KSPLIT_WAVE_K // chunk)
+    ks = 2
+    while ks <= 16:
+        nb = -(-nchunk // ks)
+        wk = -(-nb // ch)
+        # (2 and 3 bits: the transposition buffers of sixteen waves do not fit the LDS; eight do)
+        if wk <= 16 and mgemv_regs(1, ch, 1, nbits) <= mgemv_reg_limit(wk) and mgemv_lds_bytes(1, wk, ch, nbits) <= 160 * 1024:
+            break
+        ks *= 2
+    if ks > 16 or (ks - 1) * nb >= nchunk or (wk - 1) * ch >= nb:
+        return None
+    return {"MT16": 1, "WK": wk, "CH": ch, "PB": NUM_CUS // ks, "PF": 1, "KS": ks}
+
+
 def mgemv_candidates(M, N, K, nbits, group_size):
+    split = mgemv_ksplit_tiling(M, N, K, nbits, group_size)
     base = mgemv_tiling(M, N, K, nbits, group_size)
     if base is None:
-        return []
-    seen, out = set(), []
+        return [split] if split else []
+    seen, out = set(), ([split] if split else [])
     nchunk = K // (4 * (128 // plane_bits(nbits)))
 
     def add(cfg):
@@ -416,7 +466,8 @@ def mgemv_candidates(M, N, K, nbits, group_size):
 def mgemv_cfg_string(problem, t, nt_b):
     b = lambda x: "true" if x else "false"
     return (f"qf::MGemvCfg<{problem['NBITS']}, {problem['GS']}, {b(problem['SYM'])}, {problem['N']}, {problem['K']}, "
-            f"{t['MT16']}, {t['WK']}, {t['CH']}, {t['PB']}, {t['PF']}, {b(nt_b)}>")
+            f"{t['MT16']}, {t['WK']}, {t['CH']}, {t['PB']}, {t['PF']}, {b(nt_b)}"
+            + (f", {t['KS']}>" if t.get("KS", 1) > 1 else ">"))
 
 
 # --------------------------------------------------------------------------------------------

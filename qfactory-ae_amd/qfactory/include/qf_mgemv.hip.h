@@ -19,10 +19,15 @@
 //     B (columns n), so a lane holds one n and needs one scale: acc += s * group_sum in fp32.
 //   * Each wave parks its partial 16x16 tiles in its own LDS slots; one barrier at the end of the
 //     block, then the partials of the WK waves are summed and every output is written once.
+//   * Long rows (KS > 1): K is also split over KS blocks, each holding the activations of its own K/KS only.  A block
+//     writes the fp32 sums of a batch of tiles to a scratch buffer in device memory and counts itself in; the block
+//     that arrives last adds the KS partial results in the fixed order 0 .. KS-1 (the result does not depend on who
+//     arrives when), stores the outputs and clears the counter for the next launch.
 #pragma once
 
 #include <atomic>
 #include <cstdio>
+#include <mutex>
 #include "qf_dequant.hip.h"
 
 // Tiles a block finishes between two reductions through LDS (a multiple of the ring depth PF).
@@ -76,7 +81,15 @@ __device__ __forceinline__ void mg_static_for(F&& f) {
     }
 }
 
-template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_>
+// Scratch memory of a launch that splits K over blocks: KS partial results per batch of tiles and one arrival counter
+// per batch.  The counters must be zero when a launch starts; every launch leaves them zero.  Launches that share
+// one buffer must not overlap in time.
+struct MGemvScratch {
+    float* partial = nullptr;
+    unsigned* arrived = nullptr;
+};
+
+template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_, int KS_ = 1>
 struct MGemvCfg {
     static constexpr int NBITS = NBITS_, GS = GS_, N = N_, K = K_;
     static constexpr bool SYM = SYM_, NT_B = NT_B_;
@@ -91,6 +104,8 @@ struct MGemvCfg {
     static constexpr int KSTEPS = EPL / 8;         // MFMA k-steps per chunk
     static constexpr int CHUNK = 4 * EPL;          // elements of K per chunk
     static constexpr int NCHUNK = K / CHUNK;
+    static constexpr int KS = KS_;                 // blocks splitting K (1: a block covers all of K)
+    static constexpr int NCHUNK_B = (NCHUNK + KS - 1) / KS;              // chunks of one block
     static constexpr int THREADS = 64 * WK;
     static constexpr int BM = 16 * MT16;
     static constexpr int NT = (N + 15) / 16;       // 16-row weight tiles
@@ -124,13 +139,18 @@ struct MGemvCfg {
     static constexpr int WBUF_A = 16 * (CHUNK * 2 + 16);
     static constexpr int WBUF = WBUF_W > WBUF_A ? WBUF_W : WBUF_A;    // per-wave transposition buffer
     static constexpr size_t LDS_BYTES = (size_t)WK * SB * MT16 * 1024 + (size_t)WK * WBUF;
+    // split K: fp32 sums of one block and batch, and what one row block (grid.y) of a launch needs
+    static constexpr int PART = SB * MT16 * 256;
+    static constexpr size_t SCRATCH_FLOATS = KS > 1 ? (size_t)GRID_X * NBATCH * KS * PART : 0;
+    static constexpr size_t SCRATCH_COUNTERS = KS > 1 ? (size_t)GRID_X : 0;
+    static constexpr size_t SCRATCH_BYTES = (SCRATCH_FLOATS * 4 + 255) / 256 * 256 + SCRATCH_COUNTERS * 4;   // partial sums, then the counters
 };
 
 template <class C>
 __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ Cout,
-    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total, NormArgs norm) {
-    constexpr int MT16 = C::MT16, WK = C::WK, CH = C::CH, SLOTS = C::SLOTS, PF = C::PF, SB = C::SB;
+    const uint16_t* __restrict__ S, const uint8_t* __restrict__ Zp, int m_total, NormArgs norm, MGemvScratch scratch) {
+    constexpr int MT16 = C::MT16, WK = C::WK, CH = C::CH, SLOTS = C::SLOTS, PF = C::PF, SB = C::SB, KS = C::KS;
     constexpr bool NORM = QF_MGEMV_NORM_PROLOGUE != 0;
     constexpr int EPL = C::EPL, KSTEPS = C::KSTEPS, CHUNK = C::CHUNK;
     constexpr int P8 = 8 / C::ZFB;                      // zero-point fields per byte
@@ -163,8 +183,10 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 
     // chunks [lo, lo + CH) are read by this wave; it owns [own_from, own_from + CH) (a clamped last
     // wave re-reads chunks of its neighbours with zeroed activations: every address stays in bounds)
-    const int own_from = wk * CH;
-    const int lo = min(own_from, C::NCHUNK - CH);
+    // With K split over KS blocks, block z covers chunks [z NCHUNK_B, own_end).
+    const int own_from = (KS > 1 ? (int)blockIdx.z * C::NCHUNK_B : 0) + wk * CH;
+    const int own_end = KS > 1 ? min(((int)blockIdx.z + 1) * C::NCHUNK_B, C::NCHUNK) : C::NCHUNK;
+    const int lo = max(min(own_from, C::NCHUNK - CH), 0);
     const int gw_lo = (lo * CHUNK) / C::GS;              // first group of the wave's K-slice
 
     // ---- coalesced loads: LPR consecutive lanes cover one row's K-slice (CH*64 bytes) ----
@@ -257,7 +279,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     float acc2 = 0.0f;
 #pragma unroll
                     for (int c = 0; c < CH; c++) {
-                        const bool own = (lo + c >= own_from) && (lo + c < own_from + CH);
+                        const bool own = (lo + c >= own_from) && (lo + c < min(own_from + CH, own_end));
                         const size_t eoff = (size_t)min(m, m_total - 1) * C::K + (size_t)(lo + c) * CHUNK + (lane % LPRA) * 8;
                         u32x4 v = raw[mt][c][i];
                         if (norm.delta != nullptr) {
@@ -324,7 +346,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         for (int mt = 0; mt < MT16; mt++) {
 #pragma unroll
             for (int c = 0; c < CH; c++) {
-                const bool own = (lo + c >= own_from) && (lo + c < own_from + CH);
+                const bool own = (lo + c >= own_from) && (lo + c < min(own_from + CH, own_end));
 #pragma unroll
                 for (int i = 0; i < LPC; i++) {
                     const int row = i * RPIA + lane / LPRA;
@@ -503,7 +525,22 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                 if (m < m_total) Cout[(size_t)m * (C::N / 2) + n] = silu_mul_f16(gate, up);
             }
         }
-        constexpr int OUTPUTS = C::SILU ? 0 : SB * MT16 * 256;
+        if constexpr (KS > 1) {
+            // ---- K split over blocks: the block's own sums of this batch go to the scratch buffer (device-scope
+            //      stores, nobody waits for them here); the blocks meet once, behind the last batch ----
+            static_assert(!C::SILU && !NORM, "a block that sees part of K cannot normalise the rows or pair the gate with the up tile");
+            const size_t unit = (size_t)blockIdx.y * C::GRID_X + team_id;
+            float* const mine = scratch.partial + ((unit * KS + blockIdx.z) * C::NBATCH + batch) * C::PART;
+            for (int o = tid; o < C::PART; o += 64 * WK) {
+                float total = 0.f;
+                const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
+                const float* base = redf + ((size_t)p * 64 + nl + 16 * (ml >> 2)) * 4 + (ml & 3);
+#pragma unroll
+                for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
+                __hip_atomic_store(mine + o, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        constexpr int OUTPUTS = (C::SILU || KS > 1) ? 0 : SB * MT16 * 256;
         for (int o = tid; o < OUTPUTS && !(QF_MGEMV_EXPERIMENT & 4); o += 64 * WK) {
             const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
             const int sb = p / MT16, mt = p % MT16;
@@ -526,11 +563,89 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
 #pragma unroll 1
         for (int batch = 0; batch < C::NBATCH; batch++) do_batch(batch);
     }
+
+    if constexpr (KS > 1) {
+        // ---- the KS blocks of a unit meet: each counts itself in once all its sums are out; the block that finds
+        //      the other KS - 1 already counted adds the KS partial results of every tile in the order of their K
+        //      ranges (the result does not depend on who arrives when) and stores the outputs.
+        // The sums are device-scope stores (written through to where every XCD sees them), read back by device-scope
+        // loads, and the counter is a device-scope atomic: no cache is written back or invalidated as a whole (a
+        // device-wide fence per thread measured 5 - 20 times the kernel's own time).  A thread's stores have been
+        // acknowledged when its memory counter reads zero; the barrier collects that from every thread before the
+        // block is counted. ----
+        const size_t unit = (size_t)blockIdx.y * C::GRID_X + team_id;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();                                       // ... and every read of the LDS slots is done
+        unsigned* const flag = reinterpret_cast<unsigned*>(smem);
+        if (tid == 0) *flag = __hip_atomic_fetch_add(scratch.arrived + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*flag != (unsigned)(KS - 1)) return;               // block-uniform
+        const float* const all = scratch.partial + unit * KS * C::NBATCH * C::PART;
+        for (int o = tid; o < C::NBATCH * C::PART; o += 64 * WK) {
+            const int batch = o / C::PART, ob = o % C::PART;
+            const int p = ob >> 8, ml = (ob >> 4) & 15, nl = ob & 15;
+            const int sb = p / MT16, mt = p % MT16;
+            const int slot = batch * SB + sb;
+            const int tile = unit_of(slot);
+            if (slot >= SLOTS || tile >= C::NT) continue;
+            float total = 0.f;
+#pragma unroll
+            for (int z = 0; z < KS; z++)
+                total += __hip_atomic_load(all + (size_t)z * C::NBATCH * C::PART + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int m = m0 + 16 * mt + ml;
+            const int n = tile * 16 + nl;
+            if (m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, total);
+        }
+        // nobody else touches this counter again in this launch: zero for the next one
+        if (tid == 0) __hip_atomic_store(scratch.arrived + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// Row blocks (grid.y) a split-K object's scratch buffer is sized for.
+constexpr int kMGemvScratchRowBlocks = 1;
+
+// A buffer of kMGemvScratchRowBlocks * SCRATCH_BYTES bytes, 256-byte aligned, as the kernel's two arrays: the
+// partial sums of every row block first, the counters behind them.
+template <class C>
+MGemvScratch mgemv_scratch_at(void* base) {
+    MGemvScratch s;
+    s.partial = static_cast<float*>(base);
+    s.arrived = reinterpret_cast<unsigned*>(static_cast<uint8_t*>(base)
+                                            + (C::SCRATCH_FLOATS * 4 * kMGemvScratchRowBlocks + 255) / 256 * 256);
+    return s;
+}
+
+// The scratch buffer of this specialisation on the current device, allocated and cleared at the first call there and
+// kept until the process ends (null with a message if that fails).  The first call must not happen under stream
+// capture; afterwards the function only looks the pointer up.
+template <class C>
+MGemvScratch mgemv_scratch() {
+    static std::mutex lock;
+    static void* per_device[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        fprintf(stderr, "qfactory mgemv: cannot tell the current device\n");
+        return MGemvScratch{};
+    }
+    std::lock_guard<std::mutex> guard(lock);
+    if (per_device[dev] == nullptr) {
+        void* p = nullptr;
+        const size_t bytes = C::SCRATCH_BYTES * kMGemvScratchRowBlocks;
+        hipError_t e = hipMalloc(&p, bytes);
+        if (e == hipSuccess) e = hipMemset(p, 0, bytes);
+        if (e != hipSuccess) {
+            fprintf(stderr, "qfactory mgemv: cannot set up %zu bytes of scratch memory: %s\n", bytes, hipGetErrorString(e));
+            return MGemvScratch{};
+        }
+        per_device[dev] = p;
+    }
+    return mgemv_scratch_at<C>(per_device[dev]);
 }
 
 template <class C>
 int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const void* Zp, int m, hipStream_t stream,
-                 NormArgs norm = NormArgs{}) {
+                 NormArgs norm = NormArgs{}, const MGemvScratch* given = nullptr) {
     const char* why = nullptr;
     if (C::NBITS != 2 && C::NBITS != 3 && C::NBITS != 4 && C::NBITS != 8) why = "NBITS must be 2, 3, 4 or 8 for this kernel";
     else if (C::K % C::CHUNK != 0) why = "K must be a multiple of 4*128 / (bits of the main plane)";
@@ -538,8 +653,8 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
     else if (C::GS % C::EPL != 0) why = "a lane's 16 bytes of fields must lie inside one group";
     else if (!C::SYM && (C::G % (8 / C::ZFB)) != 0) why = "K/GS must fill whole zero-point bytes";
     else if (C::CH > C::NCHUNK) why = "more chunks per wave than the row has";
-    else if (C::WK * C::CH < C::NCHUNK) why = "WK*CH must cover K";
-    else if ((C::WK - 1) * C::CH >= C::NCHUNK) why = "a wave would own no chunk";
+    else if (C::KS == 1 && C::WK * C::CH < C::NCHUNK) why = "WK*CH must cover K";
+    else if (C::KS == 1 && (C::WK - 1) * C::CH >= C::NCHUNK) why = "a wave would own no chunk";
     else if (C::THREADS > 1024) why = "block too large";
     else if (C::CH != 1 && C::CH != 2 && C::CH != 4 && C::CH != 8 && C::CH != 16) why = "CH must be 1, 2, 4, 8 or 16";
     else if (C::GS % C::CHUNK != 0 && C::CHUNK % C::GS != 0) why = "GS must divide the chunk or be a multiple of it";
@@ -551,11 +666,15 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
     else if (QF_OUT_ACCUMULATE && (QF_OUT_BF16 || QF_MGEMV_GATE_UP_SILU)) why = "adding to the output is fp16 only and not combined with the SwiGLU epilogue";
     else if (QF_MGEMV_NORM_PROLOGUE && norm.gamma == nullptr) why = "an object with the norm prologue is called through launch_norm (RMSNorm weight missing)";
     else if (!QF_MGEMV_NORM_PROLOGUE && norm.gamma != nullptr) why = "this object was compiled without the norm prologue";
+    else if (C::KS < 1 || C::KS > 16) why = "KS must be 1 .. 16";
+    else if (C::KS > 1 && (QF_MGEMV_NORM_PROLOGUE || QF_MGEMV_GATE_UP_SILU)) why = "K split over blocks: neither the norm prologue nor the SwiGLU epilogue";
+    else if (C::KS > 1 && C::WK * C::CH < C::NCHUNK_B) why = "WK*CH must cover a block's share of K";
+    else if (C::KS > 1 && (C::KS - 1) * C::NCHUNK_B >= C::NCHUNK) why = "a block would own no chunk";
     else if (QF_MGEMV_NORM_PROLOGUE && (norm.x_out == A || (norm.x_out != nullptr && norm.x_out == norm.delta))) why = "x_out must be a buffer of its own: other blocks still read x and delta";
     else if (QF_MGEMV_NORM_PROLOGUE && (size_t)C::WK * C::BM * 4 > (size_t)C::WK * C::SB * C::MT16 * 1024) why = "norm sums exceed the reduction space";
     if (why) {
-        fprintf(stderr, "qfactory mgemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT16=%d WK=%d CH=%d PB=%d PF=%d)\n",
-                why, C::NBITS, C::GS, C::N, C::K, C::MT16, C::WK, C::CH, C::PB, C::PF);
+        fprintf(stderr, "qfactory mgemv: invalid configuration: %s (NBITS=%d GS=%d N=%d K=%d MT16=%d WK=%d CH=%d PB=%d PF=%d KS=%d)\n",
+                why, C::NBITS, C::GS, C::N, C::K, C::MT16, C::WK, C::CH, C::PB, C::PF, C::KS);
         return 1;
     }
     if (m <= 0) return 0;
@@ -569,9 +688,19 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
         }
         attr_set.store(true, std::memory_order_release);
     }
-    dim3 grid(C::GRID_X, (m + C::BM - 1) / C::BM);
+    dim3 grid(C::GRID_X, (m + C::BM - 1) / C::BM, C::KS);
+    MGemvScratch scratch;
+    if constexpr (C::KS > 1) {
+        if ((int)grid.y > kMGemvScratchRowBlocks) {
+            fprintf(stderr, "qfactory mgemv: an object that splits K over blocks takes at most %d rows per launch (got %d)\n",
+                    kMGemvScratchRowBlocks * C::BM, m);
+            return 1;
+        }
+        scratch = given != nullptr ? *given : mgemv_scratch<C>();
+        if (scratch.partial == nullptr) return 2;
+    }
     hipLaunchKernelGGL(mgemv_kernel<C>, grid, dim3(C::THREADS), C::LDS_BYTES, stream, (const uint16_t*)A,
-                       (const uint8_t*)W, (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m, norm);
+                       (const uint8_t*)W, (uint16_t*)Cout, (const uint16_t*)S, (const uint8_t*)Zp, m, norm, scratch);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
         fprintf(stderr, "qfactory mgemv: launch failed: %s\n", hipGetErrorString(err));

@@ -151,7 +151,8 @@ class GPTQLinear(torch.nn.Module):
         bucket = _m_bucket(m)
         if dtype != torch.float16 or self.out_features % 2:
             return False
-        regime = tiling.regime_for(bucket, self.in_features, self.n_bits, self.group_size, self.out_features)
+        # (the kernel as it is built for an epilogue that pairs columns: long rows are not split over blocks)
+        regime = tiling.regime_for(bucket, self.in_features, self.n_bits, self.group_size, self.out_features, ksplit=False)
         if regime == "mgemv":
             return self.out_features % 32 == 0
         if regime == "gemm":
@@ -192,7 +193,8 @@ class GPTQLinear(torch.nn.Module):
         kernel serves (up to 32 rows, fp16)."""
         if dtype != torch.float16 or (silu_mul and not self.fuses_silu_mul(m, dtype)):
             return False
-        return tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features) in ("gemv", "mgemv")
+        return tiling.regime_for(_m_bucket(m), self.in_features, self.n_bits, self.group_size, self.out_features,
+                                 ksplit=False) in ("gemv", "mgemv")
 
     def forward_add_rmsnorm(self, x: torch.Tensor, delta, gamma: torch.Tensor, eps: float, x_out=None, silu_mul=False):
         """The step of a decoder layer that ends in this projection: ``h = x + delta`` (fp16 add; ``delta`` may be

@@ -91,12 +91,14 @@ def test_jit_object_with_the_norm_prologue_exports_launch_norm():
 def test_add_to_output_epilogue_is_a_header_switch_of_four_kernels():
     from qfactory.core.qfunc import QMatmulQFunc
     from qfactory.core.qtile import AsymQTile, QTile
-    for m, k, regime in ((1, 512, "gemv"), (16, 1024, "mgemv"), (16, 11008, "skinny"), (64, 512, "gemm")):
-        q = QMatmulQFunc(QTile((m, k), torch.float16, 16), AsymQTile((64, k), torch.int8, 4, (1, 128)), "nt")
+    for m, k, regime, split in ((1, 512, "gemv", True), (16, 1024, "mgemv", True), (16, 11008, "skinny", False),
+                                (16, 11008, "mgemv", True), (64, 512, "gemm", True)):
+        q = QMatmulQFunc(QTile((m, k), torch.float16, 16), AsymQTile((64, k), torch.int8, 4, (1, 128)), "nt", ksplit=split)
         assert q.regime == regime
         q.output_epilogue = "accumulate"
         src = q.emit()
         assert "#define QF_OUT_ACCUMULATE 1" in src and "epilogue=accumulate" in src
+        assert ("KS=" in src) == (k == 11008 and split)          # long rows split over blocks keep the epilogue
     bf = QMatmulQFunc(QTile((1, 512), torch.bfloat16, 16), AsymQTile((64, 512), torch.int8, 4, (1, 128)), "nt")
     bf.output_epilogue = "accumulate"
     with pytest.raises(AssertionError):
@@ -113,11 +115,14 @@ def test_swiglu_epilogue_is_a_header_switch_of_three_kernels():
         q.output_epilogue = "silu_mul"
         src = q.emit()
         assert f"#define {define} 1" in src and "epilogue=silu_mul" in src
-    skinny = QMatmulQFunc(QTile((16, 11008), torch.float16, 16), AsymQTile((64, 11008), torch.int8, 4, (1, 128)), "nt")
-    assert skinny.regime == "skinny"
-    skinny.output_epilogue = "silu_mul"
-    with pytest.raises(AssertionError):
-        skinny.emit()
+    # neither the streaming kernel nor the A-stationary kernel with its rows split over blocks pairs gate with up
+    for split in (False, True):
+        long_rows = QMatmulQFunc(QTile((16, 11008), torch.float16, 16), AsymQTile((64, 11008), torch.int8, 4, (1, 128)), "nt",
+                                 ksplit=split)
+        assert long_rows.regime == ("mgemv" if split else "skinny")
+        long_rows.output_epilogue = "silu_mul"
+        with pytest.raises(AssertionError):
+            long_rows.emit()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

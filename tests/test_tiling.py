@@ -30,13 +30,56 @@ def _id(c):
     (33, 2048, 3, 128, "gemm"),
 ])
 def test_regime_routing(M, K, nbits, gs, expected):
-    assert tiling.regime_for(M, K, nbits, gs) == expected
+    """The kernel families without the split of long rows over blocks (how a layer with the norm prologue or the
+    SwiGLU epilogue is built)."""
+    assert tiling.regime_for(M, K, nbits, gs, ksplit=False) == expected
+
+
+@pytest.mark.parametrize("M,K,nbits,gs,ks", [
+    (3, 7168, 4, 128, 2), (16, 8192, 4, 128, 2), (4, 11008, 4, 128, 4), (16, 14336, 4, 128, 4), (16, 16384, 4, 128, 4),
+    (16, 28672, 4, 128, 8), (8, 53248, 4, 128, 16), (16, 8192, 8, 128, 2), (16, 11008, 8, 128, 4),
+    (16, 12288, 2, 128, 4), (16, 12288, 3, 128, 4), (16, 8192, 4, 64, 2), (16, 8192, 4, 32, 2),
+    # not split: short rows, one or two activation rows, more than sixteen, 2 and 3 bits where the unsplit kernel holds K
+    (16, 4096, 4, 128, 1), (16, 5120, 4, 128, 1), (2, 8192, 4, 128, 1), (17, 8192, 4, 128, 1), (32, 11008, 4, 128, 1),
+    (16, 8192, 2, 128, 1), (16, 8192, 3, 128, 1),
+])
+def test_long_rows_are_split_over_blocks(M, K, nbits, gs, ks):
+    t = tiling.mgemv_ksplit_tiling(M, 4096, K, nbits, gs)
+    if ks == 1:
+        assert t is None
+        assert tiling.regime_for(M, K, nbits, gs, 4096) == tiling.regime_for(M, K, nbits, gs, 4096, ksplit=False)
+        return
+    assert tiling.regime_for(M, K, nbits, gs, 4096) == "mgemv"
+    chunk = 4 * (128 // tiling.plane_bits(nbits))
+    nchunk, nb = K // chunk, -(-(K // chunk) // ks)
+    assert t["KS"] == ks and t["PB"] * ks == tiling.NUM_CUS and t["MT16"] == 1
+    assert t["WK"] <= 16 and t["WK"] * t["CH"] >= nb and (t["WK"] - 1) * t["CH"] < nb      # the waves cover a block's share, none idle
+    assert (ks - 1) * nb < nchunk                                                            # every block owns part of K
+    assert tiling.mgemv_lds_bytes(1, t["WK"], t["CH"], nbits) <= 160 * 1024
+    assert tiling.mgemv_regs(1, t["CH"], t["PF"], nbits) <= tiling.mgemv_reg_limit(t["WK"])
+    assert f", {ks}>" in tiling.mgemv_cfg_string({"NBITS": nbits, "GS": gs, "SYM": False, "N": 4096, "K": K}, t, True)
+
+
+def test_split_rows_are_not_combined_with_the_norm_prologue_or_the_swiglu_epilogue():
+    import torch
+    from qfactory.core import QMatmul
+    plain = QMatmul(16, 4096, 8192, 4, False, torch.float16, torch.int8, 128)
+    plain.init_qfuncs()
+    assert plain.qfuncs[0].tiling_configs.get("KS", 1) == 2 and "KS=2" in plain.qfuncs[0].emit()
+    add = QMatmul(16, 4096, 8192, 4, False, torch.float16, torch.int8, 128, output_epilogue="accumulate")
+    add.init_qfuncs()
+    assert add.qfuncs[0].tiling_configs.get("KS", 1) == 2
+    for kw in ({"input_prologue": "add_rmsnorm"}, {"output_epilogue": "silu_mul"}):
+        op = QMatmul(16, 4096, 8192, 4, False, torch.float16, torch.int8, 128, **kw)
+        op.init_qfuncs()
+        q = op.qfuncs[0]
+        assert q.regime == "mgemv" and q.tiling_configs.get("KS", 1) == 1 and "KS=" not in q.emit()
 
 
 @pytest.mark.parametrize("case", _cases(), ids=_id)
 def test_default_tiling_respects_the_kernel_limits(case):
     M, N, K, nbits, gs = (case[k] for k in ("M", "N", "K", "NBITS", "GS"))
-    regime = tiling.regime_for(M, K, nbits, gs, N)
+    regime = tiling.regime_for(M, K, nbits, gs, N, ksplit=False)
     if regime == "mgemv":
         t = tiling.mgemv_tiling(M, N, K, nbits, gs)
         chunk = 4 * (128 // tiling.plane_bits(nbits))
@@ -69,9 +112,9 @@ def test_default_tiling_respects_the_kernel_limits(case):
 
 
 def test_skinny_takes_longer_rows_only_with_one_tile_per_block():
-    assert tiling.regime_for(16, 18944, 4, 128, 3584) == "skinny"       # 224 tiles of 16 columns: one per block
-    assert tiling.regime_for(16, 18944, 4, 128, 8192) == "gemm"
-    assert tiling.regime_for(16, 27648, 4, 128, 3584) == "gemm"
+    assert tiling.regime_for(16, 18944, 4, 128, 3584, ksplit=False) == "skinny"       # 224 tiles of 16 columns: one per block
+    assert tiling.regime_for(16, 18944, 4, 128, 8192, ksplit=False) == "gemm"
+    assert tiling.regime_for(16, 27648, 4, 128, 3584, ksplit=False) == "gemm"
 
 
 def test_two_bit_k4096_mgemv_fits_lds():
@@ -100,7 +143,8 @@ def test_emit_names_the_kernel_of_the_regime(regime, M, N, K, nbits):
     import torch
     from qfactory.core.qfunc import QMatmulQFunc
     from qfactory.core.qtile import QTile, AsymQTile
-    q = QMatmulQFunc(QTile((M, K), torch.float16, 16), AsymQTile((N, K), torch.int8, nbits, (1, 128)), "nt")
+    q = QMatmulQFunc(QTile((M, K), torch.float16, 16), AsymQTile((N, K), torch.int8, nbits, (1, 128)), "nt",
+                     ksplit=regime != "skinny")
     assert q.regime == regime
     code = q.emit()
     header = {"gemv": "qf_gemv.hip.h", "mgemv": "qf_mgemv.hip.h", "skinny": "qf_skinny.hip.h", "gemm": "qf_gemm.hip.h"}[regime]
@@ -121,12 +165,12 @@ def test_prefill_sizes_use_the_many_rows_model_only_for_several_rounds():
     assert tiling.gemm_tiling(512, 4096, 4096, 4, 128)["WK"] == 2
 
 
-def _qfunc(M, N, K, nbits, gs, sym=False):
+def _qfunc(M, N, K, nbits, gs, sym=False, ksplit=True):
     import torch
     from qfactory.core.qfunc import QMatmulQFunc
     from qfactory.core.qtile import QTile, AsymQTile, SymQTile
     tile = SymQTile if sym else AsymQTile
-    return QMatmulQFunc(QTile((M, K), torch.float16, 16), tile((N, K), torch.int8, nbits, (1, gs)), "nt")
+    return QMatmulQFunc(QTile((M, K), torch.float16, 16), tile((N, K), torch.int8, nbits, (1, gs)), "nt", ksplit=ksplit)
 
 
 @pytest.mark.parametrize("M,N,K,nbits,gs,regime,strategies", [
@@ -135,11 +179,16 @@ def _qfunc(M, N, K, nbits, gs, sym=False):
     (16, 384, 1024, 4, 64, "mgemv", ["eager"]),                  # a chunk of 128 fields spans two groups
     (9, 64, 8192, 8, 128, "skinny", ["deferred", "eager"]),
     (11, 40, 11008, 8, 32, "skinny", ["eager"]),
+    (9, 64, 8192, 8, 128, "mgemv-split", ["deferred", "eager"]),
+    (11, 40, 11008, 8, 32, "mgemv-split", ["eager"]),
     (64, 384, 1024, 4, 128, "gemm", ["eager"]),
 ])
 def test_transform_yields_the_decode_strategies_the_kernel_implements(M, N, K, nbits, gs, regime, strategies):
     """The reference's transform() yields an eager and a deferred candidate (qfactory/core/qfunc.py:85-91)."""
-    q = _qfunc(M, N, K, nbits, gs)
+    q = _qfunc(M, N, K, nbits, gs, ksplit=regime != "skinny")
+    if regime == "mgemv-split":
+        assert q.tiling_configs["KS"] > 1
+        regime = "mgemv"
     assert q.regime == regime and q.decode_strategy == strategies[0]
     variants = q.transform()
     assert [v.decode_strategy for v in variants] == strategies
