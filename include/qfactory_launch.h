@@ -67,6 +67,21 @@ typedef void (*qf_launch_grouped_norm_fn)(int m, void* activation, void* delta, 
                                           void* weight, void* output, void* scale, void* zero, void* stream,
                                           int* return_code);
 
+/*
+ * launch_m without any allocation.  No counterpart in the reference; for callers that cannot allocate device memory:
+ * code under HIP-graph capture from its first call on, tight serving loops, harnesses that forbid hipMalloc.
+ * Exported only by objects whose kernel uses scratch memory beyond its inputs and outputs -- the A-stationary kernel
+ * with long rows split over several blocks (qf_describe names "KS=<blocks>"), whose blocks exchange partial sums and
+ * arrival counters through device memory.  launch / launch_m of such an object allocate that memory (hipMalloc, once
+ * per device, at their first call there); launch_m_static uses a static device array of the object instead (at most
+ * 8 MiB, one copy per GPU, held until the process ends) and calls no allocating routine.  Same arguments, same
+ * result bits as launch_m.  At most 16 rows; an object whose scratch memory would exceed the array returns 1 with a
+ * message (call launch_m).  All calls on one GPU share the array: calls that overlap in time on one GPU race
+ * (calls enqueued on one stream do not overlap).  Every other object already allocates nothing in launch / launch_m.
+ */
+typedef void (*qf_launch_grouped_m_static_fn)(int m, void* activation, void* weight, void* output,
+                                              void* scale, void* zero, void* stream, int* return_code);
+
 /* Static string naming the specialisation ("regime=gemv M=1 N=4096 K=4096 NBITS=4 ..."). */
 typedef const char* (*qf_describe_fn)(void);
 
@@ -79,6 +94,11 @@ const char* qf_describe(void);
 #elif defined(QF_LAUNCH_PLAIN)
 void launch(int m, void* _activation, void* _weight, void* _output, void* _stream, QF_RC_ARG __return_code);
 const char* qf_describe(void);
+#endif
+
+#if defined(QF_LAUNCH_STATIC)
+void launch_m_static(int m, void* _activation, void* _weight, void* _output, void* _scale, void* _zero,
+                     void* _stream, QF_RC_ARG __return_code);
 #endif
 
 #if defined(QF_LAUNCH_NORM)

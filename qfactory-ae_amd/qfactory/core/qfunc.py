@@ -304,6 +304,8 @@ class QMatmulQFunc(QFunc):
         else:
             raise ValueError(f"unknown regime {self.regime}")
         norm_abi = "#define QF_LAUNCH_NORM 1\n" if self.input_prologue == "add_rmsnorm" else ""
+        if self.regime == "mgemv" and t.get("KS", 1) > 1:
+            norm_abi += "#define QF_LAUNCH_STATIC 1\n"
         code += f'#if __has_include("qfactory_launch.h")\n#define QF_LAUNCH_GROUPED 1\n{norm_abi}#include "qfactory_launch.h"\n#endif\n\n'
         code += f"using Cfg = {cfg};\nconstexpr int M = {p['M']};\n\n"
         args = "_activation, _weight, _output, _scale, _zero"
@@ -311,6 +313,37 @@ class QMatmulQFunc(QFunc):
         code += f"\t__return_code = {call}({args}, M, (hipStream_t)_stream);\n}}\n\n"
         code += self._signature("launch_m", leading_m=True)
         code += f"\t__return_code = {call}({args}, m, (hipStream_t)_stream);\n}}\n\n"
+        if self.regime == "mgemv" and t.get("KS", 1) > 1:
+            # An object that splits K over blocks uses scratch memory in device memory, which launch / launch_m allocate
+            # at their first call on a device.  For callers that cannot allocate (under HIP-graph capture from the first
+            # call on, in loops that forbid it): the same launch on a static device array of this object.
+            code += ("// ---- entry point that allocates nothing ----\n"
+                     "// Scratch memory of launch_m_static: one copy per GPU, held until the process ends, shared by every call on\n"
+                     "// that GPU (calls that overlap in time on one GPU race; calls on one stream do not overlap).  Zero at load;\n"
+                     "// every launch leaves its counters zero and overwrites the partial sums before it reads them.\n"
+                     "static __device__ __align__(256) unsigned char scratch[qf::mgemv_static_scratch_bytes<Cfg>()];\n\n"
+                     "static int qf_static_scratch(qf::MGemvScratch& out) {\n"
+                     "\tstatic std::mutex lock;\n\tstatic void* address[64] = {};       // per device: each GPU holds its own copy at its own address\n"
+                     "\tint dev = 0;\n"
+                     "\tif (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {\n"
+                     "\t\tfprintf(stderr, \"qfactory mgemv: cannot tell the current device\\n\");\n\t\treturn 2;\n\t}\n"
+                     "\tstd::lock_guard<std::mutex> guard(lock);\n"
+                     "\tif (address[dev] == nullptr) {\n"
+                     "\t\tvoid* ptr = nullptr;\n"
+                     "\t\thipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));\n"
+                     "\t\tif (e != hipSuccess || ptr == nullptr) {\n"
+                     "\t\t\tfprintf(stderr, \"qfactory mgemv: no address for the static scratch array: %s\\n\", hipGetErrorString(e));\n"
+                     "\t\t\treturn 2;\n\t\t}\n"
+                     "\t\taddress[dev] = ptr;\n\t}\n"
+                     "\tout = qf::mgemv_scratch_at<Cfg>(address[dev]);\n\treturn 0;\n}\n\n")
+            code += self._signature("launch_m_static", leading_m=True)
+            code += ("\tif (Cfg::SCRATCH_BYTES * qf::kMGemvScratchRowBlocks > qf::kMGemvStaticScratchMax) {\n"
+                     "\t\tfprintf(stderr, \"qfactory mgemv: this object needs %zu bytes of scratch memory, the static array holds at most %zu: call launch_m\\n\",\n"
+                     "\t\t        (size_t)(Cfg::SCRATCH_BYTES * qf::kMGemvScratchRowBlocks), (size_t)qf::kMGemvStaticScratchMax);\n"
+                     "\t\t__return_code = 1;\n\t\treturn;\n\t}\n"
+                     "\tqf::MGemvScratch where;\n"
+                     "\t__return_code = qf_static_scratch(where);\n"
+                     f"\tif (__return_code == 0) __return_code = {call}({args}, m, (hipStream_t)_stream, qf::NormArgs{{}}, &where);\n}}\n\n")
         if self.input_prologue == "add_rmsnorm":
             # the entry point of this object (launch / launch_m return 1: they carry no norm operands)
             code += ('extern "C" void launch_norm (\n\tint m,\n\tvoid* _activation,\n\tvoid* _delta,\n\tvoid* _gamma,\n'

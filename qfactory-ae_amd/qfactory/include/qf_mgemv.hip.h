@@ -616,6 +616,15 @@ MGemvScratch mgemv_scratch_at(void* base) {
     return s;
 }
 
+// Largest scratch buffer a specialisation keeps as a static device array for its entry point that allocates nothing
+// (the generated translation unit declares the array: every GPU the object runs on holds it until the process ends).
+constexpr size_t kMGemvStaticScratchMax = 8u << 20;
+template <class C>
+constexpr size_t mgemv_static_scratch_bytes() {
+    constexpr size_t need = C::SCRATCH_BYTES * kMGemvScratchRowBlocks;
+    return need <= kMGemvStaticScratchMax ? need : 256;           // an object past the limit keeps a token array and refuses the call
+}
+
 // The scratch buffer of this specialisation on the current device, allocated and cleared at the first call there and
 // kept until the process ends (null with a message if that fails).  The first call must not happen under stream
 // capture; afterwards the function only looks the pointer up.

@@ -66,6 +66,10 @@ class Runtime:
         if self._launch_m is not None:
             self._launch_m.restype = None
             self._launch_m.argtypes = [ctypes.c_int] + sig + [rc_type]
+        self._launch_m_static = getattr(self.lib, "launch_m_static", None)    # objects that use scratch memory: the same launch on a static array
+        if self._launch_m_static is not None:
+            self._launch_m_static.restype = None
+            self._launch_m_static.argtypes = [ctypes.c_int] + sig + [rc_type]
         self._launch_norm = getattr(self.lib, "launch_norm", None)      # objects with the residual-add + RMSNorm prologue
         if self._launch_norm is not None:
             self._launch_norm.restype = None
@@ -108,6 +112,15 @@ class Runtime:
         assert self._launch_m is not None, "this specialisation takes m through launch()"
         return_code = ctypes.c_int(0)
         self._launch_m(ctypes.c_int(m), *self._marshal(args), ctypes.byref(return_code))
+        return return_code.value
+
+    def run_m_static(self, m: int, *args) -> int:
+        """Call ``launch_m_static``: ``launch_m`` of an object that uses scratch memory, on the object's static device
+        array instead of memory allocated at the first call (nothing is allocated, by the call or by this wrapper's
+        marshalling of its arguments)."""
+        assert self._launch_m_static is not None, "this specialisation uses no scratch memory: launch_m allocates nothing"
+        return_code = ctypes.c_int(0)
+        self._launch_m_static(ctypes.c_int(m), *self._marshal(args), ctypes.byref(return_code))
         return return_code.value
 
     def run_raw(self, m, ptrs, stream_handle) -> int:

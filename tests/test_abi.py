@@ -88,6 +88,26 @@ def test_jit_object_with_the_norm_prologue_exports_launch_norm():
         wide.emit()
 
 
+def test_jit_object_that_uses_scratch_memory_exports_the_entry_point_that_allocates_nothing():
+    from qfactory.core.qfunc import QMatmulQFunc
+    from qfactory.core.qtile import AsymQTile, QTile
+    from qfactory.jit import jit
+    assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_STATIC") == ["launch_m_static"]
+    split = QMatmulQFunc(QTile((16, 8192), torch.float16, 16), AsymQTile((64, 8192), torch.int8, 4, (1, 128)), "nt")
+    assert split.tiling_configs["KS"] == 2
+    runtime = jit.compile(split)
+    lib = ctypes.CDLL(os.path.join(runtime.path, "kernel.so"))
+    for name in _declared_functions("qfactory_launch.h", "QF_LAUNCH_GROUPED") + ["launch_m_static"]:
+        assert hasattr(lib, name), f"{name} missing from {runtime.path}"
+    assert runtime._launch_m_static is not None and "KS=2" in runtime.description
+    src = open(os.path.join(runtime.path, "kernel.hip")).read()
+    assert "#define QF_LAUNCH_STATIC" in src and "static __device__ __align__(256) unsigned char scratch[" in src
+    assert "hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))" in src
+    # ... and only such an object: the others use no device memory of their own, their launch_m allocates nothing
+    plain = jit.compile(QMatmulQFunc(QTile((16, 512), torch.float16, 16), AsymQTile((64, 512), torch.int8, 4, (1, 128)), "nt"))
+    assert plain._launch_m_static is None and "scratch" not in open(os.path.join(plain.path, "kernel.hip")).read()
+
+
 def test_add_to_output_epilogue_is_a_header_switch_of_four_kernels():
     from qfactory.core.qfunc import QMatmulQFunc
     from qfactory.core.qtile import AsymQTile, QTile
