@@ -9,17 +9,23 @@ than the 256 MB Infinity Cache in total), so every step streams its weights from
 pass over a real model does.  All K timed steps are captured in one HIP graph (the launch-bound
 inner loop of a decode step) and replayed once between synchronisations.
 
-Printed JSON: `value` = algorithmic bytes moved per second over the timed region (the reference's
-own footprint formula, reproduce/fig9/plot_bandwidth_size.py:37-44); `roofline` = the dominant
-kernel (gate+up) against the 8 TB/s HBM peak, its duration measured here with HIP events on the
-launch stream, beside two ceilings measured in the same run (`roofline.empirical`: a pure streaming
-read of the same number of bytes, and a large dense fp16 GEMM of the vendor library);
-`cpu_baseline` = the torch CPU dequant+matmul port of the reference's test path on the same four
-shapes, on this machine's host cores.  Further sections, none of them part of `value`:
-`small_m` (configs[1] at M = 4 / 16, configs[2]: the bit-width sweep at N = K = 8192, and the
-Llama-3-70B shapes at M = 1), `gemm_m256` and `gemm_m32_m64_m128` (configs[3]), `gemm_prefill_m8192`
-(the Llama-2-7B layers at configs[4]'s prefill row count) and `decode` (configs[4]: the Llama-2-7B-shaped
-decode loop at batch 1 / 16 / 64).
+Output.  stdout carries ONE compact JSON line (under 4 kB, `compact_line`): the headline keys (`metric`, `value` =
+algorithmic bytes moved per second over the timed region by the reference's own footprint formula,
+reproduce/fig9/plot_bandwidth_size.py:37-44, `ms_per_step`, ...), `roofline` = the dominant kernel (gate+up)
+against the 8 TB/s HBM peak, its duration measured here with HIP events on the launch stream, beside two
+ceilings measured in the same run (`roofline.empirical`: a pure streaming read of the same number of bytes, and a
+large dense fp16 GEMM of the vendor library), `cpu_baseline` = the torch CPU port of the reference's test path on
+the same four shapes on this machine's host cores (dequant + matmul, and matmul alone), and one short row per
+shape of the further sections.  The full report -- every section below with every field -- goes to stderr and to
+the side file `bench_report.json` (`write_report`).  Further sections, none of them part of `value`: `small_m` (configs[1] at
+M = 4 / 16, configs[2]: the bit-width sweep at N = K = 8192, the Llama-3-70B shapes at M = 1 and 16),
+`gemm_m256` and `gemm_m32_m64_m128` (configs[3]), `gemm_prefill_m8192` (the Llama-2-7B layers at configs[4]'s
+prefill row count) and `decode` (configs[4]: the Llama-2-7B-shaped decode loop at batch 1 / 16 / 64).
+
+Other modes (each prints its own JSON and exits): `--counter-pass` and `--counter-pass-matrix` (a few eager
+launches of the GEMV kernels / of the matrix-core kernels beside a copy of known size, for `rocprofv3 --pmc`),
+`--shape-sets` (the reference's figure 6 / 9 / 10 and table 3 shape sets: achieved bandwidth and speed-up over the
+dense fp16 GEMM).
 
 Every per-kernel timing rotates over at least 512 MB of distinct packed weights (twice the 256 MB
 Infinity Cache), so each launch streams its weights from HBM.
@@ -372,14 +378,15 @@ def counter_pass(layers, acts, reps=5):
 
 def counter_pass_matrix(reps=3):
     """The launches of the matrix-core kernels to put under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: the
-    A-stationary kernel (gate_up at M = 16), the streaming skinny kernel (down at M = 16), the GEMM kernel on the four
-    Llama-3-70B shapes at M = 256 and on the Llama-2-7B qkv and gate_up layers at 8192 rows, each `reps` times over
-    two weight copies, and the 64 MiB stream copy that scales the counters."""
+    A-stationary kernel (gate_up at M = 16; down at M = 16 and the 8192 x 8192 projection at M = 16 with their rows
+    split over four and two blocks), the GEMM kernel on the four Llama-3-70B shapes at M = 256 and on the Llama-2-7B
+    qkv and gate_up layers at 8192 rows, each `reps` times over two weight copies, and the 64 MiB stream copy that
+    scales the counters."""
     import torch
     from qfactory import native
     src = torch.randint(-128, 128, (COPY_BYTES,), dtype=torch.int8, device="cuda")
     dst = torch.empty_like(src)
-    problems = [(16, 22016, 4096), (16, 4096, 11008)] + [(256, N, K) for _, N, K in GEMM_SHAPES] + [(8192, 12288, 4096), (8192, 22016, 4096)]
+    problems = [(16, 22016, 4096), (16, 4096, 11008), (16, 8192, 8192)] + [(256, N, K) for _, N, K in GEMM_SHAPES] + [(8192, 12288, 4096), (8192, 22016, 4096)]
     for M, N, K in problems:
         lin, sets, x = _timed_problem(M, N, K, NBITS, False, copies=2)
         out = torch.empty(M, N, dtype=torch.float16, device="cuda")
@@ -437,6 +444,8 @@ def small_m_report():
     # the 28672-wide end of the "4096 - 28672-wide LLM shapes" the GEMV target names: Llama-3-70B at M = 1
     for name, N, K in GEMM_SHAPES:
         one("70b-gemv", 1, N, K, NBITS, False)
+    for name, N, K in GEMM_SHAPES:                         # ... and at sixteen rows: K = 8192 and 28672 split over blocks
+        one("70b-m16", 16, N, K, NBITS, False)
     return report
 
 
