@@ -90,6 +90,10 @@ int qf_empty_launch(int64_t blocks, int64_t threads, void* stream);
  *   of position *pos, appends k and v to the caches and writes the attention output; nothing is written
  *   if *pos is outside [0, max_len).  Results equal qf_rope_kv_store followed by qf_decode_attention.
  * qf_silu_mul: out (rows, mlp) = fp16(silu(gate_up[:, :mlp])) * gate_up[:, mlp:]; mlp a multiple of 8.
+ * qf_greedy_next: the end of a greedy decode step in one launch: tok[b] = the smallest index of the largest of
+ *   logits[b][0 .. vocab) (NaN is never chosen; vocab a multiple of 8), *pos += 1 if pos is given, and, if embed
+ *   (vocab, hidden) is given, x_next[b] = embed[tok[b]] -- the residual stream the next step starts from (hidden a
+ *   multiple of 8).  No counterpart in the reference, whose end-to-end runs leave sampling to vLLM.
  */
 int qf_add_rmsnorm(uint16_t* x, const uint16_t* delta, const uint16_t* weight, uint16_t* out, int64_t rows,
                    int64_t hidden, float eps, void* stream);
@@ -105,6 +109,8 @@ int qf_rope_decode_attention(const uint16_t* qkv, const int64_t* pos, const floa
                              uint16_t* k_cache, uint16_t* v_cache, uint16_t* out, int64_t batch, int64_t heads,
                              int64_t head_dim, int64_t max_len, void* stream);
 int qf_silu_mul(const uint16_t* gate_up, uint16_t* out, int64_t rows, int64_t mlp, void* stream);
+int qf_greedy_next(const uint16_t* logits, int64_t* tok, int64_t* pos, const uint16_t* embed, uint16_t* x_next,
+                   int64_t batch, int64_t vocab, int64_t hidden, void* stream);
 
 #ifdef __cplusplus
 }

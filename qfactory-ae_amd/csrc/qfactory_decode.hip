@@ -403,6 +403,58 @@ __global__ __launch_bounds__(kThreads) void silu_mul_kernel(const f16* __restric
     *reinterpret_cast<f16x8*>(out + m * mlp + c) = o;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Greedy choice of the next token and what the next decode step starts from, one block per sequence:
+// tok[b] = the smallest index of the largest logit of row b (NaN is never chosen), x_next[b] = embed[tok[b]] (if
+// embed is given), and *pos += 1 (block 0, if pos is given).
+// ---------------------------------------------------------------------------------------------
+constexpr int kPickThreads = 1024;
+
+__global__ __launch_bounds__(kPickThreads) void greedy_next_kernel(const f16* __restrict__ logits, int64_t* __restrict__ tok,
+                                                                  int64_t* __restrict__ pos, const f16* __restrict__ embed,
+                                                                  f16* __restrict__ x_next, int vocab, int hidden) {
+    __shared__ float best_v[kPickThreads / 64];
+    __shared__ int best_i[kPickThreads / 64];
+    __shared__ int chosen;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const f16* row = logits + (int64_t)b * vocab;
+    float v = -__builtin_inff();
+    int at = 0x7fffffff;
+    for (int c = tid * 8; c < vocab; c += kPickThreads * 8) {            // ascending indices per thread: '>' keeps the first
+        const f16x8 l = *reinterpret_cast<const f16x8*>(row + c);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float f = (float)l[e];
+            if (f > v || (f == v && c + e < at)) { v = f; at = c + e; }
+        }
+    }
+    auto better = [](float fv, int fi, float gv, int gi) { return fv > gv || (fv == gv && fi < gi); };
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const float ov = __shfl_xor(v, d);
+        const int oi = __shfl_xor(at, d);
+        if (better(ov, oi, v, at)) { v = ov; at = oi; }
+    }
+    if ((tid & 63) == 0) { best_v[tid >> 6] = v; best_i[tid >> 6] = at; }
+    __syncthreads();
+    if (tid == 0) {
+        float fv = best_v[0];
+        int fi = best_i[0];
+        for (int w = 1; w < kPickThreads / 64; w++)
+            if (better(best_v[w], best_i[w], fv, fi)) { fv = best_v[w]; fi = best_i[w]; }
+        if (fi >= vocab) fi = 0;                                           // a row without a finite or infinite maximum (all NaN)
+        chosen = fi;
+        tok[b] = fi;
+        if (b == 0 && pos != nullptr) *pos += 1;
+    }
+    __syncthreads();
+    if (embed != nullptr) {
+        const f16* src = embed + (int64_t)chosen * hidden;
+        for (int c = tid * 8; c < hidden; c += kPickThreads * 8)
+            *reinterpret_cast<f16x8*>(x_next + (int64_t)b * hidden + c) = *reinterpret_cast<const f16x8*>(src + c);
+    }
+}
+
 template <int LPK, bool FUSED>
 int launch_attention(const char* fn, const f16* q_or_qkv, f16* k, f16* v, const int64_t* pos, const float* cos_t, const float* sin_t,
                      f16* out, int batch, int heads, int max_len, hipStream_t stream) {
@@ -504,4 +556,16 @@ extern "C" int qf_silu_mul(const uint16_t* gate_up, uint16_t* out, int64_t rows,
     hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((work + kThreads - 1) / kThreads)), dim3(kThreads), 0, (hipStream_t)stream,
                        (const f16*)gate_up, (f16*)out, rows, (int)mlp);
     return launched("qf_silu_mul");
+}
+
+extern "C" int qf_greedy_next(const uint16_t* logits, int64_t* tok, int64_t* pos, const uint16_t* embed, uint16_t* x_next,
+                              int64_t batch, int64_t vocab, int64_t hidden, void* stream) {
+    if (!logits || !tok) return fail("qf_greedy_next", "null pointer");
+    if ((embed == nullptr) != (x_next == nullptr)) return fail("qf_greedy_next", "embed and x_next come together");
+    if (batch <= 0 || batch > 0x7fffffff || vocab <= 0 || vocab > 0x7fffff00 || vocab % 8 != 0)
+        return fail("qf_greedy_next", "batch positive, vocab a positive multiple of 8");
+    if (embed && (hidden <= 0 || hidden > 0x7fffffff || hidden % 8 != 0)) return fail("qf_greedy_next", "hidden a positive multiple of 8");
+    hipLaunchKernelGGL(greedy_next_kernel, dim3((unsigned)batch), dim3(kPickThreads), 0, (hipStream_t)stream, (const f16*)logits, tok,
+                       pos, (const f16*)embed, (f16*)x_next, (int)vocab, (int)hidden);
+    return launched("qf_greedy_next");
 }

@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256) void bf16_to_f16_kernel(const uint16_t* __rest
 
 }  // namespace
 
-extern "C" int qf_version(void) { return 101; }
+extern "C" int qf_version(void) { return 102; }
 
 extern "C" int qf_bf16_to_f16(const uint16_t* src, uint16_t* dst, int64_t n, void* stream_) {
     if (!src || !dst) return fail("qf_bf16_to_f16", "null pointer");

@@ -183,12 +183,15 @@ class QuantLlama:
         native.add_rmsnorm(last, None, self.final_norm, last, shape.eps)
         return self.linear(self.lm_head, last)
 
-    def decode_step(self, tok, pos):
+    def decode_step(self, tok, pos, x=None):
         """tok (B, 1) int64, pos one-element int64 device tensor: logits (B, vocab) of the next token, like
-        ``forward`` at T = 1, with every step between the linears a single launch of libqfactory_hip.so."""
+        ``forward`` at T = 1, with every step between the linears a single launch of libqfactory_hip.so.
+        ``x`` (B, hidden): the embedding rows of ``tok`` where the caller already has them (``native.greedy_next``
+        leaves them behind); the buffer is used as the residual stream and overwritten."""
         from qfactory import native
         shape = self.shape
-        x = self.embed[tok[:, 0]]                                # (B, h): the residual stream, updated in place
+        if x is None:
+            x = self.embed[tok[:, 0]]                            # (B, h): the residual stream, updated in place
         delta = None
         first = self.layers[0]
         rows = x.shape[0]
@@ -261,6 +264,7 @@ def linears_time_us(model, M, reps=8):
 
 
 def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
+    from qfactory import native
     assert prompt_len + new_tokens <= shape.max_len
     model = QuantLlama(shape, batch, seed)
     gen = torch.Generator(device="cuda").manual_seed(seed + 1)
@@ -275,25 +279,31 @@ def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
 
-    # ---- decode: one step (forward + argmax + position update) captured in a HIP graph ----
+    # ---- decode: one step (forward + greedy choice + position update) captured in a HIP graph ----
     tok = logits.argmax(-1, keepdim=True)                        # (B, 1) static buffers of the graph
     pos = torch.full((1,), prompt_len, device="cuda", dtype=torch.int64)
     tok0, pos0 = tok.clone(), pos.clone()
 
+    x0 = model.embed[tok[:, 0]]                                  # embedding rows of the current tokens, kept current by the step
+
     def step():
-        lg = model.forward(tok, pos) if torch_glue else model.decode_step(tok, pos)
-        tok.copy_(lg.argmax(-1, keepdim=True))
-        pos.add_(1)
+        if torch_glue:
+            lg = model.forward(tok, pos)
+            tok.copy_(lg.argmax(-1, keepdim=True))
+            pos.add_(1)
+        else:
+            # greedy choice, position update and the next step's embedding rows: one launch behind the output projection
+            native.greedy_next(model.decode_step(tok, pos, x0), tok, pos, model.embed, x0)
 
     step()                                                       # eager warm-up of the M = batch kernels
     torch.cuda.synchronize()
-    tok.copy_(tok0), pos.copy_(pos0)
+    tok.copy_(tok0), pos.copy_(pos0), x0.copy_(model.embed[tok0[:, 0]])
     graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
         step()
     torch.cuda.current_stream().wait_stream(side)
-    tok.copy_(tok0), pos.copy_(pos0)
+    tok.copy_(tok0), pos.copy_(pos0), x0.copy_(model.embed[tok0[:, 0]])
     torch.cuda.synchronize()
     generated = []
     t0 = time.perf_counter()

@@ -53,7 +53,9 @@
 #endif
 
 // Timing experiments (results are wrong when non-zero): bit 0 skips the activation loads, bit 1 the
-// dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores, bit 3 the weight loads.
+// dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores, bit 3 the weight loads; bit 4 keeps the
+// loads and their prefetch order but replaces the hand-off through LDS, the decode and the MFMAs by an XOR of what
+// was loaded; bit 5 skips the scale and zero-point loads.
 #ifndef QF_MGEMV_EXPERIMENT
 #define QF_MGEMV_EXPERIMENT 0
 #endif
@@ -210,6 +212,13 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             const int n = min(n_base + min(i * C::RPIH + lane / C::LPRH, 15), C::N - 1);
             const uint8_t* hp = W + (size_t)n * C::RB + C::HI_OFF + (size_t)lo * 32 + (lane % C::LPRH) * 16;
             st.h[i] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)hp) : *(const u32x4*)hp;
+        }
+        if (QF_MGEMV_EXPERIMENT & 32) {
+#pragma unroll
+            for (int j = 0; j < NSI; j++) st.s[j] = 0x2000u;
+#pragma unroll
+            for (int j = 0; j < NZI; j++) st.z[j] = 0x77u;
+            return;
         }
 #pragma unroll
         for (int j = 0; j < NSI; j++) {
@@ -394,7 +403,22 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             u32x4 wfrag[CH];
             u32x2 hfrag[C::HI ? CH : 1];
             uint32_t qs[NSI], qz[NZI];
-            if (have_slot && !(QF_MGEMV_EXPERIMENT & 2)) {
+            if (have_slot && (QF_MGEMV_EXPERIMENT & 16)) {
+                uint32_t x = 0;
+#pragma unroll
+                for (int i = 0; i < CH; i++) x ^= cur.w[i].x ^ cur.w[i].y ^ cur.w[i].z ^ cur.w[i].w;
+#pragma unroll
+                for (int j = 0; j < NSI; j++) x ^= cur.s[j];
+#pragma unroll
+                for (int j = 0; j < NZI; j++) x ^= cur.z[j];
+                acc[0][0] += __builtin_bit_cast(float, x & 0x3FFFFFFFu);
+                if constexpr (STATIC_BATCH) {
+                    if constexpr (BT::value * SB + sb + PF < SLOTS) load_tile(cur, tile_clamped(slot + PF));
+                } else {
+                    if (slot + PF < SLOTS) load_tile(cur, tile_clamped(slot + PF));
+                }
+            }
+            if (have_slot && !(QF_MGEMV_EXPERIMENT & (2 | 16))) {
                 // coalesced registers -> LDS -> fragment registers: lane (r, kb) takes the 16 bytes
                 // of row r at chunk c, k-block kb
 #pragma unroll
@@ -425,7 +449,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     if (slot + PF < SLOTS) load_tile(cur, tile_clamped(slot + PF));
                 }
             }
-            if (have_slot && tile_ok(slot) && !(QF_MGEMV_EXPERIMENT & 2)) {              // wave-uniform
+            if (have_slot && tile_ok(slot) && !(QF_MGEMV_EXPERIMENT & (2 | 16))) {       // wave-uniform
 #pragma unroll
                 for (int c = 0; c < CH; c++) {
                     const int g = ((lo + c) * CHUNK + kb * EPL) / C::GS;     // group of this lane's fields

@@ -38,6 +38,7 @@ SIGNATURES = {
     "qf_decode_attention": (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_rope_decode_attention": (_INT, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _P]),
     "qf_silu_mul": (_INT, [_P, _P, _I64, _I64, _P]),
+    "qf_greedy_next": (_INT, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _P]),
 }
 
 _lock = threading.Lock()
@@ -222,3 +223,25 @@ def silu_mul(gate_up, out):
     assert out.shape == (rows, two_mlp // 2)
     _check(load().qf_silu_mul(_f16(gate_up), _f16(out), rows, two_mlp // 2, _stream()), "qf_silu_mul")
     return out
+
+
+def greedy_next(logits, tok, pos=None, embed=None, x_next=None):
+    """The end of a greedy decode step in one launch: ``tok`` (batch, 1) int64 <- argmax of ``logits`` (batch, vocab)
+    fp16 (the first of equal maxima), ``pos`` (one int64) += 1, and ``x_next`` (batch, hidden) <- ``embed[tok]``, the
+    residual stream of the next step."""
+    import torch
+    batch, vocab = logits.shape
+    assert logits.dtype == torch.float16 and logits.is_contiguous() and logits.is_cuda
+    assert tok.dtype == torch.int64 and tok.numel() == batch and tok.is_contiguous() and tok.device == logits.device
+    assert pos is None or (pos.dtype == torch.int64 and pos.numel() == 1 and pos.device == logits.device)
+    hidden = 0
+    if embed is not None:
+        hidden = embed.shape[1]
+        assert embed.shape[0] == vocab and embed.dtype == torch.float16 and embed.is_contiguous() and embed.device == logits.device
+        assert x_next is not None and x_next.shape == (batch, hidden) and x_next.dtype == torch.float16 and x_next.is_contiguous()
+    else:
+        assert x_next is None
+    _check(load().qf_greedy_next(_f16(logits), tok.data_ptr(), None if pos is None else pos.data_ptr(),
+                                 None if embed is None else _f16(embed), None if x_next is None else _f16(x_next),
+                                 batch, vocab, hidden, _stream()), "qf_greedy_next")
+    return tok

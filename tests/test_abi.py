@@ -29,7 +29,8 @@ def _declared_functions(header, guard=None):
 def test_header_parsers_see_the_expected_prototypes():
     assert _declared_functions("qfactory_hip.h") == sorted(
         ["qf_version", "qf_pack_weight", "qf_pack_zero", "qf_transpose_scale", "qf_bf16_to_f16", "qf_stream_read", "qf_stream_copy", "qf_empty_launch",
-         "qf_add_rmsnorm", "qf_rope_kv_store", "qf_rope_kv_store_rows", "qf_decode_attention", "qf_rope_decode_attention", "qf_silu_mul"])
+         "qf_add_rmsnorm", "qf_rope_kv_store", "qf_rope_kv_store_rows", "qf_decode_attention", "qf_rope_decode_attention", "qf_silu_mul",
+         "qf_greedy_next"])
     assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_GROUPED") == ["launch", "launch_m", "qf_describe"]
     assert _declared_functions("qfactory_launch.h", "QF_LAUNCH_PLAIN") == ["launch", "qf_describe"]
 
@@ -42,7 +43,7 @@ def test_aot_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} missing from {native.LIBRARY}"
     assert sorted(native.SIGNATURES) == _declared_functions("qfactory_hip.h")
     lib.qf_version.restype = ctypes.c_int
-    assert lib.qf_version() == 101          # host-only call: no device work
+    assert lib.qf_version() == 102          # host-only call: no device work
 
 
 @pytest.mark.parametrize("gs,guard", [(128, "QF_LAUNCH_GROUPED"), (-1, "QF_LAUNCH_PLAIN")])

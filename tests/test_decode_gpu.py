@@ -198,6 +198,63 @@ def test_silu_mul_matches_torch(rows, mlp):
     assert ((out.float() - want.float()).norm() / want.float().norm()).item() <= 2e-4
 
 
+@pytest.mark.parametrize("batch,vocab,hidden", [(1, 32000, 4096), (16, 32000, 4096), (64, 1000, 256), (3, 8, 8), (2, 40000, 64)])
+def test_greedy_next_matches_argmax_position_update_and_embedding_lookup(batch, vocab, hidden):
+    from qfactory import native
+    g = _gen(batch + vocab)
+    logits = torch.randn(batch, vocab, device="cuda", generator=g).to(torch.float16)
+    # equal maxima (the first one counts), a maximum in the last element, -inf entries, a NaN that must not win
+    logits[0, vocab // 3] = logits[0, vocab // 2] = 60000.0
+    if batch > 1:
+        logits[1, :] = -3.0
+        logits[1, vocab - 1] = 5.0
+    if batch > 2:
+        logits[2, : vocab // 2] = float("-inf")
+        logits[2, 1] = float("nan")
+    want = torch.where(torch.isnan(logits), torch.full_like(logits, float("-inf")), logits).float().argmax(-1, keepdim=True)
+    assert int(want[0]) == vocab // 3
+    embed = torch.randn(vocab, hidden, device="cuda", generator=g).to(torch.float16)
+    tok = torch.full((batch, 1), -1, dtype=torch.int64, device="cuda")
+    pos = torch.tensor([41], dtype=torch.int64, device="cuda")
+    x = torch.full((batch, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    native.greedy_next(logits, tok, pos, embed, x)
+    torch.cuda.synchronize()
+    assert torch.equal(tok, want) and int(pos) == 42 and torch.equal(x, embed[want[:, 0]])
+    # without the optional operands: the choice alone
+    tok.fill_(-1)
+    native.greedy_next(logits, tok)
+    assert torch.equal(tok, want) and int(pos) == 42
+
+
+def test_graph_decode_with_the_fused_step_end_generates_what_separate_torch_ops_generate():
+    """decode_llama.run ends a step with one launch (greedy choice, position update, next embedding rows); the same
+    model stepped with torch's argmax, an add and an embedding lookup must produce the same tokens."""
+    import decode_llama
+    from qfactory import native
+    shape = decode_llama.LlamaShape(layers=2, hidden=256, heads=4, mlp=512, vocab=1000, max_len=32, group_size=64)
+    model = decode_llama.QuantLlama(shape, 2, seed=3)
+    prompt = torch.randint(0, shape.vocab, (2, 8), device="cuda", generator=_gen(4))
+    outs = []
+    for fused in (False, True):
+        model.k_cache.zero_(), model.v_cache.zero_()
+        logits = model.prefill(prompt, torch.arange(8, device="cuda"))
+        tok = logits.argmax(-1, keepdim=True)
+        pos = torch.full((1,), 8, device="cuda", dtype=torch.int64)
+        x0 = model.embed[tok[:, 0]]
+        seq = [tok.clone()]
+        for _ in range(6):
+            if fused:
+                native.greedy_next(model.decode_step(tok, pos, x0), tok, pos, model.embed, x0)
+            else:
+                lg = model.decode_step(tok, pos)
+                tok.copy_(lg.argmax(-1, keepdim=True))
+                pos.add_(1)
+            seq.append(tok.clone())
+        assert int(pos) == 14
+        outs.append(torch.cat(seq, dim=1))
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_decode_step_matches_the_torch_evaluation_of_the_same_model():
     import decode_llama
     shape = decode_llama.LlamaShape(layers=2, hidden=256, heads=4, mlp=512, vocab=1000, max_len=32, group_size=64)
