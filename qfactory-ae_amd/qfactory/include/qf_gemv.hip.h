@@ -22,6 +22,12 @@
 #include <cstdio>
 #include "qf_common.hip.h"
 
+// 1: a kernel that adds to its output (QF_OUT_ACCUMULATE) requests the output elements a thread will write when the
+// block starts; 0: right in front of the store.
+#ifndef QF_GEMV_EARLY_OUT
+#define QF_GEMV_EARLY_OUT 1
+#endif
+
 namespace qf {
 
 template <int NBITS_, int GS_, bool SYM_, bool QPARAM_, int N_, int K_, int MT_, int WK_, int WN_,
@@ -284,6 +290,22 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         }
     }
     if constexpr (QF_GEMV_A_FIRST) load_stage(st0, 0);
+#if QF_OUT_ACCUMULATE && QF_GEMV_EARLY_OUT
+    // Adding to the output: the elements this thread will write at the end (the cross-wave sum below deals them by
+    // thread index) are requested now, behind the activations and the first weight stage, instead of in front of the
+    // store, where a one-shot block would wait out their round trip with nothing else to do.
+    constexpr int OUTS = (STEPS * V + T - 1) / T;
+    uint16_t old_out[OUTS];
+    if constexpr (!(WK == 1 && !SILU)) {
+#pragma unroll
+        for (int i = 0; i < OUTS; i++) {
+            const int j = min(tt + i * T, STEPS * V - 1);
+            const int step = j / V, v = j % V;
+            const int row = min(row_base + step * U + v / MT, C::N - 1), m = min(m0 + v % MT, m_total - 1);
+            old_out[i] = Cout[(size_t)m * C::N + row];
+        }
+    }
+#endif
     if constexpr (NORM) {
         static_assert(!QF_IN_BF16, "the norm prologue is fp16 only");
         // ---- residual add, sum of squares, normalisation: a[][][] becomes the normalised row ----
@@ -569,7 +591,15 @@ __global__ __launch_bounds__(C::THREADS) QF_GEMV_OCCUPANCY void gemv_kernel(
         const int step = j / V, v = j % V;
         const int u = v / MT, m = v % MT;
         const int row = row_base + step * U + u;
+#if QF_OUT_ACCUMULATE && QF_GEMV_EARLY_OUT
+        if (row < C::N && m0 + m < m_total) {
+            // out = fp16(out + fp16(projection)) on the value requested at the top
+            const _Float16 sum = __builtin_bit_cast(_Float16, old_out[(j - tt) / T]) + (_Float16)total;
+            Cout[(size_t)(m0 + m) * C::N + row] = __builtin_bit_cast(uint16_t, sum);
+        }
+#else
         if (row < C::N && m0 + m < m_total) store_out(Cout + (size_t)(m0 + m) * C::N + row, total);
+#endif
     }
 }
 
