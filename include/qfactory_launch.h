@@ -75,7 +75,7 @@ typedef void (*qf_launch_grouped_norm_fn)(int m, void* activation, void* delta, 
  * arrival counters through device memory.  launch / launch_m of such an object allocate that memory (hipMalloc, once
  * per device, at their first call there); launch_m_static uses a static device array of the object instead (at most
  * 8 MiB, one copy per GPU, held until the process ends) and calls no allocating routine.  Same arguments, same
- * result bits as launch_m.  At most 16 rows; an object whose scratch memory would exceed the array returns 1 with a
+ * result bits as launch_m.  At most 16 rows (32 for an object built for 17 .. 32); an object whose scratch memory would exceed the array returns 1 with a
  * message (call launch_m).  All calls on one GPU share the array: calls that overlap in time on one GPU race
  * (calls enqueued on one stream do not overlap).  Every other object already allocates nothing in launch / launch_m.
  */

@@ -412,12 +412,20 @@ def mgemv_ksplit_tiling(M, N, K, nbits, group_size):
     4096 x 11008 13.7 / 17.2 -> 13.8 / 15.0.  2 and 3 bits: only where the unsplit kernel cannot hold the activations
     (4096 x 12288: 10.2 / 11.8 -> 10.1 / 10.4 at 2 bits, 23.2 / 23.5 -> 11.6 / 11.8 at 3; 16384 x 16384 at 2 bits 62 / 107
     -> 38 / 38); at K = 8192 the unsplit kernel is 1 - 2 us ahead."""
-    if nbits not in KSPLIT_BITS or not (MGEMV_MIN_M <= M <= KSPLIT_MAX_M) or K < KSPLIT_MIN_K:
+    if nbits not in KSPLIT_BITS or not (MGEMV_MIN_M <= M <= 2 * KSPLIT_MAX_M) or K < KSPLIT_MIN_K:
         return None
     if not mgemv_supported(K, nbits, group_size):
         return None
     if nbits in (2, 3) and mgemv_tiling(M, N, K, nbits, group_size) is not None:
         return None
+    mt16 = -(-M // 16)
+    if mt16 == 2:
+        # 17 .. 32 rows (two activation tiles per wave, eight to eleven waves): measured against the GEMM kernel with
+        # 32-row tiles, which serves long rows there otherwise: 4096 x 11008 19.4 -> 12.5 us, 4096 x 14336 23.8 -> 17.1;
+        # level at K = 8192 (8192 x 8192 17.2 -> 16.7, 10240 x 8192 21.0 -> 20.5), slower on wide or very long layers
+        # (57344 x 8192 67 -> 87, 8192 x 28672 45 -> 54): only narrow layers with long rows
+        if nbits != 4 or not N or N > 4096 or K < 11008 or mgemv_tiling(M, N, K, nbits, group_size) is not None:
+            return None
     chunk = 4 * (128 // plane_bits(nbits))
     if group_size % chunk and chunk % group_size:
         return None
@@ -428,12 +436,12 @@ def mgemv_ksplit_tiling(M, N, K, nbits, group_size):
         nb = -(-nchunk // ks)
         wk = -(-nb // ch)
         # (2 and 3 bits: the transposition buffers of sixteen waves do not fit the LDS; eight do)
-        if wk <= 16 and mgemv_regs(1, ch, 1, nbits) <= mgemv_reg_limit(wk) and mgemv_lds_bytes(1, wk, ch, nbits) <= 160 * 1024:
+        if wk <= 16 and mgemv_regs(mt16, ch, 1, nbits) <= mgemv_reg_limit(wk) and mgemv_lds_bytes(mt16, wk, ch, nbits) <= 160 * 1024:
             break
         ks *= 2
     if ks > 16 or (ks - 1) * nb >= nchunk or (wk - 1) * ch >= nb:
         return None
-    return {"MT16": 1, "WK": wk, "CH": ch, "PB": NUM_CUS // ks, "PF": 1, "KS": ks}
+    return {"MT16": mt16, "WK": wk, "CH": ch, "PB": NUM_CUS // ks, "PF": 1, "KS": ks}
 
 
 def mgemv_candidates(M, N, K, nbits, group_size):

@@ -40,8 +40,10 @@ def test_regime_routing(M, K, nbits, gs, expected):
     (16, 28672, 4, 128, 8), (8, 53248, 4, 128, 16), (16, 8192, 8, 128, 2), (16, 11008, 8, 128, 4),
     (16, 12288, 2, 128, 4), (16, 12288, 3, 128, 4), (16, 8192, 4, 64, 2), (16, 8192, 4, 32, 2),
     # not split: short rows, one or two activation rows, more than sixteen, 2 and 3 bits where the unsplit kernel holds K
-    (16, 4096, 4, 128, 1), (16, 5120, 4, 128, 1), (2, 8192, 4, 128, 1), (17, 8192, 4, 128, 1), (32, 11008, 4, 128, 1),
+    (16, 4096, 4, 128, 1), (16, 5120, 4, 128, 1), (2, 8192, 4, 128, 1), (17, 8192, 4, 128, 1), (33, 11008, 4, 128, 1),
     (16, 8192, 2, 128, 1), (16, 8192, 3, 128, 1),
+    # 17 .. 32 rows: two activation tiles per wave, narrow layers with long rows only
+    (32, 11008, 4, 128, 4), (17, 14336, 4, 128, 8), (32, 11008, 8, 128, 1),
 ])
 def test_long_rows_are_split_over_blocks(M, K, nbits, gs, ks):
     t = tiling.mgemv_ksplit_tiling(M, 4096, K, nbits, gs)
@@ -52,12 +54,18 @@ def test_long_rows_are_split_over_blocks(M, K, nbits, gs, ks):
     assert tiling.regime_for(M, K, nbits, gs, 4096) == "mgemv"
     chunk = 4 * (128 // tiling.plane_bits(nbits))
     nchunk, nb = K // chunk, -(-(K // chunk) // ks)
-    assert t["KS"] == ks and t["PB"] * ks == tiling.NUM_CUS and t["MT16"] == 1
+    assert t["KS"] == ks and t["PB"] * ks == tiling.NUM_CUS and t["MT16"] == -(-M // 16)
     assert t["WK"] <= 16 and t["WK"] * t["CH"] >= nb and (t["WK"] - 1) * t["CH"] < nb      # the waves cover a block's share, none idle
     assert (ks - 1) * nb < nchunk                                                            # every block owns part of K
-    assert tiling.mgemv_lds_bytes(1, t["WK"], t["CH"], nbits) <= 160 * 1024
-    assert tiling.mgemv_regs(1, t["CH"], t["PF"], nbits) <= tiling.mgemv_reg_limit(t["WK"])
+    assert tiling.mgemv_lds_bytes(t["MT16"], t["WK"], t["CH"], nbits) <= 160 * 1024
+    assert tiling.mgemv_regs(t["MT16"], t["CH"], t["PF"], nbits) <= tiling.mgemv_reg_limit(t["WK"])
     assert f", {ks}>" in tiling.mgemv_cfg_string({"NBITS": nbits, "GS": gs, "SYM": False, "N": 4096, "K": K}, t, True)
+
+
+def test_wide_layers_keep_the_gemm_kernel_at_32_rows():
+    assert tiling.mgemv_ksplit_tiling(32, 8192, 28672, 4, 128) is None and tiling.regime_for(32, 28672, 4, 128, 8192) == "gemm"
+    assert tiling.mgemv_ksplit_tiling(32, 0, 11008, 4, 128) is None          # the width is not known: no split
+    assert tiling.regime_for(32, 11008, 4, 128, 4096) == "mgemv" and tiling.regime_for(32, 11008, 4, 128) == "gemm"
 
 
 def test_split_rows_are_not_combined_with_the_norm_prologue_or_the_swiglu_epilogue():
