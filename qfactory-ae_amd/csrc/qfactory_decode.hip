@@ -162,16 +162,17 @@ __global__ __launch_bounds__(kThreads) void rope_kv_store_kernel(const f16* __re
 // store them), k and v are appended to the cache, and the new position is served from LDS rather than
 // re-read from memory the block has just written.
 // ---------------------------------------------------------------------------------------------
-// Few (sequence, head) pairs: 8 waves per block and the first 8 positions of every group requested up front; many:
-// 4 waves per block keep more blocks resident.  Measured with 32 heads of 128 at 130 / 191 / 250 cache positions,
-// cold caches: 8 waves with the up-front requests 5.4 / 5.6 / 6.0 us at batch 1 and 10.5 / 12.5 / 14.9 at batch 16;
-// 16 waves walking the cache two positions at a time 5.6 / 6.2 / 6.8 and 11.5 / 14.2 / 16.7.  Every wave repeats the
-// rotation of q and the merge steps, so more waves cost vector issue on the few CUs that have a block; a launch
+// 8 waves per block and the first 8 positions of every group requested up front, at every batch size.  Measured with 32
+// heads of 128 at 130 / 191 / 250 cache positions, cold caches: 5.4 / 5.6 / 6.0 us at batch 1, 10.4 / 12.4 / 14.9 at
+// batch 16, 28.9 / 37.1 / 47.3 at batch 64 (there the kernel reads 200 MB of cache per launch and is HBM-bound).
+// Against it: 16 waves walking the cache two positions at a time 5.6 / 6.2 / 6.8 and 11.5 / 14.2 / 16.7 at batch 1 and 16;
+// 4 waves per block and one pass with a running maximum (the variant that served 1024 pairs and more) 8.7 / 10.8 /
+// 13.7 at batch 4, 11.8 / 14.9 / 18.0 at batch 16, 30.8 / 41.9 / 52.8 at batch 64, and 5 - 7 % behind at 500 and 900
+// positions too.  Every wave repeats the rotation of q and the merge steps, so more waves cost vector issue; a launch
 // costs 4.0 us before it touches the cache (the position, then the new token's q / k / v, then the stores: three
 // dependent round trips behind a 1.7 us launch).
-constexpr int kAttnThreadsFew = 512, kAttnThreadsMany = 256;
-constexpr int kAttnManyBlocks = 1024;
-constexpr int kAttnPrefetch = 8;          // positions per group requested up front by the few-blocks variant (256 at 128-wide heads)
+constexpr int kAttnThreads = 512;
+constexpr int kAttnPrefetch = 8;          // positions per group requested up front (256 at 128-wide heads)
 
 __device__ __forceinline__ f16x8 rotate8(const f16x8 x, const float* __restrict__ c, const float* __restrict__ s) {
 #pragma clang fp contract(off)                                // same roundings as rope_kv_store_kernel
@@ -460,13 +461,8 @@ int launch_attention(const char* fn, const f16* q_or_qkv, f16* k, f16* v, const 
                      f16* out, int batch, int heads, int max_len, hipStream_t stream) {
     constexpr int HD = LPK * 8;
     const float scale = 1.0f / sqrtf((float)HD);
-    const bool many = (int64_t)batch * heads >= kAttnManyBlocks;
-    if (many)
-        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsMany, 0>), dim3(heads, batch), dim3(kAttnThreadsMany), 0,
-                           stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
-    else
-        hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreadsFew, kAttnPrefetch>), dim3(heads, batch), dim3(kAttnThreadsFew), 0,
-                           stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
+    hipLaunchKernelGGL((decode_attention_kernel<LPK, FUSED, kAttnThreads, kAttnPrefetch>), dim3(heads, batch), dim3(kAttnThreads), 0,
+                       stream, q_or_qkv, k, v, pos, cos_t, sin_t, out, heads, max_len, scale);
     return launched(fn);
 }
 
