@@ -55,8 +55,9 @@ def parity_cases():
               _case(16, 272, 14336, 4, 256), _case(12, 48, 14336, 2, 256), _case(16, 64, 14336, 2, 512, True),
               _case(9, 64, 8192, 8, 128), _case(4, 100, 8192, 8, 64), _case(11, 40, 11008, 8, 32, True),
               _case(8, 8200, 11008, 4, 128)]
-    # two activation rows on a wide layer: four stages per block in the dot2 GEMV
-    cases += [_case(2, 22016, 4096)]
+    # two activation rows: four stages per block in the dot2 GEMV, and swept tilings of the reference's shapes
+    # (one team per block, seven waves per row, eight rows per stage)
+    cases += [_case(2, 22016, 4096), _case(2, 4096, 11008), _case(2, 10240, 8192), _case(2, 5120, 13824), _case(2, 7168, 5120)]
     # 2-bit at K = 4096: the A-stationary kernel's 16-wave tiling does not fit LDS, 8 waves do
     cases += [_case(16, 100, 4096, 2, 128), _case(32, 48, 4096, 2, 64, True)]
     # 3-bit (two planes per row) in the A-stationary kernel: ragged M and N, a last wave that owns fewer
