@@ -249,6 +249,14 @@ class QMatmulQFunc(QFunc):
             # stage) 8.85 -> 8.26; two chunks per lane (K = 28672) lose 6 %, K = 11008 is level.
             defines.setdefault("QF_FUSED_AND_OR", 2)
             defines.setdefault("QF_GEMV_QUANT_DEDUP", 1)
+        if self.regime == "mgemv" and t.get("KS", 1) == 1 and t["WK"] <= 10 and t["MT16"] == 1 \
+                and self.output_epilogue != "silu_mul":
+            # ten waves and fewer leave LDS for eight partial tiles per wave between two block-wide sums instead of
+            # four; it pays where a block sweeps many tiles (K = 5120 at M = 16, cold weights: 27648 x 5120 20.6 -> 18.7 us,
+            # 55296 x 5120 36.7 -> 33.7; 15360 x 5120 13.0 -> 12.9, 7168 x 5120 level)
+            slots = -(-(-(-p["N"] // 16)) // min(-(-p["N"] // 16), t["PB"]))
+            if slots >= 6 and tiling.mgemv_lds_bytes(1, t["WK"], t["CH"], p["NBITS"], sb=8) <= 160 * 1024:
+                defines.setdefault("QF_MGEMV_SB", 8)
         if self.regime == "gemm":
             # Block -> tile map that puts the row slabs of one column of tiles on one XCD (its L2 then serves the weights to
             # all of them) instead of the columns of one slab: pays where a launch has a few slabs -- measured, FETCH_SIZE
