@@ -12,8 +12,10 @@ Five kernel families (``regime_for`` picks one):
   and load.
 * ``mgemv`` -- 3 <= M <= 32 when the activations fit the register file: persistent A-stationary MFMA
   kernel, ``qf::MGemvCfg`` (include/qf_mgemv.hip.h): ``MT16`` 16-row activation tiles, ``WK`` waves x
-  ``CH`` chunks covering K, ``PB`` blocks, ``PF`` weight tiles in flight.
-* ``skinny`` -- 3 <= M <= 16 where ``mgemv`` cannot hold the activations (K = 11008, 8-bit K = 8192 ...):
+  ``CH`` chunks covering K, ``PB`` blocks, ``PF`` weight tiles in flight.  Long rows (K >= 7168, 3 <= M <= 16;
+  narrow layers up to 32 rows): ``KS`` blocks split K and meet through scratch memory (``mgemv_ksplit_tiling``).
+* ``skinny`` -- 3 <= M <= 16 where ``mgemv`` cannot hold the activations and K is not split over blocks
+  (``ksplit=False``: layers with the norm prologue or the SwiGLU epilogue; what the split does not take):
   ``qf::SkinnyCfg`` (include/qf_skinny.hip.h): activations streamed per K-step instead of resident,
   ``WK`` waves splitting K, ``SB`` tiles per batch, ``D`` stages in flight, ``AST`` resident fragments.
 * ``gemm``  -- larger M (and what ``mgemv`` cannot hold): ``qf::GemmCfg`` (include/qf_gemm.hip.h):

@@ -20,9 +20,10 @@
 //   * Each wave parks its partial 16x16 tiles in its own LDS slots; one barrier at the end of the
 //     block, then the partials of the WK waves are summed and every output is written once.
 //   * Long rows (KS > 1): K is also split over KS blocks, each holding the activations of its own K/KS only.  A block
-//     writes the fp32 sums of a batch of tiles to a scratch buffer in device memory and counts itself in; the block
-//     that arrives last adds the KS partial results in the fixed order 0 .. KS-1 (the result does not depend on who
-//     arrives when), stores the outputs and clears the counter for the next launch.
+//     writes the fp32 sums of its tiles to a scratch buffer in device memory as it goes and counts itself in once, behind
+//     its last batch; the block that arrives last adds the KS partial results of every tile in the fixed order
+//     0 .. KS-1 (the result does not depend on who arrives when), stores the outputs and clears the counter for the
+//     next launch.
 #pragma once
 
 #include <atomic>
@@ -667,6 +668,9 @@ MGemvScratch mgemv_scratch() {
         const size_t bytes = C::SCRATCH_BYTES * kMGemvScratchRowBlocks;
         hipError_t e = hipMalloc(&p, bytes);
         if (e == hipSuccess) e = hipMemset(p, 0, bytes);
+        // the counters are zero before any launch can read them, on whatever stream it is enqueued (a stream created
+        // non-blocking does not wait for the null stream's memset by itself)
+        if (e == hipSuccess) e = hipDeviceSynchronize();
         if (e != hipSuccess) {
             fprintf(stderr, "qfactory mgemv: cannot set up %zu bytes of scratch memory: %s\n", bytes, hipGetErrorString(e));
             return MGemvScratch{};
