@@ -25,7 +25,8 @@ prefill row count) and `decode` (configs[4]: the Llama-2-7B-shaped decode loop a
 Other modes (each prints its own JSON and exits): `--counter-pass` and `--counter-pass-matrix` (a few eager
 launches of the GEMV kernels / of the matrix-core kernels beside a copy of known size, for `rocprofv3 --pmc`),
 `--shape-sets` (the reference's figure 6 / 9 / 10 and table 3 shape sets: achieved bandwidth and speed-up over the
-dense fp16 GEMM).
+dense fp16 GEMM), `--launch-floor` (an empty kernel and a pure streaming read), `--ablation` (each kernel family
+beside timing builds of itself that leave one part out).
 
 Every per-kernel timing rotates over at least 512 MB of distinct packed weights (twice the 256 MB
 Infinity Cache), so each launch streams its weights from HBM.
@@ -140,6 +141,10 @@ def warm_replays(graph):
     once = max(start.elapsed_time(end), 1e-3)
     for _ in range(max(1, min(200, int(WARM_MS / once)))):
         graph.replay()
+    torch.cuda.synchronize()
+    # One more replay on its own: the first replay behind a burst of queued ones takes about 40 us longer than
+    # every later one (2 us per step of a 20-step graph: 27.5 against 25.7 us per step measured), whatever its length.
+    graph.replay()
     torch.cuda.synchronize()
 
 
@@ -449,6 +454,33 @@ def small_m_report():
     return report
 
 
+def ablation_report():
+    """Where the time of a launch goes: per kernel family, the product's object beside timing builds of the same
+    tiling that leave one part out (`prebuild.ABLATIONS`: the headers' `QF_*_EXPERIMENT` knobs; their results are wrong
+    by design and nothing but this mode compiles them), and a pure streaming read of the same bytes.  Cold weights,
+    timed like every other kernel here."""
+    import torch
+    import prebuild
+    from qfactory.jit import jit
+    report = []
+    for M, N, K in prebuild.ABLATION_PROBLEMS:
+        op, regime, builds = prebuild.ablation_builds(M, N, K)
+        lin, sets, x = _timed_problem(M, N, K, NBITS, False)
+        rows = []
+        for bits, label, obj in builds:
+            func = op._wrap(jit.compile(obj), builds[0][2])
+            us = kernel_event_time_us(func, sets, x, N)
+            rows.append({"knob": bits, "what": label, "us": round(us, 3)})
+            log(f"[bench] ablation M={M:4d} N={N:6d} K={K:6d} {regime:6s} knob {bits:3d} {us:9.2f} us  {label}")
+        read_us = stream_read_time_us(algorithmic_bytes(M, N, K) - 2 * M * (N + K))
+        log(f"[bench] ablation M={M:4d} N={N:6d} K={K:6d} read of the packed tensors {read_us:9.2f} us")
+        report.append({"M": M, "N": N, "K": K, "regime": regime, "kernel": lin.func.runtime.description,
+                       "builds": rows, "read_of_the_packed_tensors_us": round(read_us, 3)})
+        del lin, sets, x
+        torch.cuda.empty_cache()
+    return report
+
+
 def shape_set_problems():
     """The reference's bandwidth and speed-up experiments as (figure, M, N, K, bits, group size) problems:
     fig 9 (reproduce/fig9/plot_bandwidth_size.py:12,32-33: `squares-pure`, M = 1, W4 with and without groups),
@@ -718,6 +750,9 @@ def main():
     ap.add_argument("--counter-pass-matrix", action="store_true",
                     help="the same for the matrix-core kernels: gate_up and down at M = 16, the four GEMMs at M = 256, qkv and "
                          "gate_up at 8192 rows")
+    ap.add_argument("--ablation", action="store_true",
+                    help="only the phase ablation: each kernel family's object beside timing builds that leave one part "
+                         "out, on the 7B layers at M = 1 and 16 and three GEMM problems; prints one JSON object")
     ap.add_argument("--shape-sets", action="store_true",
                     help="only the reference's bandwidth tables: its `squares` and `operator` shape sets at M in {1, 2, 4}, "
                          "8 / 4 / 2 bits, with and without groups; prints one JSON object, writes gpurun_out/shape_sets.json")
@@ -733,6 +768,9 @@ def main():
         return
     if args.counter_pass_matrix:
         counter_pass_matrix()
+        return
+    if args.ablation:
+        print(json.dumps({"ablation": ablation_report()}), flush=True)
         return
     if args.shape_sets:
         report = shape_sets_report()

@@ -402,6 +402,62 @@ def qfuncs_of(case):
     return qfuncs
 
 
+class TimingBuild:
+    """A specialisation compiled with its kernel header's timing knob set (``QF_*_EXPERIMENT``: parts of the kernel
+    left out, results wrong by design), for ``bench.py --ablation`` only.  The code generator refuses these knobs;
+    this wrapper writes them, and the define the headers ask for, in front of the generated translation unit."""
+    KNOBS = {"gemv": "QF_GEMV_EXPERIMENT", "mgemv": "QF_MGEMV_EXPERIMENT", "gemm": "QF_GEMM_EXPERIMENT"}
+
+    def __init__(self, qfunc, bits):
+        assert bits != 0 and qfunc.regime in self.KNOBS
+        self.qfunc, self.bits = qfunc, bits
+
+    def __getattr__(self, name):                      # tiling, argument list, ... are the wrapped specialisation's
+        if name in ("qfunc", "bits"):
+            raise AttributeError(name)
+        return getattr(self.qfunc, name)
+
+    @property
+    def regime(self):                                 # not "gemm": the counted waits of a timing build are not re-counted
+        return self.qfunc.regime + "-timing"
+
+    def emit(self):
+        return (f"#define QF_ALLOW_TIMING_EXPERIMENTS 1\n#define {self.KNOBS[self.qfunc.regime]} {self.bits}\n"
+                + self.qfunc.emit())
+
+
+# What each timing build leaves out (knob value, label), per kernel family; 0 is the product's own object.
+ABLATIONS = {
+    "gemv": [(0, "kernel"), (1, "without decode + dot products"), (8, "without cross-lane sums, LDS exchange, stores"),
+             (9, "without both"), (11, "also without activation loads")],
+    "mgemv": [(0, "kernel"), (4, "without cross-wave sums and stores"),
+              (16, "loads in their order, LDS hand-off + decode + MFMAs replaced by an XOR"),
+              (48, "... and without scale / zero-point loads"), (8, "without the weight loads"),
+              (1, "without the activation loads")],
+    "gemm": [(0, "kernel"), (1, "without dequantisation arithmetic"), (4, "without MFMAs"), (5, "without both"),
+             (72, "without activation tile requests and their wait"), (32, "without weight / scale / zero-point loads"),
+             (16, "without the block barrier of the K loop")],
+}
+ABLATION_PROBLEMS = ([(1, N, K) for N, K in LLAMA2_7B] + [(16, 22016, 4096), (16, 12288, 4096), (16, 4096, 11008), (16, 57344, 8192)]
+                     + [(256, 8192, 8192), (256, 57344, 8192), (8192, 4096, 4096)])
+
+
+def ablation_builds(M, N, K):
+    """(operator, regime, [(knob value, label, object to compile)]) of one ``ABLATION_PROBLEMS`` entry (W4 g128
+    asymmetric): the specialisation ``QLinear`` picks for it, and the timing builds of the same tiling."""
+    import torch
+    from qfactory.core import QMatmul
+    from qfactory.qlinear import _m_bucket
+    op = QMatmul(_m_bucket(M), N, K, 4, False, torch.float16, torch.int8, 128)
+    op.init_qfuncs()
+    q = op.qfuncs[0]
+    return op, q.regime, [(bits, label, q if bits == 0 else TimingBuild(q, bits)) for bits, label in ABLATIONS[q.regime]]
+
+
+def timing_builds():
+    return [obj for M, N, K in ABLATION_PROBLEMS for _, _, obj in ablation_builds(M, N, K)[2]]
+
+
 def prune(keep):
     """Remove cached objects of the in-tree cache that no listed problem compiles to any more (older header
     or generator versions): the cache travels with the tree, stale objects are dead weight."""
@@ -434,6 +490,12 @@ def prebuild(cases=None, force=False, workers=None, verbose=True):
                     if path not in seen:
                         seen.add(path)
                         qfuncs.append(cand)
+    if cases is None:
+        for q in timing_builds():
+            path, _ = jit.runtime_path_of(q)
+            if path not in seen:
+                seen.add(path)
+                qfuncs.append(q)
     if cases is None and os.path.abspath(os.environ["QFACTORY_CACHE_DIR"]) == os.path.join(HERE, "jit_cache"):
         removed = prune(seen)
         if verbose and removed:

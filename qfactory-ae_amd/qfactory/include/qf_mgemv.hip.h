@@ -54,7 +54,8 @@
 #endif
 
 // Timing experiments (results are wrong when non-zero): bit 0 skips the activation loads, bit 1 the
-// dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores, bit 3 the weight loads; bit 4 keeps the
+// dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores (with K split over blocks: the partial sums
+// and the meeting of the blocks), bit 3 the weight loads; bit 4 keeps the
 // loads and their prefetch order but replaces the hand-off through LDS, the decode and the MFMAs by an XOR of what
 // was loaded; bit 5 skips the scale and zero-point loads.
 #ifndef QF_MGEMV_EXPERIMENT
@@ -556,7 +557,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             static_assert(!C::SILU && !NORM, "a block that sees part of K cannot normalise the rows or pair the gate with the up tile");
             const size_t unit = (size_t)blockIdx.y * C::GRID_X + team_id;
             float* const mine = scratch.partial + ((unit * KS + blockIdx.z) * C::NBATCH + batch) * C::PART;
-            for (int o = tid; o < C::PART; o += 64 * WK) {
+            for (int o = tid; o < C::PART && !(QF_MGEMV_EXPERIMENT & 4); o += 64 * WK) {
                 float total = 0.f;
                 const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
                 const float* base = redf + ((size_t)p * 64 + nl + 16 * (ml >> 2)) * 4 + (ml & 3);
@@ -598,6 +599,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         // device-wide fence per thread measured 5 - 20 times the kernel's own time).  A thread's stores have been
         // acknowledged when its memory counter reads zero; the barrier collects that from every thread before the
         // block is counted. ----
+        if (QF_MGEMV_EXPERIMENT & 4) return;                  // timing: no block is counted in, the counters stay zero
         const size_t unit = (size_t)blockIdx.y * C::GRID_X + team_id;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);

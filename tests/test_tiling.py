@@ -248,6 +248,34 @@ def test_timing_experiments_cannot_come_from_the_generator():
     assert "#define QF_GEMV_WAVES_PER_EU 4" in q.emit()
 
 
+def test_timing_builds_wrap_the_products_own_objects():
+    """``bench.py --ablation``: every problem's first build is the object ``QLinear`` runs, the others are the same
+    translation unit behind the two defines the headers ask for; no product module refers to them."""
+    import torch
+    from qfactory.jit import jit
+    from qfactory.qlinear import _m_bucket
+    seen = set()
+    for M, N, K in prebuild.ABLATION_PROBLEMS:
+        op, regime, builds = prebuild.ablation_builds(M, N, K)
+        assert regime == tiling.regime_for(_m_bucket(M), K, 4, 128, N)
+        assert [b for b, _, _ in builds] == [b for b, _ in prebuild.ABLATIONS[regime]] and builds[0][0] == 0
+        product = builds[0][2]
+        assert not isinstance(product, prebuild.TimingBuild)
+        for bits, label, obj in builds[1:]:
+            assert isinstance(obj, prebuild.TimingBuild) and obj.regime == regime + "-timing"
+            head = f"#define QF_ALLOW_TIMING_EXPERIMENTS 1\n#define {prebuild.TimingBuild.KNOBS[regime]} {bits}\n"
+            assert obj.emit() == head + product.emit()
+            assert obj.arg_name_type() == product.arg_name_type() and obj.tiling_configs == product.tiling_configs
+            path, _ = jit.runtime_path_of(obj)
+            assert path not in seen and path != jit.runtime_path_of(product)[0]
+            seen.add(path)
+    package = os.path.join(os.path.dirname(prebuild.__file__), "qfactory")
+    for root, _, files in os.walk(package):
+        for name in files:
+            if name.endswith(".py"):
+                assert "QF_ALLOW_TIMING_EXPERIMENTS" not in open(os.path.join(root, name)).read(), name
+
+
 def test_swept_gemm_tilings_are_valid_and_override_the_model():
     """core/gemm_tuned_gfx950.json: every entry is a tiling the kernel accepts for its problem, differs from what the
     cost model alone picks (or it would not be there), and is what ``gemm_tiling`` returns; any other problem gets
