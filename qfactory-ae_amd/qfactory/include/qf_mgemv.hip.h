@@ -53,6 +53,18 @@
 #define QF_MGEMV_NORM_PROLOGUE 0
 #endif
 
+// 1: a slot past a block's last real tile (it holds the clamped last tile) is computed like any other and never stored;
+// 0: its arithmetic is skipped, which puts every tile's arithmetic into a conditional block (see there).
+#ifndef QF_MGEMV_COMPUTE_CLAMPED
+#define QF_MGEMV_COMPUTE_CLAMPED 1
+#endif
+// Non-zero: the order in which the first PF weight tiles and the activations are requested is fixed by scheduling
+// barriers (1, 2, 3: the orders listed where the loads are issued; measured on sixteen shapes at 4 and 16 rows, 3 is the
+// best or level everywhere, 1 - 3.5 % in front of the compiler's own order); 0 leaves the order to the compiler.
+#ifndef QF_MGEMV_PIN_FIRST_LOADS
+#define QF_MGEMV_PIN_FIRST_LOADS 3
+#endif
+
 // Timing experiments (results are wrong when non-zero): bit 0 skips the activation loads, bit 1 the
 // dequantisation and MFMAs, bit 2 the cross-wave reduction and the stores (with K split over blocks: the partial sums
 // and the meeting of the blocks), bit 3 the weight loads; bit 4 keeps the
@@ -200,7 +212,7 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         uint32_t s[NSI];             // lane -> (row, group) = (idx / GWN, idx % GWN), idx = lane + 64*j
         uint32_t z[NZI];             // lane -> (row, byte)  = (idx / ZB,  idx % ZB)
     };
-    auto load_tile = [&](WStage& st, int tile) {
+    auto load_tile_words = [&](WStage& st, int tile) {
         if (QF_MGEMV_EXPERIMENT & 8) return;
         const int n_base = tile * 16;
 #pragma unroll
@@ -215,6 +227,10 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             const uint8_t* hp = W + (size_t)n * C::RB + C::HI_OFF + (size_t)lo * 32 + (lane % C::LPRH) * 16;
             st.h[i] = C::NT_B ? __builtin_nontemporal_load((const u32x4*)hp) : *(const u32x4*)hp;
         }
+    };
+    auto load_tile_quant = [&](WStage& st, int tile) {
+        if (QF_MGEMV_EXPERIMENT & 8) return;
+        const int n_base = tile * 16;
         if (QF_MGEMV_EXPERIMENT & 32) {
 #pragma unroll
             for (int j = 0; j < NSI; j++) st.s[j] = 0x2000u;
@@ -238,12 +254,28 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         }
     };
 
-    // ring of PF stages: tiles slot .. slot+PF-1 of this team are in flight.  The first PF go out
-    // before anything else, so that their HBM latency overlaps the activation loads.
+    auto load_tile = [&](WStage& st, int tile) {
+        load_tile_words(st, tile);
+        load_tile_quant(st, tile);
+    };
+
+    // ring of PF stages: tiles slot .. slot+PF-1 of this team are in flight.  The first PF are requested with the
+    // activations, in an order that is kept by scheduling barriers (QF_MGEMV_PIN_FIRST_LOADS): left to itself the
+    // compiler issues the first tiles' scale and zero-point loads behind the whole activation phase (they are needed
+    // last), and the first MFMA then waits for a second trip to memory that starts only when the activations are in.
+    // Loads return in order, so what is requested in front of the activations also delays their hand-over through LDS.
+    //   1: packed words, activations, scales and zero-points (the activations' hand-over runs under the latter's latency)
+    //   2: whole tiles, then the activations            3: activations, then whole tiles
     WStage ring[PF];
 #pragma unroll
     for (int p = 0; p < PF; p++)
-        if (p < SLOTS) load_tile(ring[p], tile_clamped(p));
+        if (p < SLOTS) {
+            if (QF_MGEMV_PIN_FIRST_LOADS == 1) load_tile_words(ring[p], tile_clamped(p));
+            else if (QF_MGEMV_PIN_FIRST_LOADS != 3) load_tile(ring[p], tile_clamped(p));
+        }
+#if QF_MGEMV_PIN_FIRST_LOADS
+    __builtin_amdgcn_sched_barrier(0);
+#endif
 
     // ---- resident activations, brought into MFMA fragment order through the wave's LDS buffer:
     //      fragment (mt, c, t) = A[m0 + 16*mt + r][(lo+c)*CHUNK + kb*EPL + 8t .. +8] ----
@@ -270,6 +302,16 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                     if (QF_MGEMV_EXPERIMENT & 1) raw[mt][c][i] = u32x4{(uint32_t)lane, 1u, 2u, 3u};
                     else raw[mt][c][i] = *reinterpret_cast<const u32x4*>(ap);
                 }
+#if QF_MGEMV_PIN_FIRST_LOADS
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int p = 0; p < PF; p++)
+            if (p < SLOTS) {
+                if (QF_MGEMV_PIN_FIRST_LOADS == 1) load_tile_quant(ring[p], tile_clamped(p));
+                else if (QF_MGEMV_PIN_FIRST_LOADS == 3) load_tile(ring[p], tile_clamped(p));
+            }
+        __builtin_amdgcn_sched_barrier(0);
+#endif
         if constexpr (NORM) {
             static_assert(!QF_IN_BF16, "the norm prologue is fp16 only");
             // raw[][][] holds the wave's slices of x in load order: lane -> (row i*RPIA + lane/LPRA, 8 elements at
@@ -450,8 +492,15 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
                 } else {
                     if (slot + PF < SLOTS) load_tile(cur, tile_clamped(slot + PF));
                 }
+#if QF_MGEMV_PIN_FIRST_LOADS
+                __builtin_amdgcn_sched_barrier(0);      // the refill stays in front of this tile's arithmetic
+#endif
             }
-            if (have_slot && tile_ok(slot) && !(QF_MGEMV_EXPERIMENT & (2 | 16))) {       // wave-uniform
+            // A slot past the block's last real tile holds the clamped last tile (valid memory); it is computed like any
+            // other and its sums are never stored.  Skipping it would put the arithmetic into a conditional block, and
+            // the compiler then moves the first tile's scale and zero-point loads -- used nowhere else -- down into
+            // that block, behind the activation phase: a second trip to memory in front of the first MFMA.
+            if (have_slot && (QF_MGEMV_COMPUTE_CLAMPED || tile_ok(slot)) && !(QF_MGEMV_EXPERIMENT & (2 | 16))) {
 #pragma unroll
                 for (int c = 0; c < CH; c++) {
                     const int g = ((lo + c) * CHUNK + kb * EPL) / C::GS;     // group of this lane's fields
