@@ -42,7 +42,7 @@ CONFIG_ATTRIBUTES = ("regime", "parallel_strategy", "tiling_configs", "decode_st
 # compile unless the translation unit itself asks for them; the generator cannot.)
 TUNING_DEFINES = ("QF_FUSED_AND_OR", "QF_SCHED_FENCE_MODE", "QF_WIDE_HOLDERS", "QF_GEMV_A_FIRST",
                   "QF_GEMV_QUANT_DEDUP", "QF_GEMV_WAVES_PER_EU", "QF_GEMV_EARLY_OUT", "QF_MGEMV_SB", "QF_MGEMV_PIN_FIRST_LOADS",
-                  "QF_MGEMV_COMPUTE_CLAMPED", "QF_GEMM_FULL_DRAIN", "QF_GEMM_XCD_MAP")
+                  "QF_MGEMV_COMPUTE_CLAMPED", "QF_MGEMV_MEET_LOADS", "QF_GEMM_FULL_DRAIN", "QF_GEMM_XCD_MAP")
 
 
 def apply_config(qfunc, entry):

@@ -58,6 +58,12 @@
 #ifndef QF_MGEMV_COMPUTE_CLAMPED
 #define QF_MGEMV_COMPUTE_CLAMPED 1
 #endif
+// K split over blocks: device-scope loads the block that adds up the partial sums keeps in flight per thread (KS per
+// output, so 64 / KS outputs at a time; measured 1 / 16 / 32 / 64: 4096 x 11008 at 16 rows 9.77 / 9.45 / 9.50 / 9.57 us,
+// 57344 x 8192 48.5 / 48.2 / 47.5 / 47.8, 8192 x 28672 with eight blocks along K 28.6 / 28.9 / 29.0 / 28.3).
+#ifndef QF_MGEMV_MEET_LOADS
+#define QF_MGEMV_MEET_LOADS 64
+#endif
 // Non-zero: the order in which the first PF weight tiles and the activations are requested is fixed by scheduling
 // barriers (1, 2, 3: the orders listed where the loads are issued; measured on sixteen shapes at 4 and 16 rows, 3 is the
 // best or level everywhere, 1 - 3.5 % in front of the compiler's own order); 0 leaves the order to the compiler.
@@ -658,20 +664,36 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         __syncthreads();
         if (*flag != (unsigned)(KS - 1)) return;               // block-uniform
         const float* const all = scratch.partial + unit * KS * C::NBATCH * C::PART;
-        for (int o = tid; o < C::NBATCH * C::PART; o += 64 * WK) {
-            const int batch = o / C::PART, ob = o % C::PART;
-            const int p = ob >> 8, ml = (ob >> 4) & 15, nl = ob & 15;
-            const int sb = p / MT16, mt = p % MT16;
-            const int slot = batch * SB + sb;
-            const int tile = unit_of(slot);
-            if (slot >= SLOTS || tile >= C::NT) continue;
-            float total = 0.f;
+        // Every device-scope load is a trip to memory, and a loop of "load KS values, add, store" pays one trip per
+        // pass: the loads of up to UN passes go out together (clamped indices, no branch around a load), then the sums.
+        constexpr int TOTAL = C::NBATCH * C::PART, THREADS = 64 * WK;
+        constexpr int PASSES = (TOTAL + THREADS - 1) / THREADS;
+        constexpr int UN_MAX = QF_MGEMV_MEET_LOADS / KS > 1 ? QF_MGEMV_MEET_LOADS / KS : 1;
+        constexpr int UN = PASSES < UN_MAX ? PASSES : UN_MAX;
+        for (int first = 0; first < PASSES; first += UN) {
+            float part[UN][KS];
 #pragma unroll
-            for (int z = 0; z < KS; z++)
-                total += __hip_atomic_load(all + (size_t)z * C::NBATCH * C::PART + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int m = m0 + 16 * mt + ml;
-            const int n = tile * 16 + nl;
-            if (m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, total);
+            for (int u = 0; u < UN; u++) {
+                const int o = min(tid + (first + u) * THREADS, TOTAL - 1);
+#pragma unroll
+                for (int z = 0; z < KS; z++)
+                    part[u][z] = __hip_atomic_load(all + (size_t)z * TOTAL + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const int o = tid + (first + u) * THREADS;
+                const int batch = o / C::PART, ob = o % C::PART;
+                const int p = ob >> 8, ml = (ob >> 4) & 15, nl = ob & 15;
+                const int sb = p / MT16, mt = p % MT16;
+                const int slot = batch * SB + sb;
+                const int tile = unit_of(slot);
+                float total = 0.f;
+#pragma unroll
+                for (int z = 0; z < KS; z++) total += part[u][z];
+                const int m = m0 + 16 * mt + ml;
+                const int n = tile * 16 + nl;
+                if (o < TOTAL && slot < SLOTS && tile < C::NT && m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, total);
+            }
         }
         // nobody else touches this counter again in this launch: zero for the next one
         if (tid == 0) __hip_atomic_store(scratch.arrived + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
