@@ -263,10 +263,12 @@ def linears_time_us(model, M, reps=8):
     return t0.elapsed_time(t1) * 1e3 / reps
 
 
-def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False):
+def run(shape, batch, prompt_len, new_tokens, seed=0, torch_glue=False, fuse_norm=None):
     from qfactory import native
     assert prompt_len + new_tokens <= shape.max_len
     model = QuantLlama(shape, batch, seed)
+    if fuse_norm is not None:
+        model.fuse_norm = fuse_norm
     gen = torch.Generator(device="cuda").manual_seed(seed + 1)
     prompt = torch.randint(0, shape.vocab, (batch, prompt_len), device="cuda", generator=gen)
 
@@ -338,11 +340,14 @@ def main():
     ap.add_argument("--new-tokens", type=int, default=128)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--torch-glue", action="store_true", help="PyTorch ops between the linears of a decode step")
+    ap.add_argument("--separate-norm", action="store_true", help="residual add + RMSNorm as a launch of its own at every batch size")
+    ap.add_argument("--fused-norm", action="store_true", help="... inside the projections wherever the kernels can (up to 32 sequences)")
     args = ap.parse_args()
     assert torch.cuda.is_available(), "decode_llama.py needs the MI355X"
     shape = LlamaShape(layers=args.layers, max_len=args.prompt_len + args.new_tokens)
     for batch in args.batches:
-        print(json.dumps(run(shape, batch, args.prompt_len, args.new_tokens, torch_glue=args.torch_glue)), flush=True)
+        print(json.dumps(run(shape, batch, args.prompt_len, args.new_tokens, torch_glue=args.torch_glue,
+                             fuse_norm=False if args.separate_norm else True if args.fused_norm else None)), flush=True)
         torch.cuda.empty_cache()
 
 
