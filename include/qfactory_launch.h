@@ -5,7 +5,10 @@
  * such object exports the entry points below; all problem and tiling parameters are constants
  * inside the object.  All pointers are device addresses owned by the caller, `stream` is a
  * hipStream_t, the call only enqueues work (no synchronisation), every element of `output` is
- * written exactly once (no pre-zeroing needed) and nothing is retained after return.
+ * written exactly once (no pre-zeroing needed) and nothing of the caller's is retained after return.
+ * The entry points are re-entrant with one exception, spelled out at launch_m_static below: an object whose
+ * qf_describe names "KS=<blocks>" passes partial sums between its blocks through scratch memory it keeps per GPU, so
+ * two launches of that one object must not run on one GPU at the same time (launches on one stream never do).
  *
  * Return code (written through the last argument): 0 launched, 1 the object's static
  * configuration is invalid (reason on stderr), 2 the HIP launch itself failed.
@@ -77,7 +80,11 @@ typedef void (*qf_launch_grouped_norm_fn)(int m, void* activation, void* delta, 
  * 8 MiB, one copy per GPU, held until the process ends) and calls no allocating routine.  Same arguments, same
  * result bits as launch_m.  At most 16 rows (32 for an object built for 17 .. 32); an object whose scratch memory would exceed the array returns 1 with a
  * message (call launch_m).  All calls on one GPU share the array: calls that overlap in time on one GPU race
- * (calls enqueued on one stream do not overlap).  Every other object already allocates nothing in launch / launch_m.
+ * (calls enqueued on one stream do not overlap).  The same holds for launch / launch_m of such an object among
+ * themselves: they share the one buffer allocated per GPU (it is not the static array, so a launch_m and a
+ * launch_m_static may overlap).  Layers of equal shape share one object; a caller that runs two of them on two
+ * streams at once orders them with an event.  Every other object already allocates nothing in launch / launch_m
+ * and keeps no state at all.
  */
 typedef void (*qf_launch_grouped_m_static_fn)(int m, void* activation, void* weight, void* output,
                                               void* scale, void* zero, void* stream, int* return_code);
