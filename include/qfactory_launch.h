@@ -74,8 +74,8 @@ typedef void (*qf_launch_grouped_norm_fn)(int m, void* activation, void* delta, 
  * launch_m without any allocation.  No counterpart in the reference; for callers that cannot allocate device memory:
  * code under HIP-graph capture from its first call on, tight serving loops, harnesses that forbid hipMalloc.
  * Exported only by objects whose kernel uses scratch memory beyond its inputs and outputs -- the A-stationary kernel
- * with long rows split over several blocks (qf_describe names "KS=<blocks>"), whose blocks exchange partial sums and
- * arrival counters through device memory.  launch / launch_m of such an object allocate that memory (hipMalloc, once
+ * with long rows split over several blocks (qf_describe names "KS=<blocks>"), whose blocks exchange partial sums
+ * through device memory.  launch / launch_m of such an object allocate that memory (hipMalloc, once
  * per device, at their first call there); launch_m_static uses a static device array of the object instead (at most
  * 8 MiB, one copy per GPU, held until the process ends) and calls no allocating routine.  Same arguments, same
  * result bits as launch_m.  At most 16 rows (32 for an object built for 17 .. 32); an object whose scratch memory would exceed the array returns 1 with a

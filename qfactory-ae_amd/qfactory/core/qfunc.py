@@ -42,7 +42,7 @@ CONFIG_ATTRIBUTES = ("regime", "parallel_strategy", "tiling_configs", "decode_st
 # compile unless the translation unit itself asks for them; the generator cannot.)
 TUNING_DEFINES = ("QF_FUSED_AND_OR", "QF_SCHED_FENCE_MODE", "QF_WIDE_HOLDERS", "QF_GEMV_A_FIRST",
                   "QF_GEMV_QUANT_DEDUP", "QF_GEMV_WAVES_PER_EU", "QF_GEMV_EARLY_OUT", "QF_MGEMV_SB", "QF_MGEMV_PIN_FIRST_LOADS",
-                  "QF_MGEMV_COMPUTE_CLAMPED", "QF_MGEMV_MEET_LOADS", "QF_GEMM_FULL_DRAIN", "QF_GEMM_XCD_MAP")
+                  "QF_MGEMV_COMPUTE_CLAMPED", "QF_GEMM_FULL_DRAIN", "QF_GEMM_XCD_MAP")
 
 
 def apply_config(qfunc, entry):
@@ -329,7 +329,7 @@ class QMatmulQFunc(QFunc):
             code += ("// ---- entry point that allocates nothing ----\n"
                      "// Scratch memory of launch_m_static: one copy per GPU, held until the process ends, shared by every call on\n"
                      "// that GPU (calls that overlap in time on one GPU race; calls on one stream do not overlap).  Zero at load;\n"
-                     "// every launch leaves its counters zero and overwrites the partial sums before it reads them.\n"
+                     "// every launch leaves the slots in which its blocks exchange their sums zero.\n"
                      "static __device__ __align__(256) unsigned char scratch[qf::mgemv_static_scratch_bytes<Cfg>()];\n\n"
                      "static int qf_static_scratch(qf::MGemvScratch& out) {\n"
                      "\tstatic std::mutex lock;\n\tstatic void* address[64] = {};       // per device: each GPU holds its own copy at its own address\n"

@@ -392,6 +392,8 @@ def mgemv_tiling(M, N, K, nbits, group_size, max_waves=16, **pins):
 
 
 KSPLIT_MIN_K = 7168         # shortest rows the A-stationary kernel splits over several blocks
+KSPLIT_NARROW_MIN_K = 5120          # ... on layers of KSPLIT_NARROW_N[0] .. [1] columns
+KSPLIT_NARROW_N = (4096, 7168)
 KSPLIT_MAX_M = 16
 KSPLIT_WAVE_K = 256         # elements of K whose activations one wave keeps in registers
 KSPLIT_BITS = (2, 3, 4, 8)
@@ -414,7 +416,13 @@ def mgemv_ksplit_tiling(M, N, K, nbits, group_size):
     4096 x 11008 13.7 / 17.2 -> 13.8 / 15.0.  2 and 3 bits: only where the unsplit kernel cannot hold the activations
     (4096 x 12288: 10.2 / 11.8 -> 10.1 / 10.4 at 2 bits, 23.2 / 23.5 -> 11.6 / 11.8 at 3; 16384 x 16384 at 2 bits 62 / 107
     -> 38 / 38); at K = 8192 the unsplit kernel is 1 - 2 us ahead."""
-    if nbits not in KSPLIT_BITS or not (MGEMV_MIN_M <= M <= 2 * KSPLIT_MAX_M) or K < KSPLIT_MIN_K:
+    if nbits not in KSPLIT_BITS or not (MGEMV_MIN_M <= M <= 2 * KSPLIT_MAX_M) or K < KSPLIT_NARROW_MIN_K:
+        return None
+    if K < KSPLIT_MIN_K and (nbits != 4 or M > KSPLIT_MAX_M or not N or not (KSPLIT_NARROW_N[0] <= N <= KSPLIT_NARROW_N[1])):
+        # rows of 5120 .. 7167: two blocks along K pay on layers of about one tile per block only, now that the blocks'
+        # sums meet in one trip to memory (us at M = 4 / 16, unsplit -> split: 5120 x 5120 8.2 / 8.5 -> 7.1 / 7.4, 7168 x 5120
+        # 8.6 / 8.7 -> 7.9 / 8.3, 4096 x 6144 6.0 / 6.6 -> 5.8 / 6.3; 8192 x 5120 and 8192 x 6144 within 3 % either way, 15360 x 5120
+        # level, 3584 x 5120 5.7 / 6.0 -> 6.2 / 7.0; K = 4096: 4096 x 4096 level, 12288 and 22016 wide 8 - 13 % and 3 - 13 % slower)
         return None
     if not mgemv_supported(K, nbits, group_size):
         return None

@@ -19,11 +19,9 @@
 //     B (columns n), so a lane holds one n and needs one scale: acc += s * group_sum in fp32.
 //   * Each wave parks its partial 16x16 tiles in its own LDS slots; one barrier at the end of the
 //     block, then the partials of the WK waves are summed and every output is written once.
-//   * Long rows (KS > 1): K is also split over KS blocks, each holding the activations of its own K/KS only.  A block
-//     writes the fp32 sums of its tiles to a scratch buffer in device memory as it goes and counts itself in once, behind
-//     its last batch; the block that arrives last adds the KS partial results of every tile in the fixed order
-//     0 .. KS-1 (the result does not depend on who arrives when), stores the outputs and clears the counter for the
-//     next launch.
+//   * Long rows (KS > 1): K is also split over KS blocks (a power of two), each holding the activations of its own
+//     K/KS only.  Their fp32 sums meet pairwise in a scratch buffer in device memory, one atomic exchange per element
+//     and level of a binary tree over the blocks; the result does not depend on who arrives when (see the kernel).
 #pragma once
 
 #include <atomic>
@@ -57,12 +55,6 @@
 // 0: its arithmetic is skipped, which puts every tile's arithmetic into a conditional block (see there).
 #ifndef QF_MGEMV_COMPUTE_CLAMPED
 #define QF_MGEMV_COMPUTE_CLAMPED 1
-#endif
-// K split over blocks: device-scope loads the block that adds up the partial sums keeps in flight per thread (KS per
-// output, so 64 / KS outputs at a time; measured 1 / 16 / 32 / 64: 4096 x 11008 at 16 rows 9.77 / 9.45 / 9.50 / 9.57 us,
-// 57344 x 8192 48.5 / 48.2 / 47.5 / 47.8, 8192 x 28672 with eight blocks along K 28.6 / 28.9 / 29.0 / 28.3).
-#ifndef QF_MGEMV_MEET_LOADS
-#define QF_MGEMV_MEET_LOADS 64
 #endif
 // Non-zero: the order in which the first PF weight tiles and the activations are requested is fixed by scheduling
 // barriers (1, 2, 3: the orders listed where the loads are issued; measured on sixteen shapes at 4 and 16 rows, 3 is the
@@ -103,12 +95,11 @@ __device__ __forceinline__ void mg_static_for(F&& f) {
     }
 }
 
-// Scratch memory of a launch that splits K over blocks: KS partial results per batch of tiles and one arrival counter
-// per batch.  The counters must be zero when a launch starts; every launch leaves them zero.  Launches that share
-// one buffer must not overlap in time.
+// Scratch memory of a launch that splits K over blocks: per unit and batch of tiles, KS - 1 slots per output element
+// in which pairs of blocks exchange their sums, and one nobody reads.  The slots must be zero when a launch starts;
+// every launch leaves them zero.  Launches that share one buffer must not overlap in time.
 struct MGemvScratch {
     float* partial = nullptr;
-    unsigned* arrived = nullptr;
 };
 
 template <int NBITS_, int GS_, bool SYM_, int N_, int K_, int MT16_, int WK_, int CH_, int PB_, int PF_, bool NT_B_, int KS_ = 1>
@@ -164,8 +155,7 @@ struct MGemvCfg {
     // split K: fp32 sums of one block and batch, and what one row block (grid.y) of a launch needs
     static constexpr int PART = SB * MT16 * 256;
     static constexpr size_t SCRATCH_FLOATS = KS > 1 ? (size_t)GRID_X * NBATCH * KS * PART : 0;
-    static constexpr size_t SCRATCH_COUNTERS = KS > 1 ? (size_t)GRID_X : 0;
-    static constexpr size_t SCRATCH_BYTES = (SCRATCH_FLOATS * 4 + 255) / 256 * 256 + SCRATCH_COUNTERS * 4;   // partial sums, then the counters
+    static constexpr size_t SCRATCH_BYTES = (SCRATCH_FLOATS * 4 + 255) / 256 * 256;
 };
 
 template <class C>
@@ -432,6 +422,79 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
     // run-time branch reaches its users through a copy at the join, and that copy waits for every
     // load in flight -- measured as a full drain (vmcnt(0)) at the end of every tile, i.e. weight
     // loads and compute did not overlap at all.
+    // ---- K split over blocks: how the KS blocks of a unit add up their sums.
+    // The blocks form a binary tree over blockIdx.z.  For every output element a pair of blocks shares one 32-bit slot
+    // of the scratch buffer, empty (zero) between launches: each swaps its sum in with a device-scope atomic exchange.
+    // Whoever gets "empty" back was first and is done with the element; the other gets the partner's sum back, adds
+    // its own (one fp32 addition, the same in either order), empties the slot for the next launch and carries the
+    // result up one level, where the pair of pairs shares the next slot -- until the block that is second at the top
+    // stores the output.  So the sum of an element is (..(p0 + p1) + (p2 + p3)..): fixed by the tree, independent of
+    // who arrives when, and the meeting is log2(KS) dependent trips to memory with no barrier, no counter and no
+    // wait for acknowledged stores (the counted-arrival form it replaces took three trips and two block barriers
+    // at KS = 2).  A sum is never -0 (accumulators start at +0), so +0 travels as the bit pattern of -0 and zero can
+    // mean "empty".  Lanes that have nothing to swap at a level (they were first below, or lie past the batch's last
+    // element) sit the swap out: a swap into a spare word instead -- tried, to keep the swaps out of branches -- makes
+    // idle lanes of several blocks queue on the same addresses (2 - 28 times the kernel's time).
+    constexpr int THREADS = 64 * WK;
+    constexpr int EPB = KS > 1 ? (C::PART + THREADS - 1) / THREADS : 1;         // sums per thread and batch
+    constexpr int NQ = KS > 1 && C::NBATCH <= 8 ? C::NBATCH : 1;                // batches whose meeting waits for the last batch
+    constexpr int LV = KS <= 1 ? 0 : KS == 2 ? 1 : KS == 4 ? 2 : KS == 8 ? 3 : 4;
+    float pair_mine[NQ][EPB];
+    uint32_t pair_got[NQ][EPB];
+    const size_t split_unit = (size_t)blockIdx.y * C::GRID_X + team_id;
+    // node of the tree this block's sum enters at `level` (KS - 1 nodes; index KS - 1 is the slot nobody reads)
+    auto node_of = [&](int level) { return KS - (KS >> level) + ((int)blockIdx.z >> (level + 1)); };
+    auto node_slot = [&](int batch, int node, int o) {
+        return reinterpret_cast<uint32_t*>(scratch.partial) + ((split_unit * C::NBATCH + batch) * KS + node) * C::PART + o;
+    };
+    auto swap_in = [&](uint32_t* slot, float v) {
+        uint32_t bits = __builtin_bit_cast(uint32_t, v);
+        bits = bits == 0u ? 0x80000000u : bits;
+        return __hip_atomic_exchange(slot, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    // the meeting of the batches first_batch .. first_batch + NQ - 1, whose level-0 swaps are on their way
+    auto meet = [&](int first_batch) {
+        if (QF_MGEMV_EXPERIMENT & 4) return;
+        bool alive[NQ][EPB];
+#pragma unroll
+        for (int qq = 0; qq < NQ; qq++)
+#pragma unroll
+            for (int e = 0; e < EPB; e++) alive[qq][e] = tid + e * THREADS < C::PART;
+        mg_static_for<0, LV>([&](auto lv_tag) {
+            constexpr int L = decltype(lv_tag)::value;
+#pragma unroll
+            for (int qq = 0; qq < NQ; qq++)
+#pragma unroll
+                for (int e = 0; e < EPB; e++) {
+                    const int o = min(tid + e * THREADS, C::PART - 1);
+                    const uint32_t got = pair_got[qq][e];
+                    const bool second = alive[qq][e] && got != 0u;
+                    const float other = __builtin_bit_cast(float, got == 0x80000000u ? 0u : got);
+                    pair_mine[qq][e] = second ? other + pair_mine[qq][e] : pair_mine[qq][e];
+                    alive[qq][e] = second;
+                    pair_got[qq][e] = 0u;
+                    if (second) {
+                        // the slot is empty again for the next launch; the sum goes up one level
+                        __hip_atomic_store(node_slot(first_batch + qq, node_of(L), o), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if constexpr (L + 1 < LV) pair_got[qq][e] = swap_in(node_slot(first_batch + qq, node_of(L + 1), o), pair_mine[qq][e]);
+                    }
+                }
+        });
+#pragma unroll
+        for (int qq = 0; qq < NQ; qq++)
+#pragma unroll
+            for (int e = 0; e < EPB; e++) {
+                const int o = tid + e * THREADS;
+                const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
+                const int sb = p / MT16, mt = p % MT16;
+                const int slot = (first_batch + qq) * SB + sb;
+                const int tile = unit_of(slot);
+                const int m = m0 + 16 * mt + ml;
+                const int n = tile * 16 + nl;
+                if (alive[qq][e] && slot < SLOTS && tile < C::NT && m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, pair_mine[qq][e]);
+            }
+    };
+
     auto do_batch = [&](auto batch_v) {
         using BT = decltype(batch_v);
         constexpr bool STATIC_BATCH = mg_is_tag<BT>::value;
@@ -607,19 +670,24 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
             }
         }
         if constexpr (KS > 1) {
-            // ---- K split over blocks: the block's own sums of this batch go to the scratch buffer (device-scope
-            //      stores, nobody waits for them here); the blocks meet once, behind the last batch ----
+            // ---- K split over blocks: every sum of this batch is swapped into the slot it shares with the partner
+            //      block's sum (see the meeting below); the swaps' results are looked at behind the last batch ----
             static_assert(!C::SILU && !NORM, "a block that sees part of K cannot normalise the rows or pair the gate with the up tile");
-            const size_t unit = (size_t)blockIdx.y * C::GRID_X + team_id;
-            float* const mine = scratch.partial + ((unit * KS + blockIdx.z) * C::NBATCH + batch) * C::PART;
-            for (int o = tid; o < C::PART && !(QF_MGEMV_EXPERIMENT & 4); o += 64 * WK) {
-                float total = 0.f;
+            int q = 0;
+            if constexpr (STATIC_BATCH && NQ > 1) q = BT::value;
+#pragma unroll
+            for (int e = 0; e < EPB; e++) {
+                const int o = min(tid + e * THREADS, C::PART - 1);
                 const int p = o >> 8, ml = (o >> 4) & 15, nl = o & 15;
                 const float* base = redf + ((size_t)p * 64 + nl + 16 * (ml >> 2)) * 4 + (ml & 3);
+                float total = 0.f;
 #pragma unroll
                 for (int k2 = 0; k2 < WK; k2++) total += base[(size_t)k2 * SB * MT16 * 256];
-                __hip_atomic_store(mine + o, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                pair_mine[q][e] = total;
+                pair_got[q][e] = 0u;
+                if (!(QF_MGEMV_EXPERIMENT & 4) && tid + e * THREADS < C::PART) pair_got[q][e] = swap_in(node_slot(batch, node_of(0), o), total);
             }
+            if constexpr (NQ == 1) meet(batch);                // many batches: each one's meeting right away
         }
         constexpr int OUTPUTS = (C::SILU || KS > 1) ? 0 : SB * MT16 * 256;
         for (int o = tid; o < OUTPUTS && !(QF_MGEMV_EXPERIMENT & 4); o += 64 * WK) {
@@ -645,72 +713,17 @@ __global__ __launch_bounds__(C::THREADS) void mgemv_kernel(
         for (int batch = 0; batch < C::NBATCH; batch++) do_batch(batch);
     }
 
-    if constexpr (KS > 1) {
-        // ---- the KS blocks of a unit meet: each counts itself in once all its sums are out; the block that finds
-        //      the other KS - 1 already counted adds the KS partial results of every tile in the order of their K
-        //      ranges (the result does not depend on who arrives when) and stores the outputs.
-        // The sums are device-scope stores (written through to where every XCD sees them), read back by device-scope
-        // loads, and the counter is a device-scope atomic: no cache is written back or invalidated as a whole (a
-        // device-wide fence per thread measured 5 - 20 times the kernel's own time).  A thread's stores have been
-        // acknowledged when its memory counter reads zero; the barrier collects that from every thread before the
-        // block is counted. ----
-        if (QF_MGEMV_EXPERIMENT & 4) return;                  // timing: no block is counted in, the counters stay zero
-        const size_t unit = (size_t)blockIdx.y * C::GRID_X + team_id;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();                                       // ... and every read of the LDS slots is done
-        unsigned* const flag = reinterpret_cast<unsigned*>(smem);
-        if (tid == 0) *flag = __hip_atomic_fetch_add(scratch.arrived + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if (*flag != (unsigned)(KS - 1)) return;               // block-uniform
-        const float* const all = scratch.partial + unit * KS * C::NBATCH * C::PART;
-        // Every device-scope load is a trip to memory, and a loop of "load KS values, add, store" pays one trip per
-        // pass: the loads of up to UN passes go out together (clamped indices, no branch around a load), then the sums.
-        constexpr int TOTAL = C::NBATCH * C::PART, THREADS = 64 * WK;
-        constexpr int PASSES = (TOTAL + THREADS - 1) / THREADS;
-        constexpr int UN_MAX = QF_MGEMV_MEET_LOADS / KS > 1 ? QF_MGEMV_MEET_LOADS / KS : 1;
-        constexpr int UN = PASSES < UN_MAX ? PASSES : UN_MAX;
-        for (int first = 0; first < PASSES; first += UN) {
-            float part[UN][KS];
-#pragma unroll
-            for (int u = 0; u < UN; u++) {
-                const int o = min(tid + (first + u) * THREADS, TOTAL - 1);
-#pragma unroll
-                for (int z = 0; z < KS; z++)
-                    part[u][z] = __hip_atomic_load(all + (size_t)z * TOTAL + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-#pragma unroll
-            for (int u = 0; u < UN; u++) {
-                const int o = tid + (first + u) * THREADS;
-                const int batch = o / C::PART, ob = o % C::PART;
-                const int p = ob >> 8, ml = (ob >> 4) & 15, nl = ob & 15;
-                const int sb = p / MT16, mt = p % MT16;
-                const int slot = batch * SB + sb;
-                const int tile = unit_of(slot);
-                float total = 0.f;
-#pragma unroll
-                for (int z = 0; z < KS; z++) total += part[u][z];
-                const int m = m0 + 16 * mt + ml;
-                const int n = tile * 16 + nl;
-                if (o < TOTAL && slot < SLOTS && tile < C::NT && m < m_total && n < C::N) store_out(Cout + (size_t)m * C::N + n, total);
-            }
-        }
-        // nobody else touches this counter again in this launch: zero for the next one
-        if (tid == 0) __hip_atomic_store(scratch.arrived + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if constexpr (KS > 1 && NQ > 1) meet(0);
 }
 
 // Row blocks (grid.y) a split-K object's scratch buffer is sized for.
 constexpr int kMGemvScratchRowBlocks = 1;
 
-// A buffer of kMGemvScratchRowBlocks * SCRATCH_BYTES bytes, 256-byte aligned, as the kernel's two arrays: the
-// partial sums of every row block first, the counters behind them.
+// A buffer of kMGemvScratchRowBlocks * SCRATCH_BYTES bytes, 256-byte aligned and zero, as the kernel's slots.
 template <class C>
 MGemvScratch mgemv_scratch_at(void* base) {
     MGemvScratch s;
     s.partial = static_cast<float*>(base);
-    s.arrived = reinterpret_cast<unsigned*>(static_cast<uint8_t*>(base)
-                                            + (C::SCRATCH_FLOATS * 4 * kMGemvScratchRowBlocks + 255) / 256 * 256);
     return s;
 }
 
@@ -776,7 +789,7 @@ int mgemv_launch(const void* A, const void* W, void* Cout, const void* S, const 
     else if (QF_OUT_ACCUMULATE && (QF_OUT_BF16 || QF_MGEMV_GATE_UP_SILU)) why = "adding to the output is fp16 only and not combined with the SwiGLU epilogue";
     else if (QF_MGEMV_NORM_PROLOGUE && norm.gamma == nullptr) why = "an object with the norm prologue is called through launch_norm (RMSNorm weight missing)";
     else if (!QF_MGEMV_NORM_PROLOGUE && norm.gamma != nullptr) why = "this object was compiled without the norm prologue";
-    else if (C::KS < 1 || C::KS > 16) why = "KS must be 1 .. 16";
+    else if (C::KS != 1 && C::KS != 2 && C::KS != 4 && C::KS != 8 && C::KS != 16) why = "KS must be 1, 2, 4, 8 or 16";
     else if (C::KS > 1 && (QF_MGEMV_NORM_PROLOGUE || QF_MGEMV_GATE_UP_SILU)) why = "K split over blocks: neither the norm prologue nor the SwiGLU epilogue";
     else if (C::KS > 1 && C::WK * C::CH < C::NCHUNK_B) why = "WK*CH must cover a block's share of K";
     else if (C::KS > 1 && (C::KS - 1) * C::NCHUNK_B >= C::NCHUNK) why = "a block would own no chunk";

@@ -3,7 +3,8 @@ meet through scratch memory in device memory) and of the kernels that serve the 
 
 The split is the default of these shapes, so tests/test_qlinear_gpu.py, test_bf16_gpu.py, test_norm_prologue_gpu.py
 and the decode tests already run it on their long rows; here: its other block counts and shapes, what is special
-about it (state kept between launches: the arrival counters and the partial sums), and the unsplit kernels, which
+about it (state kept between launches: the slots in which pairs of blocks exchange their sums, empty between
+launches; a result that must not depend on which block of a pair arrives first), and the unsplit kernels, which
 remain what a layer with the norm prologue or the SwiGLU epilogue is built on."""
 import numpy as np
 import pytest
@@ -80,7 +81,7 @@ def test_long_rows_without_the_split(oracle, case):
 
 
 def test_launches_of_different_row_counts_share_the_scratch_memory(oracle):
-    """16 rows, then 3, then 16 again on one object: the counters are zero again after every launch and no launch
+    """16 rows, then 3, then 16 again on one object: the slots are empty again after every launch and no launch
     reads a partial sum an earlier one left; the same input gives the same bits every time."""
     case = prebuild._case(16, 4096, 11008)
     print("[case] split, row counts 16 / 3 / 16 on one object", flush=True)
@@ -112,7 +113,7 @@ def test_split_rows_in_a_hip_graph_replay_like_the_eager_launch():
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
         layer(x, out=out)
-        layer(x, out=out)                                                   # twice in one graph: the second finds the counters zero
+        layer(x, out=out)                                                   # twice in one graph: the second finds the slots empty
     torch.cuda.current_stream().wait_stream(side)
     for i in range(3):
         out.fill_(float("nan"))
@@ -120,6 +121,27 @@ def test_split_rows_in_a_hip_graph_replay_like_the_eager_launch():
         torch.cuda.synchronize()
         assert torch.equal(out, want), f"replay {i}"
         assert torch.equal(layer(A), want)                                  # eager work between the replays
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 8192, 8192), (16, 4096, 11008), (7, 1000, 28672), (8, 100, 53248), (4, 7168, 5120)])
+def test_the_result_does_not_depend_on_who_arrives_first(M, N, K):
+    """Two, four, eight and sixteen blocks along K: the blocks of a pair meet in whatever order the hardware runs them,
+    the sum of an output is fixed by the tree over the blocks.  Forty launches, with other work in between so that the
+    blocks start at different moments: the same bits every time (compared as integers: +0 and -0 differ)."""
+    case = {"M": M, "N": N, "K": K, "NBITS": 4, "GS": 128, "sym": N == 100}
+    print(f"[case] arrival order {_id(case)}", flush=True)
+    layer, g = _filled_layer(case, 17)
+    assert "KS=" in layer.func.runtime.description
+    A = torch.randn(M, K, device="cuda", generator=g).to(torch.float16)
+    A[0].zero_()                                                            # a row of exact zeros: sums of +0 travel as "not empty"
+    first = layer(A).view(torch.int16).clone()
+    noise = torch.empty(1 << 22, device="cuda")
+    for i in range(40):
+        if i % 3:
+            noise.normal_()                                                 # occupies part of the GPU while the launch starts
+        out = layer(A)
+        assert torch.equal(out.view(torch.int16), first), i
+    assert float(layer(A)[0].abs().max()) == 0.0
 
 
 def test_add_to_output_with_split_rows(oracle):

@@ -39,8 +39,9 @@ def test_regime_routing(M, K, nbits, gs, expected):
     (3, 7168, 4, 128, 2), (16, 8192, 4, 128, 2), (4, 11008, 4, 128, 4), (16, 14336, 4, 128, 4), (16, 16384, 4, 128, 4),
     (16, 28672, 4, 128, 8), (8, 53248, 4, 128, 16), (16, 8192, 8, 128, 2), (16, 11008, 8, 128, 4),
     (16, 12288, 2, 128, 4), (16, 12288, 3, 128, 4), (16, 8192, 4, 64, 2), (16, 8192, 4, 32, 2),
+    (16, 5120, 4, 128, 2), (4, 6144, 4, 128, 2),          # rows of 5120 .. 7167 on a layer of 4096 .. 7168 columns
     # not split: short rows, one or two activation rows, more than sixteen, 2 and 3 bits where the unsplit kernel holds K
-    (16, 4096, 4, 128, 1), (16, 5120, 4, 128, 1), (2, 8192, 4, 128, 1), (17, 8192, 4, 128, 1), (33, 11008, 4, 128, 1),
+    (16, 4096, 4, 128, 1), (16, 5120, 8, 128, 1), (2, 8192, 4, 128, 1), (17, 8192, 4, 128, 1), (33, 11008, 4, 128, 1),
     (16, 8192, 2, 128, 1), (16, 8192, 3, 128, 1),
     # 17 .. 32 rows: two activation tiles per wave, narrow layers with long rows only
     (32, 11008, 4, 128, 4), (17, 14336, 4, 128, 8), (32, 11008, 8, 128, 1),
@@ -60,6 +61,13 @@ def test_long_rows_are_split_over_blocks(M, K, nbits, gs, ks):
     assert tiling.mgemv_lds_bytes(t["MT16"], t["WK"], t["CH"], nbits) <= 160 * 1024
     assert tiling.mgemv_regs(t["MT16"], t["CH"], t["PF"], nbits) <= tiling.mgemv_reg_limit(t["WK"])
     assert f", {ks}>" in tiling.mgemv_cfg_string({"NBITS": nbits, "GS": gs, "SYM": False, "N": 4096, "K": K}, t, True)
+
+
+def test_rows_of_5120_are_split_on_narrow_layers_only():
+    for N, split in ((3584, False), (4096, True), (5120, True), (7168, True), (8192, False), (15360, False), (0, False)):
+        assert (tiling.mgemv_ksplit_tiling(16, N, 5120, 4, 128) is not None) == split, N
+    assert tiling.mgemv_ksplit_tiling(16, 5120, 4096, 4, 128) is None
+    assert tiling.mgemv_ksplit_tiling(32, 5120, 5120, 4, 128) is None
 
 
 def test_wide_layers_keep_the_gemm_kernel_at_32_rows():
