@@ -305,6 +305,8 @@ def split_cases():
     return [_case(16, 4096, 7168), _case(3, 48, 7168, 4, 64), _case(16, 16384, 16384), _case(7, 1000, 28672), _case(4, 8192, 29696),
             _case(16, 100, 53248, 4, 128, True), _case(13, 57344, 8192), _case(16, 2048, 16384, 8, 128), _case(5, 77, 12288, 2, 128),
             _case(16, 272, 12288, 3, 128, True), _case(16, 5120, 13824),
+            # five tiles per block in one batch (the last of them ragged)
+            _case(11, 8200, 8192), _case(16, 10240, 8192),
             # rows of 5120 .. 7167 on narrow layers: two blocks along K
             _case(16, 5120, 5120), _case(4, 7168, 5120), _case(9, 4096, 6144, 4, 64),
             # 17 .. 32 rows on narrow layers with long rows: two activation tiles per wave

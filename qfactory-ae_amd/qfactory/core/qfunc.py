@@ -258,6 +258,13 @@ class QMatmulQFunc(QFunc):
             slots = -(-(-(-p["N"] // 16)) // min(-(-p["N"] // 16), t["PB"]))
             if slots >= 6 and tiling.mgemv_lds_bytes(1, t["WK"], t["CH"], p["NBITS"], sb=8) <= 160 * 1024:
                 defines.setdefault("QF_MGEMV_SB", 8)
+        if self.regime == "mgemv" and t["MT16"] == 1 and t.get("KS", 1) > 1 and "QF_MGEMV_SB" not in defines:
+            # K split over blocks and five tiles per block: one batch of five instead of four and one, so that the
+            # blocks' sums go into their swaps in one go (M = 4 / 16, cold weights: 10240 x 8192 12.1 / 13.1 -> 11.3 / 12.5 us,
+            # 5120 x 14336 12.9 / 13.6 -> 11.1 / 12.1).  Without the split, or with nine tiles (five and four), level.
+            slots = -(-(-(-p["N"] // 16)) // min(-(-p["N"] // 16), t["PB"]))
+            if slots == 5 and tiling.mgemv_lds_bytes(1, t["WK"], t["CH"], p["NBITS"], sb=5) <= 160 * 1024:
+                defines.setdefault("QF_MGEMV_SB", 5)
         if self.regime == "gemm":
             # Block -> tile map that puts the row slabs of one column of tiles on one XCD (its L2 then serves the weights to
             # all of them) instead of the columns of one slab: pays where a launch has a few slabs -- measured, FETCH_SIZE
